@@ -1,0 +1,156 @@
+"""Shared by the tests: the tiny configurations, trace building and comparison."""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from wllm_amd.config import GemmaConfig
+from wllm_amd.parts import write_random_model_folder
+
+# Two tiny configurations that differ in every size and option, a third with
+# biases and an untied head, and a fourth whose head size and page size are the
+# ones the matrix-core attention kernels take.
+TINY = {
+    "A": dict(config=GemmaConfig(vocab_size=512, hidden_size=64, intermediate_size=256, num_hidden_layers=2,
+                                 num_attention_heads=4, num_key_value_heads=1, head_dim=32, rms_norm_eps=1e-6,
+                                 rope_theta=10000.0, max_position_embeddings=128, tie_word_embeddings=True),
+              seed=11, std=0.02, norm_std=0.1, page_size=4),
+    "B": dict(config=GemmaConfig(vocab_size=777, hidden_size=96, intermediate_size=384, num_hidden_layers=3,
+                                 num_attention_heads=6, num_key_value_heads=6, head_dim=24, rms_norm_eps=1e-5,
+                                 rope_theta=500.0, max_position_embeddings=256, tie_word_embeddings=True),
+              seed=22, std=0.03, norm_std=0.05, page_size=8),
+    "C": dict(config=GemmaConfig(vocab_size=301, hidden_size=80, intermediate_size=112, num_hidden_layers=2,
+                                 num_attention_heads=6, num_key_value_heads=2, head_dim=20, rms_norm_eps=1e-4,
+                                 rope_theta=77.0, max_position_embeddings=192, tie_word_embeddings=False,
+                                 attention_bias=True),
+              seed=33, std=0.05, norm_std=0.2, page_size=16),
+    "M": dict(config=GemmaConfig(vocab_size=1000, hidden_size=128, intermediate_size=320, num_hidden_layers=2,
+                                 num_attention_heads=8, num_key_value_heads=2, head_dim=64, rms_norm_eps=1e-6,
+                                 rope_theta=10000.0, max_position_embeddings=512, tie_word_embeddings=True),
+              seed=44, std=0.04, norm_std=0.1, page_size=16),
+}
+
+
+def write_tiny(name: str, folder: str) -> str:
+    t = TINY[name]
+    return write_random_model_folder(folder, t["config"], t["seed"], std=t["std"], norm_std=t["norm_std"])
+
+
+def random_ids(seed: int, length: int, vocab: int) -> list:
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (length,), generator=g).tolist()
+
+
+# ---- traces ------------------------------------------------------------------
+
+def trace_whole(requests: dict) -> list:
+    """Each request alone, all its tokens in one step, every logit wanted."""
+    return [{"step": i, "entries": [{"id": rid, "tokens": toks, "want": list(range(len(toks)))}], "end": [rid]}
+            for i, (rid, toks) in enumerate(requests.items())]
+
+
+def trace_tail(requests: dict, tail: int = 32) -> list:
+    """All but the last `tail` tokens in one step, then the rest one by one."""
+    steps = []
+    for rid, toks in requests.items():
+        head = max(1, len(toks) - tail)
+        steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": toks[:head], "want": list(range(head))}], "end": []})
+        for p in range(head, len(toks)):
+            steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": [toks[p]], "want": [0]}],
+                          "end": [rid] if p == len(toks) - 1 else []})
+        if head == len(toks):
+            steps[-1]["end"] = [rid]
+    return steps
+
+
+def trace_portions(requests: dict, sizes=(16, 5, 2, 11, 2, 7, 3, 2, 9)) -> list:
+    """Consecutive portions of changing size, down to two tokens."""
+    steps = []
+    for rid, toks in requests.items():
+        p, k = 0, 0
+        while p < len(toks):
+            size = min(sizes[k % len(sizes)], len(toks) - p)
+            k += 1
+            last = p + size == len(toks)
+            steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": toks[p:p + size], "want": list(range(size))}],
+                          "end": [rid] if last else []})
+            p += size
+    return steps
+
+
+def trace_mixed(requests: dict, seed: int = 0, live: int = 4, prompt_fraction: float = 0.6,
+                portion_sizes=(2, 3, 5, 8, 13)) -> list:
+    """Up to `live` requests at a time: portions of some beside single tokens of
+    others; a request is sometimes left out of a step; finished requests are ended
+    and new ones start, so their pages are handed out again."""
+    rng = np.random.default_rng(seed)
+    waiting = list(requests.items())
+    running = {}      # rid -> (tokens, fed, prompt_len)
+    steps = []
+    while waiting or running:
+        while waiting and len(running) < live:
+            rid, toks = waiting.pop(0)
+            running[rid] = [toks, 0, max(2, int(len(toks) * prompt_fraction))]
+        entries, ended = [], []
+        for rid in list(running):
+            toks, fed, plen = running[rid]
+            if len(running) > 1 and rng.random() < 0.2:
+                continue  # left out of this step
+            if fed < plen:
+                size = int(min(rng.choice(portion_sizes), plen - fed))
+                if plen - fed - size == 1:
+                    size += 1   # never leave a portion of one token: that is a decode
+            else:
+                size = 1
+            entries.append({"id": rid, "tokens": toks[fed:fed + size], "want": list(range(size))})
+            running[rid][1] = fed + size
+            if fed + size == len(toks):
+                ended.append(rid)
+                del running[rid]
+        if entries:
+            steps.append({"step": len(steps), "entries": entries, "end": ended})
+    return steps
+
+
+def max_live_tokens(trace: list, round_to: int = 64) -> int:
+    """The most tokens live requests hold at any time, each rounded up to `round_to`."""
+    held, worst = {}, 0
+    for step in trace:
+        for e in step["entries"]:
+            held[e["id"]] = held.get(e["id"], 0) + len(e["tokens"])
+        worst = max(worst, sum(-(-v // round_to) * round_to for v in held.values()))
+        for rid in step["end"]:
+            held.pop(rid, None)
+    return worst
+
+
+def replay_and_collect(replayer, trace: list) -> dict:
+    """Runs a trace; returns {(request, position): logits row (float32 CPU)}."""
+    fed, out = {}, {}
+    for step in trace:
+        logits = replayer.run_step(step)
+        row = 0
+        for e in step["entries"]:
+            base = fed.get(e["id"], 0)
+            for w in e["want"]:
+                out[(e["id"], base + w)] = logits[row].float().cpu()
+                row += 1
+            fed[e["id"]] = base + len(e["tokens"])
+        for rid in step["end"]:
+            fed.pop(rid, None)
+    return out
+
+
+def compare_with_plain(collected: dict, plain: dict, atol: float, rtol: float) -> float:
+    """Every collected row against the plain implementation's row of the same request
+    and position; returns the worst error in units of the tolerance.  The first wrong
+    place is named."""
+    worst = 0.0
+    for (rid, pos) in sorted(collected, key=lambda k: (str(k[0]), k[1])):
+        got, ref = collected[(rid, pos)].double(), plain[rid][pos].double()
+        assert torch.isfinite(got).all(), f"request {rid!r} position {pos}: logits are not finite"
+        err = ((got - ref).abs() / (atol + rtol * ref.abs())).max().item()
+        assert err <= 1.0, (f"request {rid!r} position {pos}: worst error {err:.2f} x tolerance "
+                            f"(max abs diff {(got - ref).abs().max().item():.3e}, ref max {ref.abs().max().item():.3e})")
+        worst = max(worst, err)
+    return worst

@@ -1,0 +1,127 @@
+"""A plain emulation of every kernel's contract, in ordinary torch arithmetic.
+
+It has two uses.  On a machine without a GPU it stands in for the kernel library
+so that the engine's bookkeeping (cache, batching, scheduling) can be compared
+with the plain implementation.  On the GPU it is each kernel's reference: the
+`-m gpu` tests run a kernel and its emulation on the same operands.  It follows
+the contracts written in `wllm_amd/kernels/ops.py`, not the kernels' code, and
+computes in float64 when `precise` is set.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+
+class EmulatedKernels:
+    def __init__(self, precise: bool = False):
+        self.acc = torch.float64 if precise else torch.float32
+        self.calls = {}
+
+    def _count(self, name):
+        self.calls[name] = self.calls.get(name, 0) + 1
+
+    def embed_lookup(self, ids, table, scale, out):
+        self._count("embed_lookup")
+        out.copy_((table[ids.long()].to(self.acc) * scale).to(out.dtype))
+
+    def rms_norm(self, x, weight, eps, offset, out, delta, rows):
+        self._count("rms_norm")
+        if rows is None:
+            v = x.to(self.acc)
+            if delta is not None:
+                v = v + delta.to(self.acc)
+                x.copy_(v.to(x.dtype))
+                v = x.to(self.acc)  # the kernel normalises what it wrote back
+        else:
+            idx = rows.long()
+            v = x[idx].to(self.acc)
+            if delta is not None:
+                v = (v + delta[idx].to(self.acc)).to(x.dtype).to(self.acc)
+        var = v.pow(2).mean(-1, keepdim=True)
+        y = v * torch.rsqrt(var + eps) * (offset + weight.to(self.acc))
+        out.copy_(y.to(out.dtype))
+
+    def rope_and_cache_write(self, qkv, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads,
+                             head_dim, rotary_dim, page_size):
+        self._count("rope_and_cache_write")
+        n = qkv.shape[0]
+        heads = num_heads + 2 * num_kv_heads
+        v = qkv.to(self.acc)
+        if bias is not None:
+            v = v + bias.to(self.acc)
+        v = v.view(n, heads, head_dim).clone()
+        if inv_freq is not None:
+            half = rotary_dim // 2
+            ang = positions.to(torch.float32)[:, None] * inv_freq[None, :]          # float32 angles
+            cos, sin = ang.cos().to(self.acc)[:, None, :], ang.sin().to(self.acc)[:, None, :]
+            r = num_heads + num_kv_heads                                              # queries and keys
+            x1 = v[:, :r, :half].clone()
+            x2 = v[:, :r, half:rotary_dim].clone()
+            v[:, :r, :half] = x1 * cos - x2 * sin
+            v[:, :r, half:rotary_dim] = x2 * cos + x1 * sin
+        qkv.copy_(v.view(n, -1).to(qkv.dtype))
+        if cache is not None:
+            rows = qkv.view(n, heads, head_dim)
+            page = (slots // page_size).long()
+            off = (slots % page_size).long()
+            k = rows[:, num_heads:num_heads + num_kv_heads]                           # [n, nkv, d]
+            val = rows[:, num_heads + num_kv_heads:]
+            kview = cache[:, 0].view(cache.shape[0], num_kv_heads, page_size, head_dim)
+            vview = cache[:, 1].view(cache.shape[0], num_kv_heads, head_dim, page_size)
+            kview[page, :, off, :] = k
+            vview[page, :, :, off] = val
+
+    def paged_attention(self, qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len, out,
+                        num_heads, num_kv_heads, head_dim, page_size, scale, window, max_q_len, max_ctx_len):
+        self._count("paged_attention")
+        n = qkv.shape[0]
+        n_rep = num_heads // num_kv_heads
+        q_all = qkv.view(n, num_heads + 2 * num_kv_heads, head_dim)[:, :num_heads].to(self.acc)
+        pages = cache.shape[0]
+        kview = cache[:, 0].view(pages, num_kv_heads, page_size, head_dim)
+        vview = cache[:, 1].view(pages, num_kv_heads, head_dim, page_size)
+        for s in range(block_tables.shape[0]):
+            q0, ql, cl = int(seg_q_start[s]), int(seg_q_len[s]), int(seg_ctx_len[s])
+            if ql == 0:
+                continue
+            npages = -(-cl // page_size)
+            ids = block_tables[s, :npages].long()
+            k = kview[ids].permute(0, 2, 1, 3).reshape(npages * page_size, num_kv_heads, head_dim)[:cl].to(self.acc)
+            v = vview[ids].permute(0, 3, 1, 2).reshape(npages * page_size, num_kv_heads, head_dim)[:cl].to(self.acc)
+            k = k.repeat_interleave(n_rep, dim=1)
+            v = v.repeat_interleave(n_rep, dim=1)
+            q = q_all[q0:q0 + ql]
+            pos = torch.arange(cl - ql, cl, device=q.device)
+            key = torch.arange(cl, device=q.device)
+            allowed = key[None, :] <= pos[:, None]
+            if window:
+                allowed &= key[None, :] > pos[:, None] - window
+            scores = torch.einsum("qhd,khd->hqk", q, k) * scale
+            # keys outside the window may hold NaN of pages given back: mask by selection, not by addition
+            scores = torch.where(allowed[None], scores, torch.full_like(scores, float("-inf")))
+            probs = torch.softmax(scores, dim=-1)
+            v = torch.where(torch.isnan(v), torch.zeros_like(v), v) if window else v
+            o = torch.einsum("hqk,khd->qhd", probs, v)
+            out[q0:q0 + ql] = o.reshape(ql, num_heads * head_dim).to(out.dtype)
+
+    def linear(self, x, weight, out):
+        self._count("linear")
+        out.copy_((x.to(self.acc) @ weight.to(self.acc).T).to(out.dtype))
+
+    def gated_activation(self, gate_up, out, activation):
+        self._count("gated_activation")
+        i = gate_up.shape[1] // 2
+        g, u = gate_up[:, :i].to(self.acc), gate_up[:, i:].to(self.acc)
+        if activation == "gelu_tanh":
+            a = 0.5 * g * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g.pow(3))))
+        elif activation == "silu":
+            a = g * torch.sigmoid(g)
+        else:
+            raise ValueError(activation)
+        out.copy_((a * u).to(out.dtype))
+
+    def argmax_rows(self, logits, out):
+        self._count("argmax_rows")
+        out.copy_(logits.argmax(dim=-1).to(torch.int32))

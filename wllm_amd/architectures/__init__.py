@@ -1,0 +1,3 @@
+"""Architectures: each module turns its typed configuration into a ModelPlan
+and registers itself under the names config.json may carry."""
+from wllm_amd.architectures import gemma  # noqa: F401  (registers GemmaForCausalLM)

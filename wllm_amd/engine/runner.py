@@ -1,0 +1,119 @@
+"""The step function: a batch of (request, its next tokens) in, logits at the wanted
+places out.
+
+`ModelRunner.step` runs only the tokens it is given, as one batch, from the cache
+that earlier steps left.  It asks the cache manager for room for every entry
+first (all or nothing: a step that does not fit raises `OutOfPages` before
+anything ran), builds the index tensors, runs the model and commits the new
+lengths.  It is the only way tokens reach the model: the scheduler, the replay
+tool and the benchmark all call it.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from wllm_amd.cache.manager import CacheManager
+from wllm_amd.cache.pages import OutOfPages
+from wllm_amd.engine.batch import StepContext, StepEntry, Workspace, pack_int32
+
+
+class StepError(ValueError):
+    """A step's entries are inconsistent with each other or with the cache."""
+
+
+class ModelRunner:
+    def __init__(self, model, cache: CacheManager):
+        self.model = model
+        self.cache = cache
+        self.device = model.device
+        self.workspace = Workspace(self.device)
+        self.steps_run = 0
+        self.tokens_run = 0
+
+    @classmethod
+    def create(cls, model, *, num_pages: int, page_size: int, max_requests: int, **cache_options):
+        cache = CacheManager(model.cache_needs(), page_size, num_pages, max_requests, model.dtype, model.device,
+                             state_shapes=model.state_shapes(), **cache_options)
+        return cls(model, cache)
+
+    def open(self, request) -> None:
+        self.cache.open(request)
+
+    def close(self, request) -> None:
+        self.cache.close(request)
+
+    def step(self, entries: list) -> torch.Tensor:
+        """Returns float32 logits [wanted, vocab] in the order of the entries and of
+        each entry's `want`.  The tensor is a view of a buffer the next step reuses."""
+        cache = self.cache
+        max_pos = self.model.plan.max_positions
+        seen = set()
+        for e in entries:
+            if e.request in seen:
+                raise StepError(f"request {e.request!r} appears twice in one step")
+            seen.add(e.request)
+            if not cache.is_open(e.request):
+                raise StepError(f"request {e.request!r} is not open")
+            if len(e.tokens) == 0:
+                raise StepError(f"request {e.request!r} brings no tokens")
+            if cache.context_len(e.request) + len(e.tokens) > max_pos:
+                raise StepError(f"request {e.request!r} would reach {cache.context_len(e.request) + len(e.tokens)} "
+                                f"tokens; the model allows {max_pos}")
+            for w in e.want:
+                if not 0 <= w < len(e.tokens):
+                    raise StepError(f"request {e.request!r}: wanted place {w} is not among its {len(e.tokens)} tokens")
+        vocab = self.model.plan.embedding.vocab_size
+        num_groups = len(cache.groups)
+        # room first: all entries or none
+        reserved = []
+        try:
+            for e in entries:
+                reserved.append(cache.reserve(e.request, len(e.tokens)))
+        except OutOfPages:
+            for e in entries[:len(reserved)]:
+                cache.trim(e.request)
+            raise
+        s = len(entries)
+        q_len = np.array([len(e.tokens) for e in entries], dtype=np.int32)
+        q_start = np.zeros(s, dtype=np.int32)
+        if s:
+            q_start[1:] = np.cumsum(q_len)[:-1]
+        n = int(q_len.sum())
+        old_len = np.array([cache.context_len(e.request) for e in entries], dtype=np.int32)
+        ctx_len = old_len + q_len
+        token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries]) if s else np.zeros(0, np.int64)
+        if n and (token_ids.min() < 0 or token_ids.max() >= vocab):
+            raise StepError(f"token id outside 0..{vocab - 1}")
+        token_ids = token_ids.astype(np.int32)
+        token_segment = np.repeat(np.arange(s, dtype=np.int32), q_len)
+        positions = (np.arange(n, dtype=np.int32) - q_start[token_segment] + old_len[token_segment]).astype(np.int32)
+        logit_rows = np.array([q_start[i] + w for i, e in enumerate(entries) for w in e.want], dtype=np.int32)
+        state_slots = np.array([cache.slot(e.request) for e in entries], dtype=np.int32)
+        group_slots, group_tables = [], []
+        for g in range(num_groups):
+            group_slots.append(np.concatenate([r[g] for r in reserved]) if s else np.zeros(0, np.int32))
+            tables = [cache.block_table(e.request, g) for e in entries]
+            width = max((len(t) for t in tables), default=1)
+            bt = np.zeros((s, max(width, 1)), dtype=np.int32)
+            for i, t in enumerate(tables):
+                # a page given back (-1) lies outside every window that is still read
+                bt[i, :len(t)] = np.maximum(np.asarray(t, dtype=np.int32), 0)
+            group_tables.append(bt)
+        arrays = [token_ids, positions, token_segment, q_start, q_len, ctx_len, state_slots, logit_rows]
+        arrays += group_slots + group_tables
+        dev = pack_int32(arrays, self.device)
+        ctx = StepContext(
+            n=n, num_segments=s, dtype=self.model.dtype, device=self.device, workspace=self.workspace,
+            cache=cache, schedule=self.model.plan.schedule,
+            token_ids=dev[0], positions=dev[1], token_segment=dev[2], seg_q_start=dev[3], seg_q_len=dev[4],
+            seg_ctx_len=dev[5], state_slots=dev[6], logit_rows=dev[7], num_logit_rows=int(logit_rows.size),
+            group_slots=dev[8:8 + num_groups], group_block_tables=dev[8 + num_groups:8 + 2 * num_groups],
+            host_q_start=q_start, host_q_len=q_len, host_ctx_len=ctx_len, host_state_slots=state_slots,
+            requests=[e.request for e in entries])
+        logits = self.model.forward(ctx)
+        for e in entries:
+            cache.commit(e.request, len(e.tokens))
+        self.steps_run += 1
+        self.tokens_run += n
+        return logits

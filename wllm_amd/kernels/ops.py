@@ -1,0 +1,237 @@
+"""The operations the parts are made of, each one a hand-written gfx950 kernel.
+
+Every function checks on the host that operand shapes, dtypes and devices are
+what its kernel and grid assume, then calls the kernel library.  There is no
+other implementation behind them: without the built library they raise
+`KernelLibraryMissing`.  Activations are float32 or bfloat16 ("T" below); the
+residual stream, norm weights, rotation frequencies and logits are float32
+always.
+
+`use_backend` swaps the object the calls go to.  The engine never does; it is
+the seam through which tests check the engine's bookkeeping against a plain
+emulation of each kernel's contract.
+"""
+from __future__ import annotations
+
+import contextlib
+from typing import Optional
+
+import torch
+
+_ACT = (torch.float32, torch.bfloat16)
+_backend = None
+
+
+class KernelShapeError(ValueError):
+    """An operand does not have the shape, dtype or layout the kernel needs."""
+
+
+def backend():
+    global _backend
+    if _backend is None:
+        from wllm_amd.kernels.hip_backend import HipBackend
+        _backend = HipBackend()
+    return _backend
+
+
+@contextlib.contextmanager
+def use_backend(obj):
+    global _backend
+    old, _backend = _backend, obj
+    try:
+        yield obj
+    finally:
+        _backend = old
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelShapeError(msg)
+
+
+def _dense(t: torch.Tensor, name: str, dtype, shape=None) -> None:
+    _need(isinstance(t, torch.Tensor), f"{name}: expected a tensor")
+    if isinstance(dtype, tuple):
+        _need(t.dtype in dtype, f"{name}: dtype {t.dtype}, expected one of {dtype}")
+    else:
+        _need(t.dtype == dtype, f"{name}: dtype {t.dtype}, expected {dtype}")
+    _need(t.is_contiguous(), f"{name}: must be contiguous")
+    if shape is not None:
+        _need(tuple(t.shape) == tuple(shape), f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
+
+
+def embed_lookup(ids: torch.Tensor, table: torch.Tensor, scale: float, out: torch.Tensor) -> None:
+    """out[i] = float32(table[ids[i]]) * scale.  ids int32 [n], table T [V, H], out float32 [n, H]."""
+    _dense(ids, "ids", torch.int32)
+    _need(ids.dim() == 1, "ids: expected one axis")
+    _dense(table, "table", _ACT)
+    _need(table.dim() == 2, "table: expected [vocab, hidden]")
+    _dense(out, "out", torch.float32, (ids.shape[0], table.shape[1]))
+    if ids.shape[0]:
+        backend().embed_lookup(ids, table, float(scale), out)
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, offset: float, out: torch.Tensor,
+             delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None) -> None:
+    """out = x * rsqrt(mean(x^2) + eps) * (offset + weight), all in float32, cast to out's dtype.
+
+    x float32 [n, H]; weight float32 [H]; out T [m, H].  With `delta` (T [n, H]) the
+    row normalised is x + delta.  Without `rows`, m = n and the sum is written back
+    to x (the residual stream moves on).  With `rows` (int32 [m]) only those rows are
+    read, x is left alone and out[i] belongs to row rows[i].
+    """
+    _dense(x, "x", torch.float32)
+    _need(x.dim() == 2, "x: expected [tokens, hidden]")
+    n, h = x.shape
+    _dense(weight, "weight", torch.float32, (h,))
+    if delta is not None:
+        _dense(delta, "delta", _ACT, (n, h))
+    m = n
+    if rows is not None:
+        _dense(rows, "rows", torch.int32)
+        _need(rows.dim() == 1, "rows: expected one axis")
+        m = rows.shape[0]
+    _dense(out, "out", _ACT, (m, h))
+    if m:
+        backend().rms_norm(x, weight, float(eps), float(offset), out, delta, rows)
+
+
+def rope_and_cache_write(qkv: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
+                         inv_freq: Optional[torch.Tensor], slots: Optional[torch.Tensor],
+                         cache: Optional[torch.Tensor], *, num_heads: int, num_kv_heads: int,
+                         head_dim: int, page_size: int) -> None:
+    """Adds `bias`, rotates queries and keys in place and stores keys and values in pages.
+
+    qkv T [n, (num_heads + 2*num_kv_heads) * head_dim]: queries, then keys, then values.
+    bias float32 of a row's width, or None.  positions int32 [n].  inv_freq float32
+    [rotary_dim/2] (None: no rotation): element j of a head is paired with j + rotary_dim/2
+    and the pair is turned by position * inv_freq[j], the angle and its sine and cosine in
+    float32.  slots int32 [n]: page * page_size + offset for each token; cache
+    T [pages, 2, num_kv_heads, page_size*head_dim] holds a page's keys as [page_size,
+    head_dim] and its values as [head_dim, page_size].  slots and cache None: nothing is
+    stored (the layer reads another layer's cache).
+    """
+    width = (num_heads + 2 * num_kv_heads) * head_dim
+    _dense(qkv, "qkv", _ACT)
+    _need(qkv.dim() == 2 and qkv.shape[1] == width, f"qkv: shape {tuple(qkv.shape)}, expected [n, {width}]")
+    n = qkv.shape[0]
+    if bias is not None:
+        _dense(bias, "bias", torch.float32, (width,))
+    _dense(positions, "positions", torch.int32, (n,))
+    rotary_dim = 0
+    if inv_freq is not None:
+        _dense(inv_freq, "inv_freq", torch.float32)
+        _need(inv_freq.dim() == 1, "inv_freq: expected one axis")
+        rotary_dim = 2 * inv_freq.shape[0]
+        _need(0 < rotary_dim <= head_dim, f"rotary_dim {rotary_dim} does not fit head_dim {head_dim}")
+    _need((slots is None) == (cache is None), "slots and cache go together")
+    if cache is not None:
+        _dense(slots, "slots", torch.int32, (n,))
+        _dense(cache, "cache", qkv.dtype)
+        _need(cache.dim() == 4 and tuple(cache.shape[1:]) == (2, num_kv_heads, page_size * head_dim),
+              f"cache: shape {tuple(cache.shape)}, expected [pages, 2, {num_kv_heads}, {page_size * head_dim}]")
+    if n:
+        backend().rope_and_cache_write(qkv, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads,
+                                       head_dim, rotary_dim, page_size)
+
+
+def paged_attention(qkv: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor,
+                    token_segment: torch.Tensor, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor,
+                    seg_ctx_len: torch.Tensor, out: torch.Tensor, *, num_heads: int, num_kv_heads: int,
+                    head_dim: int, page_size: int, scale: float, window: int = 0,
+                    max_q_len: int = 0, max_ctx_len: int = 0) -> None:
+    """Softmax attention of every query over the keys of its own request in the paged cache.
+
+    The batch is a row of segments; segment s holds tokens seg_q_start[s] .. +seg_q_len[s],
+    the last seg_q_len[s] positions of a request that is seg_ctx_len[s] long after this
+    step.  Token i of it is at position p = ctx_len - q_len + i and sees keys
+    max(0, p - window + 1) .. p (window 0: from key 0).  Query head h uses key/value head
+    h // (num_heads // num_kv_heads).  Scores are scaled by `scale`; scores, softmax and the
+    weighted sum accumulate in float32.  qkv as in `rope_and_cache_write` (only the queries
+    are read); block_tables int32 [S, max_pages]; out T [n, num_heads*head_dim].
+    max_q_len / max_ctx_len are host-side bounds of the segment arrays (0: unknown).
+    """
+    width = (num_heads + 2 * num_kv_heads) * head_dim
+    _dense(qkv, "qkv", _ACT)
+    _need(qkv.dim() == 2 and qkv.shape[1] == width, f"qkv: shape {tuple(qkv.shape)}, expected [n, {width}]")
+    n = qkv.shape[0]
+    _need(num_heads % num_kv_heads == 0, "num_heads must be a multiple of num_kv_heads")
+    _dense(cache, "cache", qkv.dtype)
+    _need(cache.dim() == 4 and tuple(cache.shape[1:]) == (2, num_kv_heads, page_size * head_dim),
+          f"cache: shape {tuple(cache.shape)}, expected [pages, 2, {num_kv_heads}, {page_size * head_dim}]")
+    _dense(block_tables, "block_tables", torch.int32)
+    _need(block_tables.dim() == 2, "block_tables: expected [segments, pages]")
+    s = block_tables.shape[0]
+    _dense(token_segment, "token_segment", torch.int32, (n,))
+    for name, t in (("seg_q_start", seg_q_start), ("seg_q_len", seg_q_len), ("seg_ctx_len", seg_ctx_len)):
+        _dense(t, name, torch.int32, (s,))
+    _dense(out, "out", qkv.dtype, (n, num_heads * head_dim))
+    _need(window >= 0, "window must not be negative")
+    if n:
+        backend().paged_attention(qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len,
+                                  out, num_heads, num_kv_heads, head_dim, page_size, float(scale), int(window),
+                                  int(max_q_len), int(max_ctx_len))
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> None:
+    """out = x @ weight^T.  x T [m, k]; weight T [n, k]; out T or float32 [m, n].
+    Products of bfloat16 accumulate in float32; float32 stays float32 throughout."""
+    _dense(x, "x", _ACT)
+    _need(x.dim() == 2, "x: expected [rows, in]")
+    _dense(weight, "weight", x.dtype)
+    _need(weight.dim() == 2 and weight.shape[1] == x.shape[1],
+          f"weight: shape {tuple(weight.shape)}, expected [out, {x.shape[1]}]")
+    _dense(out, "out", (x.dtype, torch.float32), (x.shape[0], weight.shape[0]))
+    if x.shape[0]:
+        backend().linear(x, weight, out)
+
+
+ACTIVATIONS = ("gelu_tanh", "silu")
+
+
+def gated_activation(gate_up: torch.Tensor, out: torch.Tensor, activation: str) -> None:
+    """out = act(gate_up[:, :I]) * gate_up[:, I:], in float32, cast to T.  gate_up T [n, 2I]."""
+    _need(activation in ACTIVATIONS, f"activation {activation!r}: expected one of {ACTIVATIONS}")
+    _dense(gate_up, "gate_up", _ACT)
+    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "gate_up: expected [n, 2*intermediate]")
+    _dense(out, "out", gate_up.dtype, (gate_up.shape[0], gate_up.shape[1] // 2))
+    if gate_up.shape[0]:
+        backend().gated_activation(gate_up, out, activation)
+
+
+def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> None:
+    """out[i] = index of the largest value of row i, the lowest index among equals.
+    logits float32 [m, V]; out int32 [m]."""
+    _dense(logits, "logits", torch.float32)
+    _need(logits.dim() == 2 and logits.shape[1] > 0, "logits: expected [rows, vocab]")
+    _dense(out, "out", torch.int32, (logits.shape[0],))
+    if logits.shape[0]:
+        backend().argmax_rows(logits, out)
+
+
+def sample_rows(logits: torch.Tensor, params: torch.Tensor, seeds: torch.Tensor,
+                penalty_ids: Optional[torch.Tensor], penalty_offsets: Optional[torch.Tensor],
+                out_tokens: torch.Tensor, out_logprobs: torch.Tensor) -> None:
+    """Samples one token per row.
+
+    logits float32 [m, V].  params float32 [m, 5]: temperature (0: greedy), top_k (0: off),
+    top_p (1: off), min_p (0: off), repetition_penalty (1: off).  seeds int64 [m, 2]: the
+    key and counter of the row's uniform draw.  penalty_ids int32 [P] with penalty_offsets
+    int32 [m+1]: the ids the repetition penalty applies to, row by row (None: no row has
+    any).  out_tokens int32 [m]; out_logprobs float32 [m]: log-probability of the token
+    under the penalised, temperature-scaled distribution before truncation (temperature 1
+    for greedy rows).
+    """
+    _dense(logits, "logits", torch.float32)
+    _need(logits.dim() == 2 and logits.shape[1] > 0, "logits: expected [rows, vocab]")
+    m = logits.shape[0]
+    _dense(params, "params", torch.float32, (m, 5))
+    _dense(seeds, "seeds", torch.int64, (m, 2))
+    _need((penalty_ids is None) == (penalty_offsets is None), "penalty_ids and penalty_offsets go together")
+    if penalty_ids is not None:
+        _dense(penalty_ids, "penalty_ids", torch.int32)
+        _dense(penalty_offsets, "penalty_offsets", torch.int32, (m + 1,))
+    _dense(out_tokens, "out_tokens", torch.int32, (m,))
+    _dense(out_logprobs, "out_logprobs", torch.float32, (m,))
+    if m:
+        backend().sample_rows(logits, params, seeds, penalty_ids, penalty_offsets, out_tokens, out_logprobs)

@@ -1,0 +1,93 @@
+"""The attention mixer: q/k/v projection as one product, rotation and cache write
+as one kernel, attention over the request's pages, output projection.
+
+It follows the reference's attention (src/wllm/models/llama.py:82-115 for the
+formulas, :143-247 for the cached forms) with one code path for all of them: a
+flat batch of segments, each the next tokens of some request, a decoded token
+being a segment of one.  Head h of the q/k/v rows is columns h*head_dim ..
+(h+1)*head_dim of the projection (llama.py:103-105).  The three projection
+matrices are stacked at load so that one product makes the [n, (nh+2nkv)*d]
+row the kernels read.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from wllm_amd.cache.manager import CacheNeed
+from wllm_amd.kernels import ops
+from wllm_amd.parts.registry import build_position, register_mixer
+from wllm_amd.parts.specs import AttentionSpec
+from wllm_amd.weights.checkpoint import ExpectedTensor
+
+
+@register_mixer("attention")
+class PagedAttention:
+    def __init__(self, spec: AttentionSpec):
+        if spec.num_heads % spec.num_kv_heads:
+            raise ValueError("num_heads must be a multiple of num_kv_heads")
+        if spec.window is not None and spec.window <= 0:
+            raise ValueError(f"window must be positive or None, got {spec.window}")
+        self.spec = spec
+        self.position = build_position(spec.position)
+        self.w_qkv = None
+        self.b_qkv = None
+        self.w_o = None
+
+    @property
+    def qkv_width(self) -> int:
+        s = self.spec
+        return (s.num_heads + 2 * s.num_kv_heads) * s.head_dim
+
+    def expected_tensors(self) -> dict:
+        s = self.spec
+        q, kv = s.num_heads * s.head_dim, s.num_kv_heads * s.head_dim
+        out = {
+            s.q_weight: ExpectedTensor((q, s.hidden_size)),
+            s.k_weight: ExpectedTensor((kv, s.hidden_size)),
+            s.v_weight: ExpectedTensor((kv, s.hidden_size)),
+            s.o_weight: ExpectedTensor((s.hidden_size, q)),
+        }
+        for name, width in ((s.q_bias, q), (s.k_bias, kv), (s.v_bias, kv)):
+            if name is not None:
+                out[name] = ExpectedTensor((width,), role="vector")
+        return out
+
+    def load(self, fetch) -> None:
+        s = self.spec
+        w = torch.cat([fetch.matrix(s.q_weight), fetch.matrix(s.k_weight), fetch.matrix(s.v_weight)], dim=0)
+        self.w_qkv = fetch.to_device(w)
+        self.w_o = fetch.to_device(fetch.matrix(s.o_weight))
+        if s.q_bias is not None or s.k_bias is not None or s.v_bias is not None:
+            q, kv = s.num_heads * s.head_dim, s.num_kv_heads * s.head_dim
+            parts = [fetch.vector(name) if name is not None else torch.zeros(width)
+                     for name, width in ((s.q_bias, q), (s.k_bias, kv), (s.v_bias, kv))]
+            self.b_qkv = fetch.to_device(torch.cat(parts))
+        self.position.prepare(fetch.device)
+
+    def cache_need(self) -> Optional[CacheNeed]:
+        return CacheNeed(self.spec.num_kv_heads, self.spec.head_dim, self.spec.window)
+
+    def state_shape(self):
+        return None
+
+    def forward(self, ctx, entry: int, h: torch.Tensor) -> torch.Tensor:
+        s = self.spec
+        n = h.shape[0]
+        qkv = ctx.buffer("qkv", (n, self.qkv_width), h.dtype)
+        ops.linear(h, self.w_qkv, qkv)
+        pages = ctx.pages(entry)
+        ops.rope_and_cache_write(
+            qkv, self.b_qkv, ctx.positions, self.position.inv_freq,
+            pages.slots if pages.writes else None, pages.storage if pages.writes else None,
+            num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim, page_size=pages.page_size)
+        attn = ctx.buffer("attn", (n, s.num_heads * s.head_dim), h.dtype)
+        ops.paged_attention(
+            qkv, pages.storage, pages.block_tables, ctx.token_segment, ctx.seg_q_start, ctx.seg_q_len,
+            ctx.seg_ctx_len, attn, num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim,
+            page_size=pages.page_size, scale=s.scale, window=s.window or 0,
+            max_q_len=ctx.max_q_len, max_ctx_len=ctx.max_ctx_len)
+        y = ctx.buffer("mixer_out", (n, s.hidden_size), h.dtype)
+        ops.linear(attn, self.w_o, y)
+        return y

@@ -1,0 +1,46 @@
+"""Feed-forward parts.  "gated_mlp": down(act(gate(x)) * up(x)) without biases;
+with act = gelu_tanh it is the reference's GemmaMLP (src/wllm/models/gemma.py:54-62).
+Gate and up matrices are stacked at load so that one product makes both halves
+of the row the activation kernel reads."""
+from __future__ import annotations
+
+import torch
+
+from wllm_amd.kernels import ops
+from wllm_amd.parts.registry import register_feed_forward
+from wllm_amd.parts.specs import GatedMLPSpec
+from wllm_amd.weights.checkpoint import ExpectedTensor
+
+
+@register_feed_forward("gated_mlp")
+class GatedMLP:
+    def __init__(self, spec: GatedMLPSpec):
+        if spec.activation not in ops.ACTIVATIONS:
+            raise ValueError(f"activation {spec.activation!r} is not implemented; known: {ops.ACTIVATIONS}")
+        self.spec = spec
+        self.w_gate_up = None
+        self.w_down = None
+
+    def expected_tensors(self) -> dict:
+        s = self.spec
+        return {
+            s.gate_weight: ExpectedTensor((s.intermediate_size, s.hidden_size)),
+            s.up_weight: ExpectedTensor((s.intermediate_size, s.hidden_size)),
+            s.down_weight: ExpectedTensor((s.hidden_size, s.intermediate_size)),
+        }
+
+    def load(self, fetch) -> None:
+        s = self.spec
+        self.w_gate_up = fetch.to_device(torch.cat([fetch.matrix(s.gate_weight), fetch.matrix(s.up_weight)], dim=0))
+        self.w_down = fetch.to_device(fetch.matrix(s.down_weight))
+
+    def forward(self, ctx, h: torch.Tensor) -> torch.Tensor:
+        s = self.spec
+        n = h.shape[0]
+        gate_up = ctx.buffer("gate_up", (n, 2 * s.intermediate_size), h.dtype)
+        ops.linear(h, self.w_gate_up, gate_up)
+        act = ctx.buffer("ffn_act", (n, s.intermediate_size), h.dtype)
+        ops.gated_activation(gate_up, act, s.activation)
+        y = ctx.buffer("ffn_out", (n, s.hidden_size), h.dtype)
+        ops.linear(act, self.w_down, y)
+        return y

@@ -1,0 +1,57 @@
+"""Registries of part kinds: norm, position encoding, mixer, feed-forward, block.
+
+A part is a class built from its specification alone.  It says which checkpoint
+tensors it expects, loads them, and runs on the flat batch of a step.  The
+interfaces:
+
+norm          expected_tensors(); load(fetch); forward(x, out, delta=None, rows=None)
+position      prepare(dtype, device); arguments for the mixer's rotation kernel
+mixer         expected_tensors(); load(fetch); cache_need() -> CacheNeed | None;
+              state_shape() -> tuple | None; forward(ctx, entry, h) -> y
+feed-forward  expected_tensors(); load(fetch); forward(ctx, h) -> y
+block         built from a BlockSpec and the parts above; forward(ctx, entry, stream)
+
+`ctx` is the step's `StepContext`, `entry` the index of the schedule entry being
+run, `h` the normalised input [tokens, hidden] in the activation dtype, `y` the
+part's contribution to the residual stream, same shape and dtype.
+"""
+from __future__ import annotations
+
+_NORMS: dict = {}
+_POSITIONS: dict = {}
+_MIXERS: dict = {}
+_FEED_FORWARDS: dict = {}
+_BLOCKS: dict = {}
+
+
+def _register(table: dict, what: str):
+    def register(kind: str, cls=None, *, replace: bool = False):
+        def add(c):
+            if kind in table and not replace:
+                raise ValueError(f"{what} kind {kind!r} is already registered")
+            table[kind] = c
+            return c
+        return add(cls) if cls is not None else add
+    return register
+
+
+def _build(table: dict, what: str):
+    def build(spec, *args, **kwargs):
+        kind = spec.kind if hasattr(spec, "kind") else spec.arrangement
+        if kind not in table:
+            raise ValueError(f"unknown {what} kind {kind!r}; registered: {sorted(table)}")
+        return table[kind](spec, *args, **kwargs)
+    return build
+
+
+register_norm = _register(_NORMS, "norm")
+register_position = _register(_POSITIONS, "position encoding")
+register_mixer = _register(_MIXERS, "mixer")
+register_feed_forward = _register(_FEED_FORWARDS, "feed-forward")
+register_block = _register(_BLOCKS, "block arrangement")
+
+build_norm = _build(_NORMS, "norm")
+build_position = _build(_POSITIONS, "position encoding")
+build_mixer = _build(_MIXERS, "mixer")
+build_feed_forward = _build(_FEED_FORWARDS, "feed-forward")
+build_block = _build(_BLOCKS, "block arrangement")
