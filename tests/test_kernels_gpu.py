@@ -1,0 +1,235 @@
+"""Each kernel alone against the plain emulation of its contract, at sizes other than
+the engine's tests use: widths and vocabularies that are no power of two, odd head
+counts and groups, partial rotation, windows, page sizes from 4 to 32."""
+import math
+
+import pytest
+import torch
+
+from kernel_emulation import EmulatedKernels
+from wllm_amd.kernels import ops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype):
+    # float32: accumulation order only; bfloat16: one rounding of the result (2^-8) on top
+    return (1e-5, 2e-5) if dtype == torch.float32 else (1e-2, 8e-3)
+
+
+def close(got, ref, dtype, what=""):
+    atol, rtol = tol(dtype)
+    got, ref = got.double().cpu(), ref.double().cpu()
+    err = ((got - ref).abs() / (atol + rtol * ref.abs())).max().item()
+    assert err <= 1.0, f"{what}: worst error {err:.2f} x tolerance, max abs diff {(got - ref).abs().max().item():.3e}"
+
+
+def both(fn_name, make, dtype):
+    """Runs an op on the GPU kernels and on the float64 emulation with equal operands."""
+    args_gpu, kwargs = make()
+    args_ref = [a.clone() if isinstance(a, torch.Tensor) else a for a in args_gpu]
+    getattr(ops, fn_name)(*args_gpu, **kwargs)
+    torch.cuda.synchronize()
+    with ops.use_backend(EmulatedKernels(precise=True)):
+        getattr(ops, fn_name)(*args_ref, **kwargs)
+    return args_gpu, args_ref
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("vocab,hidden,n", [(1000, 200, 37), (777, 96, 1), (4099, 2048, 5)])
+def test_embed_lookup(dtype, vocab, hidden, n):
+    torch.manual_seed(0)
+    table = torch.randn(vocab, hidden, device=DEV).to(dtype)
+    ids = torch.randint(0, vocab, (n,), device=DEV, dtype=torch.int32)
+    ids[0] = vocab - 1
+    out = torch.zeros(n, hidden, device=DEV)
+    ops.embed_lookup(ids, table, 3.25, out)
+    assert torch.equal(out, table[ids.long()].float() * 3.25)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden,n", [(200, 9), (96, 3), (2048, 4), (3072, 2), (70, 130)])
+@pytest.mark.parametrize("mode", ["plain", "delta", "rows", "delta_rows"])
+def test_rms_norm(dtype, hidden, n, mode):
+    torch.manual_seed(1)
+
+    def make():
+        x = torch.randn(n, hidden, device=DEV) * 3
+        w = torch.randn(hidden, device=DEV) * 0.2
+        delta = torch.randn(n, hidden, device=DEV).to(dtype) if "delta" in mode else None
+        rows = torch.tensor([n - 1, 0, n // 2], device=DEV, dtype=torch.int32) if "rows" in mode else None
+        out = torch.zeros(3 if rows is not None else n, hidden, device=DEV, dtype=dtype)
+        return [x, w, 1e-5, 1.0, out], dict(delta=delta, rows=rows)
+
+    torch.manual_seed(1)
+    g, r = both("rms_norm", make, dtype)
+    close(g[4], r[4], dtype, "out")
+    close(g[0], r[0], torch.float32, "residual stream")
+    if mode == "rows":
+        assert torch.equal(g[0], r[0]), "x is left alone when rows are given"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,rot,ps,bias", [(3, 1, 40, 24, 8, True), (8, 1, 256, 256, 16, False),
+                                                 (6, 6, 24, 24, 4, False), (4, 2, 64, 32, 32, True)])
+def test_rope_and_cache_write(dtype, nh, nkv, d, rot, ps, bias):
+    n, pages = 29, 12
+    torch.manual_seed(2)
+    width = (nh + 2 * nkv) * d
+
+    def make():
+        qkv = torch.randn(n, width, device=DEV).to(dtype)
+        b = torch.randn(width, device=DEV) * 0.1 if bias else None
+        positions = torch.randint(0, 5000, (n,), device=DEV, dtype=torch.int32)
+        positions[0] = 0
+        inv_freq = (1.0 / (10000.0 ** (torch.arange(0, rot, 2, dtype=torch.float32) / rot))).to(DEV)
+        slots = torch.randperm(pages * ps, device=DEV)[:n].to(torch.int32)
+        cache = torch.full((pages, 2, nkv, ps * d), 7.0, device=DEV, dtype=dtype)
+        return [qkv, b, positions, inv_freq, slots, cache], dict(num_heads=nh, num_kv_heads=nkv, head_dim=d, page_size=ps)
+
+    torch.manual_seed(2)
+    g, r = both("rope_and_cache_write", make, dtype)
+    close(g[0], r[0], dtype, "rotated rows")
+    # the cache holds exactly what the rows hold, and nothing else moved
+    k_rows = g[0].view(n, nh + 2 * nkv, d)[:, nh:nh + nkv]
+    v_rows = g[0].view(n, nh + 2 * nkv, d)[:, nh + nkv:]
+    slots = g[4].long()
+    kview = g[5][:, 0].view(pages, nkv, ps, d)
+    vview = g[5][:, 1].view(pages, nkv, d, ps)
+    assert torch.equal(kview[slots // ps, :, slots % ps, :], k_rows)
+    assert torch.equal(vview[slots // ps, :, :, slots % ps], v_rows)
+    untouched = torch.ones(pages * ps, dtype=torch.bool, device=DEV)
+    untouched[slots] = False
+    assert (kview.permute(0, 2, 1, 3).reshape(pages * ps, -1)[untouched] == 7.0).all()
+    assert (vview.permute(0, 3, 1, 2).reshape(pages * ps, -1)[untouched] == 7.0).all()
+
+
+def test_rope_position_zero_is_identity_and_no_cache():
+    nh, nkv, d = 2, 1, 16
+    qkv = torch.randn(3, (nh + 2 * nkv) * d, device=DEV)
+    before = qkv.clone()
+    inv_freq = (1.0 / (100.0 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).to(DEV)
+    ops.rope_and_cache_write(qkv, None, torch.zeros(3, device=DEV, dtype=torch.int32), inv_freq, None, None,
+                             num_heads=nh, num_kv_heads=nkv, head_dim=d, page_size=4)
+    assert torch.equal(qkv, before)
+
+
+def _attention_case(dtype, nh, nkv, d, ps, segs, window, seed=0, spike=False):
+    """segs: list of (q_len, ctx_len).  Pages are handed out in a shuffled order."""
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    n = sum(q for q, _ in segs)
+    pages_needed = sum(-(-c // ps) for _, c in segs)
+    pages = pages_needed + 5
+    order = torch.randperm(pages, generator=g).tolist()
+    max_pages = max(-(-c // ps) for _, c in segs)
+    bt = torch.zeros(len(segs), max_pages, dtype=torch.int32)
+    for s, (_, c) in enumerate(segs):
+        for p in range(-(-c // ps)):
+            bt[s, p] = order.pop()
+    cache = torch.randn(pages, 2, nkv, ps * d, generator=g).to(dtype)
+    qkv = torch.randn(n, (nh + 2 * nkv) * d, generator=g).to(dtype)
+    if spike:
+        # one far key that must dominate: scale a query and its key so that the score stands out
+        qkv[:, :d] *= 4.0
+    q_len = torch.tensor([q for q, _ in segs], dtype=torch.int32)
+    ctx = torch.tensor([c for _, c in segs], dtype=torch.int32)
+    q_start = torch.cumsum(q_len, 0, dtype=torch.int32) - q_len
+    tok_seg = torch.repeat_interleave(torch.arange(len(segs), dtype=torch.int32), q_len.long())
+    out = torch.zeros(n, nh * d, dtype=dtype)
+    args = [t.to(DEV) for t in (qkv, cache, bt, tok_seg, q_start.to(torch.int32), q_len, ctx, out)]
+    kwargs = dict(num_heads=nh, num_kv_heads=nkv, head_dim=d, page_size=ps, scale=1.0 / math.sqrt(d), window=window,
+                  max_q_len=int(q_len.max()), max_ctx_len=int(ctx.max()))
+    return args, kwargs
+
+
+ATTENTION_SHAPES = [
+    # the reference's own kernel test: 14 query heads, 2 kv heads, head 64, pages of 16
+    # (tests/test_paged_attention_kernel.py:11-15,69-91), context lengths 1, 5, 16, 17, 33, 100
+    (14, 2, 64, 16, [(1, 1), (1, 5), (1, 16), (1, 17), (1, 33), (1, 100)], 0),
+    (8, 1, 256, 16, [(1, 300), (7, 7), (33, 90), (1, 1)], 0),
+    (6, 6, 24, 8, [(5, 5), (16, 47), (1, 64), (2, 130)], 0),
+    (4, 1, 32, 4, [(23, 23), (1, 9), (3, 40)], 0),
+    (16, 16, 128, 32, [(1, 77), (40, 40)], 0),
+    (6, 2, 20, 16, [(9, 30), (1, 200)], 0),
+    (12, 1, 48, 16, [(1, 150), (20, 64)], 0),
+    (4, 2, 64, 16, [(1, 100), (30, 70), (50, 50)], 17),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,ps,segs,window", ATTENTION_SHAPES)
+def test_paged_attention(dtype, nh, nkv, d, ps, segs, window):
+    g, r = both("paged_attention", lambda: _attention_case(dtype, nh, nkv, d, ps, segs, window), dtype)
+    close(g[7], r[7], dtype, "attention output")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_finds_one_far_key(dtype):
+    """One key among hundreds carries the whole weight: its value must come out."""
+    nh, nkv, d, ps = 8, 1, 64, 16
+    args, kwargs = _attention_case(dtype, nh, nkv, d, ps, [(1, 700)], 0, seed=3)
+    qkv, cache, bt = args[0], args[1], args[2]
+    far = 123
+    page, off = int(bt[0, far // ps]), far % ps
+    kview = cache[:, 0].view(cache.shape[0], nkv, ps, d)
+    vview = cache[:, 1].view(cache.shape[0], nkv, d, ps)
+    q = qkv[0, :d].float()
+    kview[page, 0, off] = (q / q.norm() * 40.0).to(dtype)          # score far above the rest
+    ops.paged_attention(*args, **kwargs)
+    got = args[7][0, :d].float()
+    assert torch.allclose(got, vview[page, 0, :, off].float(), atol=2e-2), "the far key's value is the output"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(1, 100, 64), (7, 777, 250), (65, 130, 96), (128, 64, 2048), (3, 2560, 2048)])
+def test_linear(dtype, m, n, k):
+    torch.manual_seed(4)
+    for out_dtype in {dtype, torch.float32}:
+        def make():
+            x = torch.randn(m, k, device=DEV).to(dtype)
+            w = (torch.randn(n, k, device=DEV) / math.sqrt(k)).to(dtype)
+            return [x, w, torch.zeros(m, n, device=DEV, dtype=out_dtype)], {}
+        torch.manual_seed(4)
+        g, r = both("linear", make, dtype)
+        close(g[2], r[2], out_dtype, f"product to {out_dtype}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("act", ["gelu_tanh", "silu"])
+def test_gated_activation(dtype, act):
+    torch.manual_seed(5)
+
+    def make():
+        gu = (torch.randn(13, 2 * 250, device=DEV) * 3).to(dtype)
+        return [gu, torch.zeros(13, 250, device=DEV, dtype=dtype), act], {}
+
+    torch.manual_seed(5)
+    g, r = both("gated_activation", make, dtype)
+    close(g[1], r[1], dtype)
+    if act == "gelu_tanh":
+        ref = torch.nn.functional.gelu(g[0][:, :250].float(), approximate="tanh") * g[0][:, 250:].float()
+        close(g[1], ref, dtype, "against the library's gelu")
+
+
+def test_argmax_rows_lowest_index_among_equals():
+    torch.manual_seed(6)
+    logits = torch.randn(9, 777, device=DEV)
+    logits[2, 500] = logits[2, 30] = 50.0
+    logits[3] = 0.0
+    logits[4, 776] = 60.0
+    out = torch.zeros(9, device=DEV, dtype=torch.int32)
+    ops.argmax_rows(logits, out)
+    assert out.tolist() == logits.argmax(-1).tolist()
+    assert out[2] == 30 and out[3] == 0 and out[4] == 776
+
+
+def test_shape_errors_are_raised_on_the_host():
+    x = torch.zeros(4, 64, device=DEV)
+    with pytest.raises(ops.KernelShapeError):
+        ops.rms_norm(x, torch.zeros(63, device=DEV), 1e-6, 1.0, torch.zeros(4, 64, device=DEV))
+    with pytest.raises(ops.KernelShapeError):
+        ops.linear(x, torch.zeros(10, 32, device=DEV), torch.zeros(4, 10, device=DEV))
+    with pytest.raises(ops.KernelShapeError):
+        ops.linear(x.to(torch.bfloat16), torch.zeros(10, 64, device=DEV), torch.zeros(4, 10, device=DEV))

@@ -1,0 +1,56 @@
+// Shared by all kernels: element types, conversions, reductions over a 64-wide
+// wavefront and over a workgroup, launch checks.  gfx950 only.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define WLLM_API extern "C" __attribute__((visibility("default")))
+
+constexpr int kWave = 64;
+
+// bfloat16 as its bits; conversions are explicit so that every rounding is visible.
+struct bf16 {
+    uint16_t bits;
+};
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(bf16 v) { return __uint_as_float(static_cast<uint32_t>(v.bits) << 16); }
+
+template <typename T> __device__ __forceinline__ T from_float(float v);
+template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16 from_float<bf16>(float v) {
+    // round to nearest, ties to even; NaN stays NaN
+    uint32_t x = __float_as_uint(v);
+    if ((x & 0x7fffffffu) > 0x7f800000u) return bf16{static_cast<uint16_t>((x >> 16) | 0x0040u)};
+    x += 0x7fffu + ((x >> 16) & 1u);
+    return bf16{static_cast<uint16_t>(x >> 16)};
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+// Sum over a workgroup of up to 1024 threads; `scratch` holds 16 floats.  Every thread
+// gets the result.  The order of the additions is fixed by the thread ids.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int waves = (blockDim.x + kWave - 1) / kWave;
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float total = 0.f;
+    for (int w = 0; w < waves; ++w) total += scratch[w];
+    return total;
+}
+
+// The error a launch left, as an int for the caller (0 = hipSuccess).
+__host__ inline int launch_status() { return static_cast<int>(hipGetLastError()); }

@@ -1,0 +1,206 @@
+// Embedding lookup, RMS norm with residual add, rotation with cache write, gated
+// activation.  Each is bound by memory traffic; the fusions are the ones that save
+// a pass over the residual stream or over the q/k/v rows.
+#include "common.h"
+
+// ---- embedding: out[i] = float(table[ids[i]]) * scale ---------------------------------
+template <typename T>
+__global__ void embed_lookup_kernel(const int* __restrict__ ids, const T* __restrict__ table, float scale,
+                                    float* __restrict__ out, int hidden, int vocab) {
+    const int row = blockIdx.x;
+    int id = ids[row];
+    // ids are checked on the host; clamp all the same so that a bad id cannot fault
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    const T* src = table + static_cast<size_t>(id) * hidden;
+    float* dst = out + static_cast<size_t>(row) * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]) * scale;
+}
+
+template <typename T>
+static int embed_lookup_launch(const int* ids, const void* table, float scale, float* out, int n, int hidden,
+                               int vocab, hipStream_t stream) {
+    embed_lookup_kernel<T><<<n, 256, 0, stream>>>(ids, static_cast<const T*>(table), scale, out, hidden, vocab);
+    return launch_status();
+}
+
+WLLM_API int wllm_embed_lookup(const int* ids, const void* table, int is_bf16, float scale, float* out, int n,
+                               int hidden, int vocab, hipStream_t stream) {
+    return is_bf16 ? embed_lookup_launch<bf16>(ids, table, scale, out, n, hidden, vocab, stream)
+                   : embed_lookup_launch<float>(ids, table, scale, out, n, hidden, vocab, stream);
+}
+
+// ---- RMS norm: out = v * rsqrt(mean(v^2) + eps) * (offset + w), v = x (+ delta) ------------
+// One workgroup per output row.  Without `rows` the sum x + delta is written back to x.
+template <typename TD, typename TO>
+__global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ delta, const float* __restrict__ weight,
+                                const int* __restrict__ rows, TO* __restrict__ out, int hidden, float eps,
+                                float offset) {
+    __shared__ float scratch[16];
+    const int orow = blockIdx.x;
+    const int irow = rows ? rows[orow] : orow;
+    float* xr = x + static_cast<size_t>(irow) * hidden;
+    const TD* dr = delta ? delta + static_cast<size_t>(irow) * hidden : nullptr;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float v = xr[i];
+        if (dr) {
+            v += to_float(dr[i]);
+            if (!rows) xr[i] = v;
+        }
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = rsqrtf(ss / static_cast<float>(hidden) + eps);
+    TO* o = out + static_cast<size_t>(orow) * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float v = xr[i];
+        if (dr && rows) v += to_float(dr[i]);
+        o[i] = from_float<TO>(v * inv * (offset + weight[i]));
+    }
+}
+
+WLLM_API int wllm_rms_norm(float* x, const void* delta, int delta_bf16, const float* weight, const int* rows,
+                           void* out, int out_bf16, int num_out_rows, int hidden, float eps, float offset,
+                           hipStream_t stream) {
+    const int threads = hidden >= 1024 ? 256 : (hidden >= 256 ? 128 : 64);
+#define LAUNCH(TD, TO)                                                                                         \
+    rms_norm_kernel<TD, TO><<<num_out_rows, threads, 0, stream>>>(x, static_cast<const TD*>(delta), weight, rows, \
+                                                                  static_cast<TO*>(out), hidden, eps, offset)
+    if (delta_bf16 && out_bf16) LAUNCH(bf16, bf16);
+    else if (delta_bf16) LAUNCH(bf16, float);
+    else if (out_bf16) LAUNCH(float, bf16);
+    else LAUNCH(float, float);
+#undef LAUNCH
+    return launch_status();
+}
+
+// ---- rotation of queries and keys, bias, and the write of keys and values into pages ----------
+// One workgroup per token.  A row of qkv is [num_heads | num_kv_heads | num_kv_heads] heads of
+// head_dim.  Element j < rotary_dim/2 of a query or key head is paired with j + rotary_dim/2 and
+// the pair is turned by position * inv_freq[j]; angle, sine and cosine are float32.  Keys go to
+// the cache as [page_size, head_dim], values transposed as [head_dim, page_size].
+template <typename T>
+__global__ void rope_cache_kernel(T* __restrict__ qkv, const float* __restrict__ bias, const int* __restrict__ positions,
+                                  const float* __restrict__ inv_freq, const int* __restrict__ slots,
+                                  T* __restrict__ cache, int num_heads, int num_kv_heads, int head_dim, int rotary_dim,
+                                  int page_size, long long num_pages) {
+    const int token = blockIdx.x;
+    const int width = (num_heads + 2 * num_kv_heads) * head_dim;
+    T* row = qkv + static_cast<size_t>(token) * width;
+    const float pos = static_cast<float>(positions[token]);
+    const int half = rotary_dim / 2;
+    const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * head_dim;
+    T* kpage = nullptr;
+    T* vpage = nullptr;
+    int off = 0;
+    if (cache) {
+        const int slot = slots[token];
+        const long long page = slot / page_size;
+        off = slot % page_size;
+        if (slot >= 0 && page < num_pages) {
+            kpage = cache + page * page_elems;
+            vpage = kpage + static_cast<size_t>(num_kv_heads) * page_size * head_dim;
+        }
+    }
+    // rotated pairs of query and key heads
+    const int rot_heads = num_heads + num_kv_heads;
+    for (int idx = threadIdx.x; idx < rot_heads * half; idx += blockDim.x) {
+        const int head = idx / half, j = idx % half;
+        const int ia = head * head_dim + j, ib = ia + half;
+        float a = to_float(row[ia]), b = to_float(row[ib]);
+        if (bias) {
+            a += bias[ia];
+            b += bias[ib];
+        }
+        float s, c;
+        sincosf(pos * inv_freq[j], &s, &c);
+        const T ra = from_float<T>(a * c - b * s), rb = from_float<T>(b * c + a * s);
+        row[ia] = ra;
+        row[ib] = rb;
+        if (kpage && head >= num_heads) {
+            T* dst = kpage + (static_cast<size_t>(head - num_heads) * page_size + off) * head_dim;
+            dst[j] = ra;
+            dst[j + half] = rb;
+        }
+    }
+    // the part of query and key heads that is not rotated
+    const int rest = head_dim - rotary_dim;
+    if (rest > 0 && (bias || kpage)) {
+        for (int idx = threadIdx.x; idx < rot_heads * rest; idx += blockDim.x) {
+            const int head = idx / rest, j = rotary_dim + idx % rest;
+            const int i = head * head_dim + j;
+            T v = row[i];
+            if (bias) {
+                v = from_float<T>(to_float(v) + bias[i]);
+                row[i] = v;
+            }
+            if (kpage && head >= num_heads)
+                kpage[(static_cast<size_t>(head - num_heads) * page_size + off) * head_dim + j] = v;
+        }
+    }
+    // values
+    if (bias || vpage) {
+        const int vbase = rot_heads * head_dim;
+        for (int idx = threadIdx.x; idx < num_kv_heads * head_dim; idx += blockDim.x) {
+            const int head = idx / head_dim, j = idx % head_dim;
+            T v = row[vbase + idx];
+            if (bias) {
+                v = from_float<T>(to_float(v) + bias[vbase + idx]);
+                row[vbase + idx] = v;
+            }
+            if (vpage) vpage[(static_cast<size_t>(head) * head_dim + j) * page_size + off] = v;
+        }
+    }
+}
+
+WLLM_API int wllm_rope_cache_write(void* qkv, int is_bf16, const float* bias, const int* positions,
+                                   const float* inv_freq, const int* slots, void* cache, long long num_pages, int n,
+                                   int num_heads, int num_kv_heads, int head_dim, int rotary_dim, int page_size,
+                                   hipStream_t stream) {
+    if (is_bf16)
+        rope_cache_kernel<bf16><<<n, 256, 0, stream>>>(static_cast<bf16*>(qkv), bias, positions, inv_freq, slots,
+                                                       static_cast<bf16*>(cache), num_heads, num_kv_heads, head_dim,
+                                                       rotary_dim, page_size, num_pages);
+    else
+        rope_cache_kernel<float><<<n, 256, 0, stream>>>(static_cast<float*>(qkv), bias, positions, inv_freq, slots,
+                                                        static_cast<float*>(cache), num_heads, num_kv_heads, head_dim,
+                                                        rotary_dim, page_size, num_pages);
+    return launch_status();
+}
+
+// ---- gated activation: out = act(g) * u with g, u the two halves of a row -----------------------
+__device__ __forceinline__ float gelu_tanh(float z) {
+    // 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
+    const float k = 0.7978845608028654f;
+    return 0.5f * z * (1.f + tanhf(k * (z + 0.044715f * z * z * z)));
+}
+__device__ __forceinline__ float silu(float z) { return z / (1.f + expf(-z)); }
+
+template <typename T, int ACT>
+__global__ void gated_activation_kernel(const T* __restrict__ gate_up, T* __restrict__ out, long long total,
+                                        int inter) {
+    const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
+    for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const long long r = i / inter;
+        const int c = static_cast<int>(i % inter);
+        const float g = to_float(gate_up[r * 2 * inter + c]);
+        const float u = to_float(gate_up[r * 2 * inter + inter + c]);
+        out[i] = from_float<T>((ACT == 0 ? gelu_tanh(g) : silu(g)) * u);
+    }
+}
+
+WLLM_API int wllm_gated_activation(const void* gate_up, void* out, int is_bf16, int activation, int n, int inter,
+                                   hipStream_t stream) {
+    const long long total = static_cast<long long>(n) * inter;
+    long long blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+#define LAUNCH(T, A)                                                                                              \
+    gated_activation_kernel<T, A><<<static_cast<int>(blocks), 256, 0, stream>>>(static_cast<const T*>(gate_up), \
+                                                                                static_cast<T*>(out), total, inter)
+    if (is_bf16 && activation == 0) LAUNCH(bf16, 0);
+    else if (is_bf16) LAUNCH(bf16, 1);
+    else if (activation == 0) LAUNCH(float, 0);
+    else LAUNCH(float, 1);
+#undef LAUNCH
+    return launch_status();
+}

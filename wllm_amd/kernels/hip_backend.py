@@ -1,0 +1,109 @@
+"""Calls into the kernel library: tensors to raw pointers, the current stream, error codes
+to exceptions.  Shapes were checked in `ops`; what is checked here is that tensors live
+on the GPU, since a host pointer handed to a kernel faults the device."""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_longlong, c_void_p
+
+import torch
+
+from wllm_amd.kernels.library import load
+
+
+class KernelError(RuntimeError):
+    """A kernel launch failed or a kernel refused its operands."""
+
+
+def _ptr(t):
+    return c_void_p(t.data_ptr()) if t is not None else c_void_p(0)
+
+
+_SIGNATURES = {
+    "wllm_embed_lookup": [c_void_p, c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
+    "wllm_rms_norm": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float,
+                      c_void_p],
+    "wllm_rope_cache_write": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong, c_int,
+                              c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "wllm_gated_activation": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "wllm_paged_attention_generic": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+    "wllm_gemm_generic": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "wllm_argmax_rows": [c_void_p, c_void_p, c_int, c_int, c_void_p],
+}
+
+
+class HipBackend:
+    def __init__(self):
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible; the kernels run on gfx950 only and there is no other path")
+        self.lib = load()
+        for name, argtypes in _SIGNATURES.items():
+            fn = getattr(self.lib, name)
+            fn.argtypes = argtypes
+            fn.restype = c_int
+
+    @staticmethod
+    def _on_gpu(*tensors) -> None:
+        for t in tensors:
+            if t is not None and not t.is_cuda:
+                raise KernelError("a kernel operand is not on the GPU")
+
+    @staticmethod
+    def _stream() -> c_void_p:
+        return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    @staticmethod
+    def _check(code: int, what: str) -> None:
+        if code == -1:
+            raise KernelError(f"{what}: the kernel does not take these sizes")
+        if code != 0:
+            raise KernelError(f"{what}: HIP error {code}")
+
+    def embed_lookup(self, ids, table, scale, out):
+        self._on_gpu(ids, table, out)
+        self._check(self.lib.wllm_embed_lookup(_ptr(ids), _ptr(table), int(table.dtype == torch.bfloat16), scale,
+                                               _ptr(out), ids.shape[0], table.shape[1], table.shape[0],
+                                               self._stream()), "embed_lookup")
+
+    def rms_norm(self, x, weight, eps, offset, out, delta, rows):
+        self._on_gpu(x, weight, out, delta, rows)
+        self._check(self.lib.wllm_rms_norm(
+            _ptr(x), _ptr(delta), int(delta is not None and delta.dtype == torch.bfloat16), _ptr(weight), _ptr(rows),
+            _ptr(out), int(out.dtype == torch.bfloat16), out.shape[0], x.shape[1], eps, offset, self._stream()),
+            "rms_norm")
+
+    def rope_and_cache_write(self, qkv, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads, head_dim,
+                             rotary_dim, page_size):
+        self._on_gpu(qkv, bias, positions, inv_freq, slots, cache)
+        self._check(self.lib.wllm_rope_cache_write(
+            _ptr(qkv), int(qkv.dtype == torch.bfloat16), _ptr(bias), _ptr(positions), _ptr(inv_freq), _ptr(slots),
+            _ptr(cache), cache.shape[0] if cache is not None else 0, qkv.shape[0], num_heads, num_kv_heads, head_dim,
+            rotary_dim, page_size, self._stream()), "rope_and_cache_write")
+
+    def paged_attention(self, qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len, out,
+                        num_heads, num_kv_heads, head_dim, page_size, scale, window, max_q_len, max_ctx_len):
+        self._on_gpu(qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len, out)
+        if head_dim % 4 or head_dim > 256:
+            raise KernelError(f"paged_attention: head_dim {head_dim} is not a multiple of 4 up to 256")
+        self._check(self.lib.wllm_paged_attention_generic(
+            _ptr(qkv), _ptr(cache), int(qkv.dtype == torch.bfloat16), _ptr(block_tables), _ptr(token_segment),
+            _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out), qkv.shape[0], num_heads, num_kv_heads,
+            head_dim, page_size, block_tables.shape[1], scale, window, self._stream()), "paged_attention")
+
+    def linear(self, x, weight, out):
+        self._on_gpu(x, weight, out)
+        self._check(self.lib.wllm_gemm_generic(
+            _ptr(x), _ptr(weight), int(x.dtype == torch.bfloat16), _ptr(out), int(out.dtype == torch.bfloat16),
+            x.shape[0], weight.shape[0], x.shape[1], self._stream()), "linear")
+
+    def gated_activation(self, gate_up, out, activation):
+        self._on_gpu(gate_up, out)
+        self._check(self.lib.wllm_gated_activation(
+            _ptr(gate_up), _ptr(out), int(gate_up.dtype == torch.bfloat16), 0 if activation == "gelu_tanh" else 1,
+            gate_up.shape[0], out.shape[1], self._stream()), "gated_activation")
+
+    def argmax_rows(self, logits, out):
+        self._on_gpu(logits, out)
+        self._check(self.lib.wllm_argmax_rows(_ptr(logits), _ptr(out), logits.shape[0], logits.shape[1],
+                                              self._stream()), "argmax_rows")

@@ -1,0 +1,158 @@
+"""Building and loading the kernel library.
+
+The kernels under `wllm_amd/csrc` are compiled with hipcc for gfx950 into one
+shared library, `wllm_amd/libwllm_kernels.so`, whose `extern "C"` entry points
+are called through ctypes with raw device pointers and a stream.  Nothing of
+torch is compiled against, so a build takes about a minute from nothing.
+
+`load()` loads the library if it is built from the present sources and builds it
+first if not (a line is printed per compiled file, so that a first call in a
+fresh checkout shows what it is doing).  If the package folder cannot be
+written to, the build goes to a folder under the system's temporary directory.
+"""
+from __future__ import annotations
+
+import ctypes
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import time
+from concurrent.futures import ThreadPoolExecutor
+
+PACKAGE_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SOURCE_DIR = os.path.join(PACKAGE_DIR, "csrc")
+LIBRARY_NAME = "libwllm_kernels.so"
+ARCH = "gfx950"
+# packed float32 instructions are switched off for all device code
+FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
+         "-packed-fp32-ops", "-fvisibility=hidden", "-Wno-unused-command-line-argument"]
+
+
+class KernelLibraryMissing(RuntimeError):
+    """The kernel library is not built and cannot be built here."""
+
+
+def sources() -> list:
+    return sorted(f for f in os.listdir(SOURCE_DIR) if f.endswith(".hip"))
+
+
+def _fingerprint() -> str:
+    h = hashlib.sha256()
+    h.update(" ".join(FLAGS).encode())
+    for name in sorted(os.listdir(SOURCE_DIR)):
+        if name.endswith((".hip", ".h")):
+            h.update(name.encode())
+            with open(os.path.join(SOURCE_DIR, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.isfile(cand) and os.access(cand, os.X_OK):
+            return cand
+    raise KernelLibraryMissing("hipcc was not found (looked at $HIPCC, PATH and /opt/rocm/bin); "
+                               "the kernel library cannot be built")
+
+
+def _writable(folder: str) -> bool:
+    try:
+        os.makedirs(folder, exist_ok=True)
+        probe = os.path.join(folder, f".probe{os.getpid()}")
+        with open(probe, "w"):
+            pass
+        os.remove(probe)
+        return True
+    except OSError:
+        return False
+
+
+def _locations(fingerprint: str) -> list:
+    """(library path, object folder) candidates, in-tree first."""
+    fallback = os.path.join(tempfile.gettempdir(), f"wllm_amd_build_{os.getuid()}_{fingerprint[:16]}")
+    return [(os.path.join(PACKAGE_DIR, LIBRARY_NAME), os.path.join(SOURCE_DIR, "_build")),
+            (os.path.join(fallback, LIBRARY_NAME), os.path.join(fallback, "obj"))]
+
+
+def _is_current(lib_path: str, fingerprint: str) -> bool:
+    stamp = lib_path + ".stamp"
+    if not (os.path.isfile(lib_path) and os.path.isfile(stamp)):
+        return False
+    with open(stamp, "r", encoding="utf-8") as f:
+        return f.read().strip() == fingerprint
+
+
+def build(verbose: bool = True, force: bool = True) -> str:
+    """Compiles every source for gfx950 and links the library; returns its path."""
+    fingerprint = _fingerprint()
+    hipcc = _hipcc()
+    lib_path = obj_dir = None
+    for cand_lib, cand_obj in _locations(fingerprint):
+        if _writable(os.path.dirname(cand_lib)) and _writable(cand_obj):
+            lib_path, obj_dir = cand_lib, cand_obj
+            break
+    if lib_path is None:
+        raise KernelLibraryMissing("no writable place for the kernel library (package folder and temporary folder)")
+    if not force and _is_current(lib_path, fingerprint):
+        return lib_path
+    names = sources()
+    env = dict(os.environ)
+    env.setdefault("TMPDIR", tempfile.gettempdir())
+    t0 = time.time()
+
+    def say(msg: str) -> None:
+        if verbose:
+            print(f"[wllm_amd build] {msg}", file=sys.stderr, flush=True)
+
+    say(f"compiling {len(names)} kernel files for {ARCH} with {hipcc}")
+
+    def compile_one(name: str):
+        obj = os.path.join(obj_dir, name[:-4] + ".o")
+        cmd = [hipcc] + FLAGS + ["-I", SOURCE_DIR, "-c", os.path.join(SOURCE_DIR, name), "-o", obj]
+        r = subprocess.run(cmd, capture_output=True, text=True, env=env)
+        return name, obj, r
+
+    objects = []
+    with ThreadPoolExecutor(max_workers=min(8, max(1, len(names)))) as pool:
+        for name, obj, r in pool.map(compile_one, names):
+            if r.returncode != 0:
+                raise KernelLibraryMissing(f"hipcc failed on {name}:\n{r.stderr[-4000:]}")
+            say(f"compiled {name} ({time.time() - t0:.0f} s)")
+            objects.append(obj)
+    tmp = lib_path + f".tmp{os.getpid()}"
+    r = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", tmp] + objects,
+                       capture_output=True, text=True, env=env)
+    if r.returncode != 0:
+        raise KernelLibraryMissing(f"linking the kernel library failed:\n{r.stderr[-4000:]}")
+    os.replace(tmp, lib_path)
+    with open(lib_path + ".stamp", "w", encoding="utf-8") as f:
+        f.write(fingerprint)
+    say(f"built {lib_path} in {time.time() - t0:.0f} s")
+    return lib_path
+
+
+_loaded = None
+
+
+def load(verbose: bool = True) -> ctypes.CDLL:
+    """The loaded library; built first when no build of the present sources exists."""
+    global _loaded
+    if _loaded is not None:
+        return _loaded
+    fingerprint = _fingerprint()
+    path = None
+    for cand_lib, _ in _locations(fingerprint):
+        if _is_current(cand_lib, fingerprint):
+            path = cand_lib
+            break
+    if path is None:
+        path = build(verbose=verbose)
+    try:
+        _loaded = ctypes.CDLL(path)
+    except OSError as e:
+        raise KernelLibraryMissing(f"{path} cannot be loaded: {e}") from e
+    _loaded.wllm_path = path
+    return _loaded
