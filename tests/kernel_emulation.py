@@ -125,3 +125,16 @@ class EmulatedKernels:
     def argmax_rows(self, logits, out):
         self._count("argmax_rows")
         out.copy_(logits.argmax(dim=-1).to(torch.int32))
+
+    def sample_rows(self, logits, params, seeds, penalty_ids, penalty_offsets, out_tokens, out_logprobs):
+        from plain.sampling_plain import philox_uniform, sample_row
+        self._count("sample_rows")
+        for r in range(logits.shape[0]):
+            t, k, p, mp, pen = (float(x) for x in params[r])
+            gen = []
+            if penalty_ids is not None:
+                gen = penalty_ids[int(penalty_offsets[r]):int(penalty_offsets[r + 1])].tolist()
+            u = philox_uniform(int(seeds[r, 0]), int(seeds[r, 1]))
+            tok, lp, _, _ = sample_row(logits[r].cpu(), t, int(k), p, mp, pen, gen, u)
+            out_tokens[r] = tok
+            out_logprobs[r] = lp

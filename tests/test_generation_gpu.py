@@ -1,0 +1,149 @@
+"""Generation on the GPU through the entry point and the scheduler, the replay program as a
+subprocess, long decoding and the first tokens of a sequence."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import TINY, compare_with_plain, random_ids, replay_and_collect, trace_tail, trace_whole
+from plain import gemma_plain
+from wllm_amd.engine import LLM, ModelRunner, Request, Scheduler
+from wllm_amd.engine.replay import TraceReplayer
+from wllm_amd.parts import load_model
+from wllm_amd.sampling import SamplingParams
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def plain_model(folder):
+    return gemma_plain.read_config(folder), gemma_plain.read_weights(folder, torch.float32)
+
+
+@pytest.mark.parametrize("name,lengths,new", [("A", [7, 16, 23], 8), ("B", [5, 31, 64], 6), ("C", [9, 20], 6), ("M", [33, 70], 6)])
+def test_greedy_generation_through_the_entry_point_float32(model_folders, name, lengths, new):
+    # BASELINE's tiny workload: prompts of 7/16/23 ids, 8 greedy tokens each, pages of 4
+    cfg, w = plain_model(model_folders[name])
+    prompts = [random_ids(i + 1, n, cfg["vocab_size"]) for i, n in enumerate(lengths)]
+    llm = LLM(model_folders[name], dtype="float32", num_blocks=64, block_size=TINY[name]["page_size"])
+    outs = llm.generate(prompts, max_new_tokens=new)
+    for p, o in zip(prompts, outs):
+        assert o.token_ids == gemma_plain.generate_greedy(cfg, w, p, new)
+        assert o.finish_reason == "length" and len(o.logprobs) == new
+        full = gemma_plain.forward_logits(cfg, w, p + o.token_ids[:-1])
+        ref_lp = torch.log_softmax(full[len(p) - 1:].double(), -1).gather(-1, torch.tensor(o.token_ids)[:, None])[:, 0]
+        assert torch.allclose(torch.tensor(o.logprobs, dtype=torch.float64), ref_lp, atol=1e-4)
+    llm.runner.cache.check()
+
+
+@pytest.mark.parametrize("name", ["A", "M"])
+def test_greedy_generation_bfloat16_follows_the_plain_implementation_up_to_near_ties(model_folders, name):
+    cfg, w = plain_model(model_folders[name])
+    prompts = [random_ids(i + 50, n, cfg["vocab_size"]) for i, n in enumerate([12, 40])]
+    llm = LLM(model_folders[name], dtype="bfloat16", num_blocks=64, block_size=16)
+    for p, o in zip(prompts, llm.generate(prompts, max_new_tokens=8)):
+        tokens = list(p)
+        for t in o.token_ids:
+            logits = gemma_plain.forward_logits(cfg, w, tokens, scale_rounding=torch.bfloat16)[-1]
+            best = int(logits.argmax())
+            if t != best:
+                # a different token is acceptable only where the plain logits nearly tie
+                assert (logits[best] - logits[t]).item() < 2e-2, f"token {t} instead of {best}, gap {(logits[best] - logits[t]).item()}"
+                break
+            tokens.append(t)
+
+
+def test_chunked_prefill_beside_decodes_with_seeded_temperature(model_folders):
+    """BASELINE's second tiny workload: four prompts of 5/31/64/97 ids, portions of 16 beside
+    decoding requests, temperature 0.8 from a seeded generator, pages of 8.  Each request's tokens
+    equal those it gets alone, and each token is one the plain implementation's distribution gives
+    the request's uniform number."""
+    from plain import sampling_plain
+    folder = model_folders["B"]
+    cfg, w = plain_model(folder)
+    model = load_model(folder, "float32", "cuda")
+    prompts = [random_ids(7 * i + 3, n, cfg["vocab_size"]) for i, n in enumerate([5, 31, 64, 97])]
+    params = [SamplingParams(temperature=0.8, seed=500 + i) for i in range(4)]
+
+    def run(which, budget):
+        runner = ModelRunner.create(model, num_pages=40, page_size=8, max_requests=4)
+        s = Scheduler(runner, max_prefill_tokens_per_step=budget)
+        reqs = [Request(i, prompts[i], 10, sampling_params=params[i]) for i in which]
+        for r in reqs:
+            s.add_request(r)
+        s.run_to_completion()
+        runner.cache.check()
+        return reqs
+
+    together = run(range(4), 16)
+    for i, r in enumerate(together):
+        assert run([i], None)[0].output_token_ids == r.output_token_ids
+        tokens = list(prompts[i])
+        for k, t in enumerate(r.output_token_ids):
+            logits = gemma_plain.forward_logits(cfg, w, tokens)[-1]
+            u = sampling_plain.philox_uniform(r.seed, k)
+            _, _, _, (low, high) = sampling_plain.sample_row(logits, 0.8, 0, 1.0, 0.0, 1.0, [], u)
+            assert low[t] - 1e-4 <= u <= high[t] + 1e-4
+            tokens.append(t)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(model_folders, dtype):
+    """300 tokens decoded one by one after a short prompt, over many page boundaries."""
+    folder = model_folders["M"]
+    cfg, w = plain_model(folder)
+    toks = random_ids(9, 340, cfg["vocab_size"])
+    plain = {"r": gemma_plain.forward_logits(cfg, w, toks, scale_rounding=torch.bfloat16 if dtype == "bfloat16" else None)}
+    runner = ModelRunner.create(load_model(folder, dtype, "cuda"), num_pages=22, page_size=16, max_requests=2)
+    got = replay_and_collect(TraceReplayer(runner), trace_tail({"r": toks}, tail=300))
+    tol = dict(atol=2e-5, rtol=1e-4) if dtype == "float32" else dict(atol=1e-2, rtol=1e-2)
+    compare_with_plain(got, plain, **tol)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_first_tokens_of_a_sequence(model_folders, name, dtype):
+    """Prompts of one, two and three tokens, whole and token by token."""
+    folder = model_folders[name]
+    cfg, w = plain_model(folder)
+    requests = {f"r{n}": random_ids(n, n, cfg["vocab_size"]) for n in (1, 2, 3)}
+    plain = {rid: gemma_plain.forward_logits(cfg, w, t, scale_rounding=torch.bfloat16 if dtype == "bfloat16" else None)
+             for rid, t in requests.items()}
+    model = load_model(folder, dtype, "cuda")
+    tol = dict(atol=2e-5, rtol=1e-4) if dtype == "float32" else dict(atol=1e-2, rtol=1e-2)
+    for trace in (trace_whole(requests), trace_tail(requests, tail=3)):
+        runner = ModelRunner.create(model, num_pages=8, page_size=TINY[name]["page_size"], max_requests=2)
+        compare_with_plain(replay_and_collect(TraceReplayer(runner), trace), plain, **tol)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(model_folders, tmp_path, dtype):
+    """bin/trace_run as a user calls it: steps on standard input, `done <step>` lines, logits files."""
+    folder = model_folders["A"]
+    cfg, w = plain_model(folder)
+    a, b = random_ids(1, 30, 512), random_ids(2, 21, 512)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:17], "want": [0, 16]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[17:19], "want": []}, {"id": "b", "tokens": b[:20], "want": [19]}], "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": b[20:], "want": [0]}, {"id": "a", "tokens": a[19:], "want": [10]}], "end": ["a", "b"]},
+        {"step": 7, "entries": [{"id": "a", "tokens": b[:2], "want": [1]}], "end": ["a"]},
+    ]
+    out = tmp_path / "out"
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                           "--out", str(out), "--max-tokens", "128"],
+                          input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split() == ["done", "0", "done", "1", "done", "2", "done", "7"]
+    rounding = torch.bfloat16 if dtype == "bfloat16" else None
+    pa = gemma_plain.forward_logits(cfg, w, a, scale_rounding=rounding)
+    pb = gemma_plain.forward_logits(cfg, w, b, scale_rounding=rounding)
+    expect = {0: [pa[0], pa[16]], 1: [pb[19]], 2: [pb[20], pa[29]], 7: [pb[1]]}
+    atol, rtol = (2e-5, 1e-4) if dtype == "float32" else (1e-2, 1e-2)
+    for step, rows in expect.items():
+        got = torch.from_numpy(np.fromfile(out / f"{step}.f32", dtype="<f4").reshape(len(rows), 512))
+        ref = torch.stack(rows)
+        assert ((got.double() - ref.double()).abs() <= atol + rtol * ref.double().abs()).all(), f"step {step}"

@@ -1,0 +1,241 @@
+"""Pins of the plain implementation: what fixes each formula beside the reference's text.
+
+Special cases that reduce to a library routine, invariants, and the vectors the
+reference's own tests hold.  Each is chosen so that a plausible mistake fails it: a wrong
+sign or pairing in the rotation, a norm that multiplies by w instead of 1 + w, a scale by
+hidden/heads instead of head_dim, a head mapped to the wrong key/value head.
+"""
+import math
+
+import pytest
+import torch
+
+from plain import gemma_plain as P
+from plain import sampling_plain as S
+
+torch.manual_seed(0)
+
+
+# ---- norm ---------------------------------------------------------------------------
+def test_norm_with_zero_weight_is_plain_normalisation():
+    x = torch.randn(5, 48, dtype=torch.float64)
+    y = P.rms_norm_one_plus_w(x, torch.zeros(48, dtype=torch.float64), 1e-6)
+    assert torch.allclose(y, x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6))
+    # unit-RMS rows, eps 0: identity
+    x = x / x.pow(2).mean(-1, keepdim=True).sqrt()
+    assert torch.allclose(P.rms_norm_one_plus_w(x, torch.zeros(48, dtype=torch.float64), 0.0), x)
+
+
+def test_norm_weight_is_an_offset_from_one():
+    x = torch.randn(3, 16, dtype=torch.float64)
+    w = torch.randn(16, dtype=torch.float64)
+    base = P.rms_norm_one_plus_w(x, torch.zeros(16, dtype=torch.float64), 1e-6)
+    assert torch.allclose(P.rms_norm_one_plus_w(x, w, 1e-6), base * (1 + w))
+    assert not torch.allclose(P.rms_norm_one_plus_w(x, w, 1e-6), base * w)
+
+
+def test_norm_ignores_the_scale_of_its_input():
+    x = torch.randn(4, 32, dtype=torch.float64)
+    w = torch.randn(32, dtype=torch.float64) * 0.1
+    assert torch.allclose(P.rms_norm_one_plus_w(7.0 * x, w, 1e-12), P.rms_norm_one_plus_w(x, w, 1e-12), atol=1e-9)
+
+
+# ---- embedding ---------------------------------------------------------------------------
+def test_embedding_is_scaled_by_sqrt_hidden():
+    table = torch.randn(10, 64, dtype=torch.float64)
+    ids = torch.tensor([3, 3, 9])
+    assert torch.equal(P.embed(ids, table, 64), table[ids] * 8.0)           # sqrt(64) exactly
+    # the factor held in bfloat16: sqrt(2048) = 45.2548... becomes 45.25
+    t = torch.ones(1, 2048, dtype=torch.float32)
+    assert P.embed(torch.tensor([0]), t, 2048, torch.bfloat16)[0, 0].item() == 45.25
+    assert abs(P.embed(torch.tensor([0]), t, 2048)[0, 0].item() - math.sqrt(2048)) < 1e-5
+
+
+# ---- rotation ----------------------------------------------------------------------------------
+def test_rotation_at_position_zero_is_identity_and_norms_are_kept():
+    x = torch.randn(6, 3, 16, dtype=torch.float64)
+    cos, sin = P.rope_cos_sin(torch.zeros(6, dtype=torch.long), 16, 10000.0, torch.float64)
+    assert torch.allclose(P.apply_rope(x, cos, sin), x)
+    cos, sin = P.rope_cos_sin(torch.arange(6), 16, 10000.0, torch.float64)
+    y = P.apply_rope(x, cos, sin)
+    pair = lambda t: t[..., :8].pow(2) + t[..., 8:].pow(2)     # element j with j + d/2
+    assert torch.allclose(pair(y), pair(x))
+
+
+def test_rotation_pairs_halves_and_turns_counterclockwise():
+    # d = 4, position 1: pairs are (0, 2) and (1, 3); the first pair turns by 1 radian
+    x = torch.tensor([[[1.0, 0.0, 0.0, 0.0]]], dtype=torch.float64)
+    cos, sin = P.rope_cos_sin(torch.tensor([1]), 4, 10000.0, torch.float64)
+    y = P.apply_rope(x, cos, sin)[0, 0]
+    assert torch.allclose(y, torch.tensor([math.cos(1.0), 0.0, math.sin(1.0), 0.0], dtype=torch.float64))
+    # frequency of pair j is theta^(-2j/d)
+    x = torch.tensor([[[0.0, 1.0, 0.0, 0.0]]], dtype=torch.float64)
+    y = P.apply_rope(x, cos, sin)[0, 0]
+    a = 10000.0 ** (-2.0 / 4.0)
+    assert torch.allclose(y, torch.tensor([0.0, math.cos(a), 0.0, math.sin(a)], dtype=torch.float64))
+
+
+def test_rotated_dot_products_depend_on_distance_only():
+    q = torch.randn(1, 1, 32, dtype=torch.float64)
+    k = torch.randn(1, 1, 32, dtype=torch.float64)
+
+    def dot(m, n):
+        cq, sq = P.rope_cos_sin(torch.tensor([m]), 32, 500.0, torch.float64)
+        ck, sk = P.rope_cos_sin(torch.tensor([n]), 32, 500.0, torch.float64)
+        return (P.apply_rope(q, cq, sq) * P.apply_rope(k, ck, sk)).sum()
+
+    assert torch.allclose(dot(5, 2), dot(105, 102))
+    assert not torch.allclose(dot(5, 2), dot(2, 5))
+
+
+def test_rotation_vanishes_for_huge_theta():
+    x = torch.randn(4, 2, 8, dtype=torch.float64)
+    cos, sin = P.rope_cos_sin(torch.arange(4), 8, 1e300, torch.float64)
+    y = P.apply_rope(x, cos, sin)
+    # only the first pair (frequency 1) still turns
+    assert torch.allclose(y[..., 1:4], x[..., 1:4]) and torch.allclose(y[..., 5:], x[..., 5:])
+
+
+# ---- attention -----------------------------------------------------------------------------------
+def test_attention_equals_the_library_routine():
+    T, nh, d = 9, 4, 16
+    q, k, v = (torch.randn(T, nh, d, dtype=torch.float64) for _ in range(3))
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None], is_causal=True)[0].transpose(0, 1)
+    assert torch.allclose(P.causal_attention(q, k, v, d), ref)
+
+
+def test_attention_scale_is_head_dim_not_hidden_over_heads():
+    T, nh, d = 5, 2, 16
+    q, k, v = (torch.randn(T, nh, d, dtype=torch.float64) for _ in range(3))
+    scores = torch.einsum("qhd,khd->hqk", q, k) / math.sqrt(d)
+    probs = torch.softmax(scores.masked_fill(~torch.ones(T, T, dtype=torch.bool).tril(), float("-inf")), -1)
+    assert torch.allclose(P.causal_attention(q, k, v, d), torch.einsum("hqk,khd->qhd", probs, v))
+
+
+def test_attention_first_token_returns_its_value_and_equal_scores_give_the_mean():
+    T, d = 6, 8
+    q = torch.zeros(T, 1, d, dtype=torch.float64)
+    k, v = torch.randn(T, 1, d, dtype=torch.float64), torch.randn(T, 1, d, dtype=torch.float64)
+    o = P.causal_attention(q, k, v, d)
+    assert torch.allclose(o[0, 0], v[0, 0])
+    for t in range(T):
+        assert torch.allclose(o[t, 0], v[:t + 1, 0].mean(0))
+
+
+def test_grouped_heads_read_the_key_head_of_their_group():
+    # query head h uses kv head h // (nh // nkv): grouped attention equals full attention
+    # on key/value heads repeated in place
+    T, nh, nkv, d = 7, 6, 2, 8
+    q = torch.randn(T, nh, d, dtype=torch.float64)
+    k, v = torch.randn(T, nkv, d, dtype=torch.float64), torch.randn(T, nkv, d, dtype=torch.float64)
+    full = P.causal_attention(q, k.repeat_interleave(3, 1), v.repeat_interleave(3, 1), d)
+    assert torch.allclose(P.causal_attention(q, k, v, d), full)
+    wrong = P.causal_attention(q, k.repeat(1, 3, 1), v.repeat(1, 3, 1), d)      # interleaved the other way
+    assert not torch.allclose(P.causal_attention(q, k, v, d), wrong)
+
+
+# ---- feed-forward ----------------------------------------------------------------------------
+def test_gelu_is_the_tanh_approximation():
+    z = torch.linspace(-6, 6, 101, dtype=torch.float64)
+    assert torch.allclose(P.gelu_tanh(z), torch.nn.functional.gelu(z, approximate="tanh"))
+    assert not torch.allclose(P.gelu_tanh(z), torch.nn.functional.gelu(z), atol=1e-5)
+
+
+def test_feed_forward_gates_with_the_gate_projection():
+    h = torch.randn(3, 8, dtype=torch.float64)
+    wg, wu, wd = (torch.randn(*s, dtype=torch.float64) for s in ((12, 8), (12, 8), (8, 12)))
+    ref = (torch.nn.functional.gelu(h @ wg.T, approximate="tanh") * (h @ wu.T)) @ wd.T
+    assert torch.allclose(P.geglu_mlp(h, wg, wu, wd), ref)
+    assert torch.equal(P.geglu_mlp(h, torch.zeros_like(wg), wu, wd), torch.zeros(3, 8, dtype=torch.float64))
+
+
+# ---- the whole model -----------------------------------------------------------------------------
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_logits_do_not_change_when_all_positions_move(model_folders, name):
+    cfg = P.read_config(model_folders[name])
+    w = P.read_weights(model_folders[name], torch.float64)
+    ids = torch.randint(0, cfg["vocab_size"], (11,))
+    a = P.forward_logits(cfg, w, ids)
+    b = P.forward_logits(cfg, w, ids, positions=torch.arange(11) + 37)
+    assert torch.allclose(a, b, atol=1e-9)
+
+
+def test_logits_are_causal_and_the_head_is_the_unscaled_table(model_folders):
+    cfg = P.read_config(model_folders["A"])
+    w = P.read_weights(model_folders["A"], torch.float64)
+    ids = torch.randint(0, cfg["vocab_size"], (10,))
+    full = P.forward_logits(cfg, w, ids)
+    assert torch.allclose(P.forward_logits(cfg, w, ids[:6]), full[:6], atol=1e-10)
+    # doubling the table doubles the logits through the head but not through the (normalised) body
+    w2 = dict(w)
+    w2["model.embed_tokens.weight"] = w["model.embed_tokens.weight"] * 2
+    assert not torch.allclose(P.forward_logits(cfg, w2, ids), full, atol=1e-3)
+
+
+def test_head_dim_key_wins_over_the_derived_value(tmp_path):
+    # the reference's own vector: 3072 / 16 gives 192, the key says 256
+    # (tests/test_gemma_architecture.py:40-60)
+    import json
+    raw = dict(vocab_size=100, hidden_size=3072, intermediate_size=256, num_hidden_layers=1,
+               num_attention_heads=16, num_key_value_heads=16, head_dim=256)
+    (tmp_path / "config.json").write_text(json.dumps(raw))
+    assert P.read_config(str(tmp_path))["head_dim"] == 256
+    del raw["head_dim"]
+    (tmp_path / "config.json").write_text(json.dumps(raw))
+    assert P.read_config(str(tmp_path))["head_dim"] == 192
+
+
+def test_greedy_generation_recomputes_everything(model_folders):
+    cfg = P.read_config(model_folders["A"])
+    w = P.read_weights(model_folders["A"], torch.float32)
+    out = P.generate_greedy(cfg, w, [5, 9, 2], 4)
+    assert len(out) == 4
+    assert out[0] == int(P.forward_logits(cfg, w, [5, 9, 2])[-1].argmax())
+    assert out[1] == int(P.forward_logits(cfg, w, [5, 9, 2, out[0]])[-1].argmax())
+
+
+# ---- sampling --------------------------------------------------------------------------------
+def test_repetition_penalty_vector_of_the_reference():
+    # tests/test_sampling.py:49-55: [2, -2, 0.5], ids [0, 1], penalty 2 -> [1, -4, 0.5]
+    out = S.apply_repetition_penalty(torch.tensor([2.0, -2.0, 0.5]), [0, 1, 1], 2.0)
+    assert out.tolist() == [1.0, -4.0, 0.5]
+
+
+def test_greedy_and_top_k_one_are_argmax_and_logprob_is_log_softmax():
+    logits = torch.randn(100)
+    tok, lp, _, _ = S.sample_row(logits, 0.0, 0, 1.0, 0.0, 1.0, [], 0.99)
+    assert tok == int(logits.argmax())
+    assert abs(lp - float(torch.log_softmax(logits.double(), -1)[tok])) < 1e-12
+    for u in (0.0, 0.5, 0.999):
+        assert S.sample_row(logits, 1.0, 1, 1.0, 0.0, 1.0, [], u)[0] == int(logits.argmax())
+
+
+def test_top_p_keeps_the_top_token_even_if_it_alone_exceeds_p():
+    # tests/test_sampling.py:90-97
+    logits = torch.full((10,), -100.0)
+    logits[3] = 100.0
+    assert S.sample_row(logits, 1.0, 0, 0.1, 0.0, 1.0, [], 0.7)[0] == 3
+
+
+def test_truncations_on_a_known_distribution():
+    probs = torch.tensor([0.5, 0.25, 0.125, 0.0625, 0.0625])
+    scaled = probs.log().double()
+    assert S.keep_mask(scaled, 2, 1.0, 0.0).tolist() == [True, True, False, False, False]
+    # cumulative 0.5, 0.75, 0.875 ...: the token that crosses p is dropped
+    assert S.keep_mask(scaled, 0, 0.8, 0.0).tolist() == [True, True, False, False, False]
+    assert S.keep_mask(scaled, 0, 0.4, 0.0).tolist() == [True, False, False, False, False]
+    assert S.keep_mask(scaled, 0, 1.0, 0.2).tolist() == [True, True, True, False, False]
+
+
+def test_draw_inverts_the_cumulative_distribution():
+    logits = torch.tensor([0.5, 0.25, 0.125, 0.125]).log()
+    draws = [S.sample_row(logits, 1.0, 0, 1.0, 0.0, 1.0, [], u)[0] for u in (0.0, 0.49, 0.51, 0.74, 0.76, 0.9)]
+    assert draws == [0, 0, 1, 1, 2, 3]
+
+
+def test_philox_known_answers():
+    # Random123's known-answer vectors for philox4x32-10: all-zero and all-ones counter and key
+    assert abs(S.philox_uniform(0, 0) - (((0x6627e8d5 << 32) | 0xe169c58d) >> 11) / 2 ** 53) < 1e-18
+    us = [S.philox_uniform(7, c) for c in range(2000)]
+    assert 0.45 < sum(us) / len(us) < 0.55 and len(set(us)) == 2000

@@ -46,3 +46,251 @@ WLLM_API int wllm_argmax_rows(const float* logits, int* out, int rows, int vocab
     argmax_rows_kernel<<<rows, 256, 0, stream>>>(logits, out, vocab);
     return launch_status();
 }
+
+// ---- sampling with temperature, top-k, top-p, min-p and repetition penalty -----------------------
+// One workgroup of 1024 threads per row.  The steps follow the reference's sampler in its order
+// (src/wllm/engine/sampling.py:101-143): repetition penalty on the ids already generated
+// (positive logits divided, negative multiplied, :45-58), temperature (:122-123), the three
+// truncations on the full temperature-scaled distribution (:61-98: rank < k; cumulative
+// probability in descending order <= p, the top token always kept; probability >= min_p times
+// the top probability), a draw from what is left, and the log-probability of the drawn token
+// before truncation (:125-130,142).  Two things differ by design.  The draw is the inverse of
+// the cumulative distribution, in index order, at one uniform number from a counter-based
+// generator keyed by (seed, counter), so a row's token does not depend on the other rows of the
+// batch.  And all sums that decide a threshold or the draw are made in 40-bit fixed point with
+// integer additions, so they do not depend on the order of the additions: the same row gives
+// the same token on every run.  Equal logits are kept or dropped together.
+constexpr int kSampleThreads = 1024;
+constexpr double kFixedOne = 1099511627776.0;   // 2^40
+
+__device__ __forceinline__ uint32_t sortable_key(float v) {
+    const uint32_t u = __float_as_uint(v);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+__device__ __forceinline__ void philox4x32_10(uint32_t ctr[4], uint32_t key0, uint32_t key1) {
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        const uint32_t hi0 = __umulhi(0xD2511F53u, ctr[0]), lo0 = 0xD2511F53u * ctr[0];
+        const uint32_t hi1 = __umulhi(0xCD9E8D57u, ctr[2]), lo1 = 0xCD9E8D57u * ctr[2];
+        const uint32_t c0 = hi1 ^ ctr[1] ^ key0, c2 = hi0 ^ ctr[3] ^ key1;
+        ctr[0] = c0;
+        ctr[1] = lo1;
+        ctr[2] = c2;
+        ctr[3] = lo0;
+        key0 += 0x9E3779B9u;
+        key1 += 0xBB67AE85u;
+    }
+}
+
+// Walks the radix tree of the keys, most significant byte first, to the key at which the
+// running total (of counts, or of fixed-point mass), taken over keys in descending order,
+// first goes beyond `target` (counts: reaches it).  Returns false if it never does.
+template <bool MASS>
+__device__ bool radix_descend(const float* __restrict__ row, int vocab, float row_max, float inv_t,
+                              unsigned long long target, unsigned long long* hist, uint32_t* shared_sel,
+                              uint32_t* result_key) {
+    uint32_t prefix = 0, prefix_mask = 0;
+    unsigned long long above = 0;
+    for (int level = 0; level < 4; ++level) {
+        const int shift = 24 - 8 * level;
+        for (int b = threadIdx.x; b < 256; b += blockDim.x) hist[b] = 0ull;
+        __syncthreads();
+        for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+            const float v = row[i];
+            const uint32_t key = sortable_key(v);
+            if ((key & prefix_mask) == prefix) {
+                unsigned long long w = 1ull;
+                if (MASS) w = static_cast<unsigned long long>(static_cast<double>(expf((v - row_max) * inv_t)) * kFixedOne);
+                atomicAdd(&hist[(key >> shift) & 255u], w);
+            }
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            unsigned long long cum = above;
+            int sel = -1;
+            for (int b = 255; b >= 0; --b) {
+                const unsigned long long next = cum + hist[b];
+                if (MASS ? next > target : next >= target) {
+                    sel = b;
+                    break;
+                }
+                cum = next;
+            }
+            shared_sel[0] = static_cast<uint32_t>(sel);
+            reinterpret_cast<unsigned long long*>(shared_sel + 2)[0] = cum;
+        }
+        __syncthreads();
+        const int sel = static_cast<int>(shared_sel[0]);
+        above = reinterpret_cast<unsigned long long*>(shared_sel + 2)[0];
+        __syncthreads();
+        if (sel < 0) return false;
+        prefix |= static_cast<uint32_t>(sel) << shift;
+        prefix_mask |= 255u << shift;
+    }
+    *result_key = prefix;
+    return true;
+}
+
+__global__ void __launch_bounds__(kSampleThreads)
+sample_rows_kernel(float* __restrict__ logits, const float* __restrict__ params, const long long* __restrict__ seeds,
+                   const int* __restrict__ penalty_ids, const int* __restrict__ penalty_offsets,
+                   int* __restrict__ out_tokens, float* __restrict__ out_logprobs, int vocab) {
+    __shared__ unsigned long long hist[256];
+    __shared__ unsigned long long scan[kSampleThreads / kWave];
+    __shared__ float red_v[kSampleThreads / kWave];
+    __shared__ int red_i[kSampleThreads / kWave];
+    __shared__ __align__(8) uint32_t sel_s[4];
+    __shared__ int found_s;
+    const int r = blockIdx.x, tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    constexpr int kWavesHere = kSampleThreads / kWave;
+    float* row = logits + static_cast<size_t>(r) * vocab;
+    const float temperature = params[r * 5 + 0];
+    const int top_k = static_cast<int>(params[r * 5 + 1]);
+    const float top_p = params[r * 5 + 2], min_p = params[r * 5 + 3], penalty = params[r * 5 + 4];
+
+    // repetition penalty, in place; the ids of a row are distinct
+    if (penalty_ids && penalty != 1.0f) {
+        for (int j = penalty_offsets[r] + tid; j < penalty_offsets[r + 1]; j += blockDim.x) {
+            const int id = penalty_ids[j];
+            if (id >= 0 && id < vocab) {
+                const float v = row[id];
+                row[id] = v > 0.f ? v / penalty : v * penalty;
+            }
+        }
+        __syncthreads();
+    }
+
+    // maximum and its lowest index
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = tid; i < vocab; i += blockDim.x) {
+        const float v = row[i];
+        if (v > bv || bi == 0x7fffffff) {
+            bv = v == v ? v : -INFINITY;
+            bi = i;
+        }
+    }
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, kWave);
+        const int oi = __shfl_xor(bi, off, kWave);
+        if (ov > bv || (ov == bv && oi < bi)) {
+            bv = ov;
+            bi = oi;
+        }
+    }
+    if (lane == 0) {
+        red_v[wave] = bv;
+        red_i[wave] = bi;
+    }
+    __syncthreads();
+    bv = red_v[0];
+    bi = red_i[0];
+    for (int w = 1; w < kWavesHere; ++w)
+        if (red_v[w] > bv || (red_v[w] == bv && red_i[w] < bi)) {
+            bv = red_v[w];
+            bi = red_i[w];
+        }
+    __syncthreads();
+    const float row_max = bv;
+    const int arg_max = bi == 0x7fffffff ? 0 : bi;
+    const bool greedy = temperature == 0.0f;
+    const float inv_t = greedy ? 1.0f : 1.0f / fmaxf(temperature, 1e-5f);
+
+    // normaliser of the whole (scaled) distribution, in fixed point
+    unsigned long long part = 0;
+    for (int i = tid; i < vocab; i += blockDim.x)
+        part += static_cast<unsigned long long>(static_cast<double>(expf((row[i] - row_max) * inv_t)) * kFixedOne);
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) part += __shfl_xor(part, off, kWave);
+    if (lane == 0) scan[wave] = part;
+    __syncthreads();
+    unsigned long long z_fixed = 0;
+    for (int w = 0; w < kWavesHere; ++w) z_fixed += scan[w];
+    __syncthreads();
+    const float log_z = static_cast<float>(log(static_cast<double>(z_fixed) / kFixedOne));
+
+    if (greedy) {
+        if (tid == 0) {
+            out_tokens[r] = arg_max;
+            out_logprobs[r] = -log_z;      // (max - max) * 1 - log Z
+        }
+        return;
+    }
+
+    // thresholds of the truncations, as keys
+    const uint32_t max_key = sortable_key(row_max);
+    uint32_t k_key = 0;          // keep key >= k_key
+    uint32_t p_key = 0;          // keep key >  p_key
+    bool k_on = top_k > 0 && top_k < vocab, p_on = top_p < 1.0f;
+    if (k_on) k_on = radix_descend<false>(row, vocab, row_max, inv_t, static_cast<unsigned long long>(top_k), hist, sel_s, &k_key);
+    if (p_on) {
+        const unsigned long long target = static_cast<unsigned long long>(static_cast<double>(top_p) * static_cast<double>(z_fixed));
+        p_on = radix_descend<true>(row, vocab, row_max, inv_t, target, hist, sel_s, &p_key);
+    }
+    const bool mp_on = min_p > 0.0f;
+
+    // mass kept, per thread over a contiguous range of indices, then the draw
+    const int chunk = (vocab + kSampleThreads - 1) / kSampleThreads;
+    const int begin = min(vocab, tid * chunk), end = min(vocab, begin + chunk);
+    auto kept_mass = [&](int i) -> unsigned long long {
+        const float v = row[i];
+        const uint32_t key = sortable_key(v);
+        const float e = expf((v - row_max) * inv_t);
+        const bool keep = key == max_key || ((!k_on || key >= k_key) && (!p_on || key > p_key) && (!mp_on || e >= min_p));
+        return keep ? static_cast<unsigned long long>(static_cast<double>(e) * kFixedOne) : 0ull;
+    };
+    unsigned long long mine = 0;
+    for (int i = begin; i < end; ++i) mine += kept_mass(i);
+    // exclusive scan over the threads
+    unsigned long long incl = mine;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const unsigned long long o = __shfl_up(incl, off, kWave);
+        if (lane >= off) incl += o;
+    }
+    if (lane == kWave - 1) scan[wave] = incl;
+    __syncthreads();
+    unsigned long long wave_base = 0, total = 0;
+    for (int w = 0; w < kWavesHere; ++w) {
+        if (w < wave) wave_base += scan[w];
+        total += scan[w];
+    }
+    const unsigned long long excl = wave_base + incl - mine;
+
+    uint32_t ctr[4] = {static_cast<uint32_t>(seeds[r * 2 + 1]), static_cast<uint32_t>(seeds[r * 2 + 1] >> 32), 0u, 0u};
+    philox4x32_10(ctr, static_cast<uint32_t>(seeds[r * 2]), static_cast<uint32_t>(seeds[r * 2] >> 32));
+    const double u = static_cast<double>(((static_cast<unsigned long long>(ctr[0]) << 32) | ctr[1]) >> 11) * (1.0 / 9007199254740992.0);
+    unsigned long long target = static_cast<unsigned long long>(u * static_cast<double>(total));
+    if (target >= total) target = total - 1;
+    if (tid == 0) found_s = -1;
+    __syncthreads();
+    if (mine > 0 && target >= excl && target < excl + mine) {
+        unsigned long long cum = excl;
+        int tok = begin;
+        for (int i = begin; i < end; ++i) {
+            const unsigned long long w = kept_mass(i);
+            if (w > 0 && target < cum + w) {
+                tok = i;
+                break;
+            }
+            cum += w;
+        }
+        found_s = tok;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        const int tok = found_s >= 0 ? found_s : arg_max;
+        out_tokens[r] = tok;
+        out_logprobs[r] = (row[tok] - row_max) * inv_t - log_z;
+    }
+}
+
+WLLM_API int wllm_sample_rows(float* logits, const float* params, const long long* seeds, const int* penalty_ids,
+                              const int* penalty_offsets, int* out_tokens, float* out_logprobs, int rows, int vocab,
+                              hipStream_t stream) {
+    sample_rows_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, params, seeds, penalty_ids, penalty_offsets,
+                                                            out_tokens, out_logprobs, vocab);
+    return launch_status();
+}

@@ -46,6 +46,21 @@ class ModelRunner:
     def step(self, entries: list) -> torch.Tensor:
         """Returns float32 logits [wanted, vocab] in the order of the entries and of
         each entry's `want`.  The tensor is a view of a buffer the next step reuses."""
+        ctx = self.prepare(entries)
+        logits = self.model.forward(ctx)
+        self.commit(entries)
+        return logits
+
+    def commit(self, entries: list) -> None:
+        """Moves the requests' lengths after all layers wrote."""
+        for e in entries:
+            self.cache.commit(e.request, len(e.tokens))
+        self.steps_run += 1
+        self.tokens_run += sum(len(e.tokens) for e in entries)
+
+    def prepare(self, entries: list) -> StepContext:
+        """Checks the entries, takes room for them in the cache (all or none) and builds
+        the step's index tensors."""
         cache = self.cache
         max_pos = self.model.plan.max_positions
         seen = set()
@@ -111,9 +126,4 @@ class ModelRunner:
             group_slots=dev[8:8 + num_groups], group_block_tables=dev[8 + num_groups:8 + 2 * num_groups],
             host_q_start=q_start, host_q_len=q_len, host_ctx_len=ctx_len, host_state_slots=state_slots,
             requests=[e.request for e in entries])
-        logits = self.model.forward(ctx)
-        for e in entries:
-            cache.commit(e.request, len(e.tokens))
-        self.steps_run += 1
-        self.tokens_run += n
-        return logits
+        return ctx

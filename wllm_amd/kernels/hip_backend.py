@@ -30,6 +30,7 @@ _SIGNATURES = {
                                      c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
     "wllm_gemm_generic": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_argmax_rows": [c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "wllm_sample_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
 
 
@@ -107,3 +108,9 @@ class HipBackend:
         self._on_gpu(logits, out)
         self._check(self.lib.wllm_argmax_rows(_ptr(logits), _ptr(out), logits.shape[0], logits.shape[1],
                                               self._stream()), "argmax_rows")
+
+    def sample_rows(self, logits, params, seeds, penalty_ids, penalty_offsets, out_tokens, out_logprobs):
+        self._on_gpu(logits, params, seeds, penalty_ids, penalty_offsets, out_tokens, out_logprobs)
+        self._check(self.lib.wllm_sample_rows(
+            _ptr(logits), _ptr(params), _ptr(seeds), _ptr(penalty_ids), _ptr(penalty_offsets), _ptr(out_tokens),
+            _ptr(out_logprobs), logits.shape[0], logits.shape[1], self._stream()), "sample_rows")
