@@ -1,0 +1,212 @@
+"""Decode and prefill throughput of the engine at the Gemma-2B layer sizes, on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+A step is one decode step of the engine: the scheduler's step over a batch of running
+requests (model step from the paged cache, sampling, bookkeeping), measured as the
+reference measures decode (scripts/benchmark_decode.py:59-75): warm-up steps, then K timed
+steps between device synchronisations, tokens/s = K * batch / elapsed.  Weights are random
+(seeded normal, std 0.02), prompts are seeded uniform token ids; no dataset and no checkpoint
+is used.  One JSON line is printed.  For more than one GPU the program says that it runs
+on one and exits with 2.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# MI355X's published peaks: HBM3E bandwidth and dense matrix rates per dtype
+PEAK_HBM_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}
+
+
+def build_model(shape: dict, dtype: str, seed: int):
+    import torch
+
+    from wllm_amd.parts import build_model as build
+    from wllm_amd.weights.random_init import RandomFetcher
+    model = build(shape)
+    tdt = {"bf16": torch.bfloat16, "fp32": torch.float32}[dtype]
+    model.load_from(RandomFetcher(model.expected_tensors(), seed, tdt, "cuda:0", std=0.02, norm_std=0.1))
+    return model
+
+
+def step_flops(model, tokens: int, context_before: int, logit_rows: int) -> float:
+    """Floating-point operations of one step over `tokens` new tokens of one request."""
+    flops = 0.0
+    for e in model.plan.schedule:
+        spec = model.plan.layers[e.layer]
+        m, f = spec.mixer, spec.feed_forward
+        qkv = (m.num_heads + 2 * m.num_kv_heads) * m.head_dim
+        flops += 2.0 * tokens * m.hidden_size * (qkv + m.num_heads * m.head_dim)
+        flops += 2.0 * tokens * f.hidden_size * f.intermediate_size * 3
+        # scores and weighted sums over the keys each query sees (causal)
+        keys = tokens * context_before + tokens * (tokens + 1) / 2.0
+        flops += 4.0 * m.num_heads * m.head_dim * keys
+    flops += 2.0 * logit_rows * model.plan.head.hidden_size * model.plan.head.vocab_size
+    return flops
+
+
+def kv_bytes_per_token(model) -> int:
+    total = 0
+    for i, need in model.cache_needs().items():
+        total += 2 * need.num_kv_heads * need.head_dim * (2 if model.dtype.itemsize == 2 else 4)
+    return total
+
+
+def measure_prefill(model, tokens: int, block_size: int, repeats: int = 3):
+    import torch
+
+    from wllm_amd.engine import ModelRunner, StepEntry
+    pages = -(-tokens // block_size) + 1
+    runner = ModelRunner.create(model, num_pages=pages, page_size=block_size, max_requests=2)
+    g = torch.Generator().manual_seed(1)
+    ids = torch.randint(0, model.plan.embedding.vocab_size, (tokens,), generator=g).tolist()
+    best = None
+    for i in range(repeats + 1):
+        runner.open("p")
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        runner.step([StepEntry("p", ids, [tokens - 1])])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        runner.close("p")
+        if i > 0:
+            best = dt if best is None else min(best, dt)
+    del runner
+    torch.cuda.empty_cache()
+    return best
+
+
+def measure_decode(model, batch: int, context: int, steps: int, warmup: int, block_size: int, hip_graphs: bool,
+                   chunk: int = 2048):
+    """Returns (seconds for `steps` steps, mean context length during them)."""
+    import torch
+
+    from wllm_amd.engine import ModelRunner, Request, Scheduler
+    total_new = warmup + steps + 1
+    pages = batch * (-(-(context + total_new) // block_size))
+    runner = ModelRunner.create(model, num_pages=pages, page_size=block_size, max_requests=batch)
+    if hip_graphs and hasattr(runner, "enable_graphs"):
+        runner.enable_graphs()
+    sched = Scheduler(runner, max_prefill_tokens_per_step=chunk, compute_logprobs=False)
+    g = torch.Generator().manual_seed(2)
+    vocab = model.plan.embedding.vocab_size
+    for i in range(batch):
+        sched.add_request(Request(i, torch.randint(0, vocab, (context,), generator=g).tolist(), total_new))
+    while sched.waiting or any(r.status.value != "running" for r in sched.running):
+        sched.step()
+    for _ in range(warmup):
+        sched.step()
+    assert len(sched.running) == batch and all(r.status.value == "running" for r in sched.running)
+    first_len = sched.running[0].num_computed
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        sched.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    mean_ctx = first_len + (steps + 1) / 2.0
+    del sched, runner
+    torch.cuda.empty_cache()
+    return dt, mean_ctx
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=2048, help="prompt length of every request")
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--shape", default="gemma-2b", help="a named layer shape or a config.json")
+    ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the shape has")
+    ap.add_argument("--block-size", type=int, default=16)
+    ap.add_argument("--no-graphs", action="store_true", help="do not replay captured graphs for decode")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args()
+    world = int(os.environ.get("WORLD_SIZE", "1"))
+    if args.gpus != 1 or world != 1:
+        if int(os.environ.get("RANK", "0")) == 0:
+            print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} (world size {world}) is not supported")
+        return 2
+
+    import torch
+
+    import wllm_amd  # noqa: F401
+    from wllm_amd.cli import read_shape
+    from wllm_amd.kernels import ops
+
+    ops.backend()
+    shape = read_shape(args.shape)
+    full_layers = shape["num_hidden_layers"]
+    if args.layers is not None:
+        shape["num_hidden_layers"] = args.layers
+    with torch.inference_mode():
+        model = build_model(shape, args.dtype, args.seed)
+        graphs = not args.no_graphs
+        weight_bytes = model.weight_bytes()
+        kv_per_token = kv_bytes_per_token(model)
+
+        t_prefill = measure_prefill(model, args.prefill_tokens, args.block_size)
+        prefill_flops = step_flops(model, args.prefill_tokens, 0, 1)
+
+        dt, mean_ctx = measure_decode(model, args.batch, args.context, args.steps, args.warmup, args.block_size, graphs)
+        ms_per_step = 1000.0 * dt / args.steps
+        value = args.steps * args.batch / dt
+        step_bytes = weight_bytes + args.batch * mean_ctx * kv_per_token
+        achieved = step_bytes / (dt / args.steps) / 1e9
+
+        points = {}
+        if not args.no_points:
+            for b, k in ((1, args.steps), (64, max(8, args.steps // 2))):
+                d, _ = measure_decode(model, b, args.context, k, min(args.warmup, 4), args.block_size, graphs)
+                points[f"decode_b{b}"] = round(k * b / d, 1)
+
+    c = model.config
+    line = {
+        "metric": "decode tokens/s, Gemma-2B layer sizes, after 2,048-token prompts",
+        "value": round(value, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": args.dtype,
+        "data": "synthetic: seeded random weights (normal, std 0.02) and seeded uniform token ids",
+        "config": {
+            "model": "Gemma-2B layer sizes (GemmaForCausalLM), random weights",
+            "global_batch": args.batch, "seq_len": args.context, "parallelism": "single GPU",
+            "layers": c.num_hidden_layers, "layers_of_full_model": full_layers, "hidden_size": c.hidden_size,
+            "intermediate_size": c.intermediate_size, "num_attention_heads": c.num_attention_heads,
+            "num_key_value_heads": c.num_key_value_heads, "head_dim": c.head_dim, "vocab_size": c.vocab_size,
+            "tied_embeddings": c.tie_word_embeddings, "rope_theta": c.rope_theta, "rms_norm_eps": c.rms_norm_eps,
+            "max_position_embeddings": c.max_position_embeddings, "kv_block_size": args.block_size,
+            "sampling": "greedy", "hip_graphs": graphs,
+        },
+        "prefill": {"value": round(args.prefill_tokens / t_prefill, 1), "tokens": args.prefill_tokens,
+                    "ms": round(1000.0 * t_prefill, 3),
+                    "frac": round(prefill_flops / t_prefill / PEAK_FLOPS[args.dtype], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+        "points": points,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

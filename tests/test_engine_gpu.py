@@ -17,7 +17,7 @@ FAMILIES = {"whole": trace_whole, "tail": trace_tail, "portions": trace_portions
 # float32: the engine and the oracle differ by the order of float32 sums only.
 # bfloat16: activations between kernels are rounded to 8 bits of mantissa; logits of
 # these models are O(0.1..1), and errors of a few 1e-3 per rounding pile up over the layers.
-TOLERANCE = {"float32": dict(atol=2e-5, rtol=1e-4), "bfloat16": dict(atol=3e-2, rtol=3e-2)}
+TOLERANCE = {"float32": dict(atol=2e-5, rtol=1e-4), "bfloat16": dict(atol=1e-2, rtol=1e-2)}
 
 
 def _requests(name):

@@ -94,6 +94,10 @@ class HipBackend:
 
     def linear(self, x, weight, out):
         self._on_gpu(x, weight, out)
+        if x.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and x.shape[0] > 64:
+            # many rows, bfloat16: the library's matrix-core product (float32 accumulation)
+            torch.mm(x, weight.t(), out=out)
+            return
         self._check(self.lib.wllm_gemm_generic(
             _ptr(x), _ptr(weight), int(x.dtype == torch.bfloat16), _ptr(out), int(out.dtype == torch.bfloat16),
             x.shape[0], weight.shape[0], x.shape[1], self._stream()), "linear")

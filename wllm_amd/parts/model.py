@@ -94,13 +94,20 @@ class CausalLM:
             extra = (tied_head_name,)
         checkpoint.check(self.expected_tensors(), self.plan.ignored_tensor_suffixes, allowed_extra=extra)
         fetch = TensorFetcher(checkpoint, dtype, device)
-        table = fetch.matrix(emb.weight)
         if extra:
+            table = fetch.matrix(emb.weight)
             if checkpoint.shape(tied_head_name) != tuple(table.shape) or not torch.equal(
                     fetch.matrix(tied_head_name), table):
                 raise WeightError(f"{tied_head_name} is stored although the embeddings are tied, and differs from "
                                   f"{emb.weight}", unexpected=[tied_head_name])
-        self.embed_table = fetch.to_device(table)
+        self.load_from(fetch)
+
+    def load_from(self, fetch) -> None:
+        """Loads every part through a fetcher: an object with `matrix(name)`, `vector(name)`,
+        `table(name)`, `to_device(tensor)`, `has(name)` and the attributes `dtype`, `device`."""
+        emb, head = self.plan.embedding, self.plan.head
+        dtype, device = fetch.dtype, fetch.device
+        self.embed_table = fetch.to_device(fetch.matrix(emb.weight))
         for block in self.blocks:
             for part in block.parts():
                 part.load(fetch)

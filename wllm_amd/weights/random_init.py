@@ -51,3 +51,36 @@ def write_random_model(folder: str, config_json: dict, expected: dict, seed: int
     with open(os.path.join(folder, "config.json"), "w", encoding="utf-8") as f:
         json.dump(config_json, f, indent=1, sort_keys=True)
     return folder
+
+
+class RandomFetcher:
+    """Random weights made on the device, for measurements at sizes whose folder would be
+    many gigabytes: the same distributions as `write_random_model`, drawn by the device's
+    generator (so not the same numbers as a written folder of that seed)."""
+
+    def __init__(self, expected: dict, seed: int, dtype: torch.dtype, device, std: float = 0.02,
+                 norm_std: float = 0.1):
+        self.expected, self.dtype, self.device = expected, dtype, torch.device(device)
+        self.std, self.norm_std = std, norm_std
+        self._gen = torch.Generator(device=self.device)
+        self._seed = seed
+
+    def has(self, name: str) -> bool:
+        return name in self.expected and not self.expected[name].optional
+
+    def _draw(self, name: str, dtype: torch.dtype) -> torch.Tensor:
+        exp = self.expected[name]
+        digest = hashlib.sha256(f"{self._seed}:{name}".encode("utf-8")).digest()
+        self._gen.manual_seed(int.from_bytes(digest[:8], "little") & 0x7FFF_FFFF_FFFF_FFFF)
+        t = torch.empty(tuple(exp.shape), dtype=torch.bfloat16, device=self.device)
+        t.normal_(0.0, self.norm_std if exp.init == "norm" else self.std, generator=self._gen)
+        return t.to(dtype)
+
+    def matrix(self, name: str) -> torch.Tensor:
+        return self._draw(name, self.dtype)
+
+    def vector(self, name: str) -> torch.Tensor:
+        return self._draw(name, torch.float32)
+
+    def to_device(self, t: torch.Tensor) -> torch.Tensor:
+        return t.contiguous().to(self.device)
