@@ -74,7 +74,8 @@ class EmulatedKernels:
             vview[page, :, :, off] = val
 
     def paged_attention(self, qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len, out,
-                        num_heads, num_kv_heads, head_dim, page_size, scale, window, max_q_len, max_ctx_len):
+                        num_heads, num_kv_heads, head_dim, page_size, scale, window, max_q_len, max_ctx_len,
+                        plan=None):
         self._count("paged_attention")
         n = qkv.shape[0]
         n_rep = num_heads // num_kv_heads
@@ -105,6 +106,9 @@ class EmulatedKernels:
             v = torch.where(torch.isnan(v), torch.zeros_like(v), v) if window else v
             o = torch.einsum("hqk,khd->qhd", probs, v)
             out[q0:q0 + ql] = o.reshape(ql, num_heads * head_dim).to(out.dtype)
+
+    def plan_paged_attention(self, *args):
+        return None
 
     def linear(self, x, weight, out):
         self._count("linear")

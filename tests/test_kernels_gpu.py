@@ -158,11 +158,60 @@ ATTENTION_SHAPES = [
 ]
 
 
+def _with_plan(args, kwargs):
+    """Adds the work-item plan the engine would make for these segments (None where the generic kernel runs)."""
+    kwargs = dict(kwargs)
+    kwargs["plan"] = ops.plan_paged_attention(
+        args[5].cpu().numpy(), args[6].cpu().numpy(), num_heads=kwargs["num_heads"], num_kv_heads=kwargs["num_kv_heads"],
+        head_dim=kwargs["head_dim"], page_size=kwargs["page_size"], window=kwargs["window"], dtype=args[0].dtype,
+        device=args[0].device)
+    return kwargs
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nh,nkv,d,ps,segs,window", ATTENTION_SHAPES)
 def test_paged_attention(dtype, nh, nkv, d, ps, segs, window):
     g, r = both("paged_attention", lambda: _attention_case(dtype, nh, nkv, d, ps, segs, window), dtype)
     close(g[7], r[7], dtype, "attention output")
+
+
+MFMA_SHAPES = ATTENTION_SHAPES + [
+    (8, 1, 256, 16, [(1, 2048), (1, 700), (1, 257), (1, 256), (1, 255)], 0),      # decoded tokens, keys split over workgroups
+    (8, 1, 256, 16, [(2048, 2048)], 0),                                           # a whole prompt
+    (16, 16, 256, 16, [(1, 513), (70, 300)], 0),                                   # no grouping
+    (6, 2, 96, 4, [(5, 5), (1, 300), (17, 64), (2, 40)], 0),                       # pages of 4: 8-byte value loads
+    (8, 2, 64, 8, [(1, 600), (3, 100), (50, 50)], 33),                             # window
+    (8, 2, 64, 16, [(1, 1000), (40, 500)], 300),                                   # window over several key chunks
+    (10, 5, 160, 32, [(1, 90), (33, 33)], 0),
+    (3, 1, 224, 16, [(1, 400), (6, 6), (7, 20)], 0),                               # group of 3: rows straddle tokens
+]
+
+
+@pytest.mark.parametrize("nh,nkv,d,ps,segs,window", MFMA_SHAPES)
+def test_paged_attention_matrix_cores(nh, nkv, d, ps, segs, window):
+    """The bfloat16 kernel the engine uses for these sizes (with its plan of work items)."""
+    dtype = torch.bfloat16
+    args, kwargs = _attention_case(dtype, nh, nkv, d, ps, segs, window, seed=11)
+    ref_args = [a.clone() for a in args]
+    kw = _with_plan(args, kwargs)
+    expect_plan = d % 32 == 0 and ps % 4 == 0
+    assert (kw["plan"] is not None) == expect_plan
+    # stale slots beyond a request's length hold NaN: they must not leak into the result
+    cache, bt, ctx = args[1], args[2], args[6]
+    kview = cache[:, 0].view(cache.shape[0], nkv, ps, d)
+    vview = cache[:, 1].view(cache.shape[0], nkv, d, ps)
+    for s_, (_, c) in enumerate(segs):
+        if c % ps:
+            last = int(bt[s_, (c - 1) // ps])
+            kview[last, :, c % ps:, :] = float("nan")
+            vview[last, :, :, c % ps:] = float("nan")
+    ref_args[1] = cache.clone()
+    ops.paged_attention(*args, **kw)
+    torch.cuda.synchronize()
+    with ops.use_backend(EmulatedKernels(precise=True)):
+        ops.paged_attention(*ref_args, **kwargs)
+    assert torch.isfinite(args[7].float()).all()
+    close(args[7], ref_args[7], dtype, "attention output")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -1,0 +1,338 @@
+// Paged attention on the matrix cores for bfloat16: head sizes 32..256 in steps of 32, pages
+// of a multiple of 4 tokens, any number of heads and groups, optional window.  One kernel serves
+// prompt portions and decoded tokens.
+//
+// Rows.  For one request (segment) and one key/value head, the query rows are the pairs (token,
+// query head of the group): row r = token * G + head.  All rows of a tile read the same keys and
+// values, so under multi-query attention the G heads of a token share one pass over the cache
+// (the reference's kernel runs one workgroup per query head and reads the cache G times,
+// src/wllm/kernels/csrc/paged_attention.cu:44-45,185).
+//
+// Work items.  The host cuts every (segment, key/value head) into work items, one workgroup of 4
+// wavefronts each: up to 4 tiles of 16 rows, and a range of keys.  With 4 row tiles each
+// wavefront owns a tile and walks all keys; with fewer, the spare wavefronts split the keys and
+// are merged through shared memory.  Segments of at most 16 rows (decoded tokens) are also split
+// over workgroups in fixed chunks of keys; those write partial results (running maximum, sum,
+// unnormalised accumulator) that `attention_reduce_kernel` combines.  Chunk boundaries depend
+// on the key index only, never on the batch.
+//
+// Matrix products (v_mfma_f32_16x16x32_bf16, 64 lanes: i = lane % 16, g = lane / 16):
+//   scores^T[key, row] = K[key, :] . Q[row, :]     A = K: lane (i, g) holds K[key_i][32c + 8g ..+8]
+//                                                  B = Q: lane (i, g) holds Q[row_i][32c + 8g ..+8]
+//                                                  C: lane (i, g) holds rows (keys) 4g..4g+3, column row_i
+//   out^T[d, row] = V^T[d, keys] . P^T[keys, row]  A = V^T: lane (i, g) holds V^T[16t + i][8 keys of g]
+//                                                  B = P^T: the lane's own 8 probabilities of row_i
+// so every value a lane holds belongs to one query row, softmax needs two shuffles per tile, and the
+// probabilities feed the second product from the registers they were computed in.  Keys are read as
+// [page_size, head_dim] rows, values transposed as [head_dim, page_size] rows (16-byte loads when the
+// page size is a multiple of 8).  Scores, maxima, sums and accumulators are float32.
+#include "common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kItemInts = 8;
+constexpr int kRowsPerTile = 16;
+constexpr int kKeysPerBlock = 32;
+
+union Pack16 {
+    uint4 u;
+    bf16x8_t v;
+    uint2 half[2];
+    uint16_t s[8];
+};
+
+__device__ __forceinline__ uint16_t bf16_bits(float f) { return from_float<bf16>(f).bits; }
+
+template <int HD, bool V16>
+__global__ void __launch_bounds__(256)
+paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict__ cache,
+                            const int* __restrict__ block_tables, const int* __restrict__ items,
+                            const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
+                            const int* __restrict__ seg_ctx_len, bf16* __restrict__ out,
+                            float* __restrict__ partial_o, float* __restrict__ partial_ml, int num_heads,
+                            int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window) {
+    constexpr int DC = HD / 32;   // 32-wide chunks of the head for the score product
+    constexpr int DT = HD / 16;   // 16-row tiles of out^T
+    // merge buffer: two slots of [16 rows][HD + 2] floats
+    __shared__ float merge_s[2][kRowsPerTile * (HD + 2)];
+
+    const int* item = items + static_cast<size_t>(blockIdx.x) * kItemInts;
+    const int seg = item[0], kvh = item[1], row_begin = item[2], row_tiles = item[3];
+    const int key_begin = item[4], key_end = item[5], partial_slot = item[6];
+    if (seg < 0) return;    // padding item
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int i = lane % 16, g = lane / 16;
+    const int key_splits = 4 / row_tiles;           // wavefronts that share a row tile
+    const int rt = wave % row_tiles, ks = wave / row_tiles;
+
+    const int group = num_heads / num_kv_heads;
+    const int q_start = seg_q_start[seg], q_len = seg_q_len[seg], ctx = seg_ctx_len[seg];
+    const int total_rows = q_len * group;
+    const int first_pos = ctx - q_len;
+    const int seg_lo = window > 0 ? max(0, first_pos - window + 1) : 0;   // keys below may be given back
+    const int r0 = row_begin + rt * kRowsPerTile;
+    const bool tile_active = r0 < total_rows;
+    const int row = r0 + i;
+    const bool row_valid = row < total_rows;
+    const int tok = row_valid ? row / group : 0;
+    const int head = kvh * group + (row_valid ? row % group : 0);
+    const int pos = first_pos + tok;
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+
+    const int width = (num_heads + 2 * num_kv_heads) * HD;
+    const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * HD;
+    const size_t k_off = static_cast<size_t>(kvh) * page_size * HD;
+    const size_t v_off = (static_cast<size_t>(num_kv_heads) + kvh) * page_size * HD;
+    const int* table = block_tables + static_cast<size_t>(seg) * max_pages;
+
+    // the queries of this lane's row
+    bf16x8_t qreg[DC];
+    {
+        const bf16* qrow = qkv + static_cast<size_t>(q_start + tok) * width + static_cast<size_t>(head) * HD;
+#pragma unroll
+        for (int c = 0; c < DC; ++c) {
+            Pack16 p;
+            p.u = row_valid ? *reinterpret_cast<const uint4*>(qrow + c * 32 + 8 * g) : make_uint4(0, 0, 0, 0);
+            qreg[c] = p.v;
+        }
+    }
+
+    float4_t acc[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t) acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+
+    if (tile_active) {
+        // keys this tile can need: from the lowest window start to the highest position of its rows
+        const int last_row = min(total_rows - 1, r0 + kRowsPerTile - 1);
+        const int tile_hi = min(key_end, first_pos + last_row / group + 1);
+        const int tile_lo = max(key_begin, window > 0 ? max(0, first_pos + r0 / group - window + 1) : 0);
+        const int blk_first = tile_lo / kKeysPerBlock;
+        const int blk_end = (tile_hi + kKeysPerBlock - 1) / kKeysPerBlock;
+        for (int blk = blk_first + ks; blk < blk_end; blk += key_splits) {
+            const int kbase = blk * kKeysPerBlock;
+            const bool edge = kbase < seg_lo || kbase + kKeysPerBlock > ctx;
+            // ---- scores of two tiles of 16 keys ----
+            float4_t s[2];
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2) {
+                // which key the A row i of this product is; see the header for why
+                int kk = kbase + (V16 ? 8 * (i / 4) + 4 * t2 + (i % 4) : 16 * t2 + i);
+                kk = min(kk, ctx - 1);
+                const int page = table[kk / page_size];
+                const bf16* krow = cache + static_cast<size_t>(page) * page_elems + k_off +
+                                   static_cast<size_t>(kk % page_size) * HD;
+                float4_t sc = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int c = 0; c < DC; ++c) {
+                    Pack16 a;
+                    a.u = *reinterpret_cast<const uint4*>(krow + c * 32 + 8 * g);
+                    sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qreg[c], sc, 0, 0, 0);
+                }
+                s[t2] = sc;
+            }
+            // ---- mask, running maximum, probabilities ----
+            float sv[8];
+            bool ok[8];
+            float tile_max = -INFINITY;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int t2 = e / 4, v = e % 4;
+                const int key = kbase + (V16 ? 8 * g + 4 * t2 + v : 16 * t2 + 4 * g + v);
+                ok[e] = row_valid && key <= pos && key >= lo && key >= key_begin && key < key_end;
+                sv[e] = s[t2][v];
+                if (ok[e]) tile_max = fmaxf(tile_max, sv[e]);
+            }
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
+            const float m_new = fmaxf(m_run, tile_max);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            const float alpha = exp2f((m_run - m_use) * scale_log2e);    // 0 while nothing was seen
+            Pack16 pv;
+            float psum = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float p = ok[e] ? exp2f((sv[e] - m_use) * scale_log2e) : 0.f;
+                psum += p;
+                pv.s[e] = bf16_bits(p);
+            }
+            l_run = l_run * alpha + psum;      // per lane; the four lanes of a row are added at the end
+            m_run = m_new;
+            // ---- out^T += V^T . P^T ----
+            int vpage0, vslot0, vpage1 = 0, vslot1 = 0;
+            if (V16) {
+                const int kk = min(kbase + 8 * g, ctx - 1) & ~7;
+                vpage0 = table[kk / page_size];
+                vslot0 = kk % page_size;
+            } else {
+                const int ka = min(kbase + 4 * g, ctx - 1) & ~3, kb = min(kbase + 16 + 4 * g, ctx - 1) & ~3;
+                vpage0 = table[ka / page_size];
+                vslot0 = ka % page_size;
+                vpage1 = table[kb / page_size];
+                vslot1 = kb % page_size;
+            }
+            const bf16* vbase0 = cache + static_cast<size_t>(vpage0) * page_elems + v_off + vslot0;
+            const bf16* vbase1 = cache + static_cast<size_t>(vpage1) * page_elems + v_off + vslot1;
+#pragma unroll
+            for (int t = 0; t < DT; ++t) {
+                const size_t drow = static_cast<size_t>(t * 16 + i) * page_size;
+                Pack16 a;
+                if (V16) {
+                    a.u = *reinterpret_cast<const uint4*>(vbase0 + drow);
+                } else {
+                    a.half[0] = *reinterpret_cast<const uint2*>(vbase0 + drow);
+                    a.half[1] = *reinterpret_cast<const uint2*>(vbase1 + drow);
+                }
+                if (edge) {
+                    // keys outside the request (stale slots, pages given back) may hold anything,
+                    // NaN included; 0 * NaN would poison the sum, so they are cleared
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const int key = kbase + (V16 ? 8 * g + e : (e < 4 ? 4 * g + e : 16 + 4 * g + e - 4));
+                        if (key >= ctx || key < seg_lo) a.s[e] = 0;
+                    }
+                }
+                acc[t] *= alpha;
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pv.v, acc[t], 0, 0, 0);
+            }
+        }
+        // the row's sum over its four lanes
+        l_run += __shfl_xor(l_run, 16, kWave);
+        l_run += __shfl_xor(l_run, 32, kWave);
+    }
+
+    // ---- merge the wavefronts that split the keys of one row tile ----
+    // lane (i, g) holds out^T[16t + 4g + v][row i]: element d = 16t + 4g + v of row i
+    for (int step = key_splits / 2; step >= 1; step /= 2) {
+        // wavefronts with ks in [step, 2*step) hand over to ks - step
+        __syncthreads();
+        const bool sender = ks >= step && ks < 2 * step;
+        const bool receiver = ks < step;
+        const int slot = (rt + row_tiles * (ks % step)) % 2;   // at most two pairs are live per step
+        float* buf = merge_s[slot] + i * (HD + 2);
+        if (sender) {
+#pragma unroll
+            for (int t = 0; t < DT; ++t)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) buf[t * 16 + 4 * g + v] = acc[t][v];
+            if (g == 0) {
+                buf[HD] = m_run;
+                buf[HD + 1] = l_run;
+            }
+        }
+        __syncthreads();
+        if (receiver) {
+            const float m_o = buf[HD], l_o = buf[HD + 1];
+            const float m_new = fmaxf(m_run, m_o);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            const float a_me = exp2f((m_run - m_use) * scale_log2e), a_o = exp2f((m_o - m_use) * scale_log2e);
+#pragma unroll
+            for (int t = 0; t < DT; ++t)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) acc[t][v] = acc[t][v] * a_me + buf[t * 16 + 4 * g + v] * a_o;
+            l_run = l_run * a_me + l_o * a_o;
+            m_run = m_new;
+        }
+    }
+
+    if (ks != 0 || !row_valid) return;
+    if (partial_slot < 0) {
+        const float inv = 1.f / l_run;
+        bf16* orow = out + (static_cast<size_t>(q_start + tok) * num_heads + head) * HD;
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+            uint2 w;
+            w.x = bf16_bits(acc[t][0] * inv) | (static_cast<uint32_t>(bf16_bits(acc[t][1] * inv)) << 16);
+            w.y = bf16_bits(acc[t][2] * inv) | (static_cast<uint32_t>(bf16_bits(acc[t][3] * inv)) << 16);
+            *reinterpret_cast<uint2*>(orow + t * 16 + 4 * g) = w;
+        }
+    } else {
+        const size_t prow = static_cast<size_t>(partial_slot) * kRowsPerTile + (row - row_begin);
+        float* po = partial_o + prow * HD;
+#pragma unroll
+        for (int t = 0; t < DT; ++t)
+            *reinterpret_cast<float4_t*>(po + t * 16 + 4 * g) = acc[t];
+        if (g == 0) {
+            partial_ml[prow * 2] = m_run;
+            partial_ml[prow * 2 + 1] = l_run;
+        }
+    }
+}
+
+// Combines the partial results of a (segment, key/value head) whose keys were split over workgroups.
+// reduce items: seg, kvh, first partial slot, number of splits.
+template <int HD>
+__global__ void __launch_bounds__(256)
+attention_reduce_kernel(const int* __restrict__ reduce_items, const float* __restrict__ partial_o,
+                        const float* __restrict__ partial_ml, const int* __restrict__ seg_q_start,
+                        const int* __restrict__ seg_q_len, bf16* __restrict__ out, int num_heads, int num_kv_heads,
+                        float scale_log2e) {
+    const int* item = reduce_items + static_cast<size_t>(blockIdx.x) * 4;
+    const int seg = item[0], kvh = item[1], first = item[2], splits = item[3];
+    if (seg < 0) return;
+    const int group = num_heads / num_kv_heads;
+    const int rows = seg_q_len[seg] * group;      // at most 16
+    const int q_start = seg_q_start[seg];
+    for (int idx = threadIdx.x; idx < rows * HD; idx += blockDim.x) {
+        const int r = idx / HD, d = idx % HD;
+        float m = -INFINITY;
+        for (int s = 0; s < splits; ++s) m = fmaxf(m, partial_ml[(static_cast<size_t>(first + s) * kRowsPerTile + r) * 2]);
+        float num = 0.f, den = 0.f;
+        for (int s = 0; s < splits; ++s) {
+            const size_t prow = static_cast<size_t>(first + s) * kRowsPerTile + r;
+            const float ms = partial_ml[prow * 2];
+            const float f = ms == -INFINITY ? 0.f : exp2f((ms - m) * scale_log2e);
+            num = fmaf(partial_o[prow * HD + d], f, num);
+            den = fmaf(partial_ml[prow * 2 + 1], f, den);
+        }
+        const int tok = r / group, head = kvh * group + r % group;
+        out[(static_cast<size_t>(q_start + tok) * num_heads + head) * HD + d] = from_float<bf16>(num / den);
+    }
+}
+
+// Returns 0, a HIP error code, or -1 for sizes these kernels do not take.
+WLLM_API int wllm_paged_attention_mfma(const void* qkv, const void* cache, const int* block_tables, const int* items,
+                                       int num_items, const int* reduce_items, int num_reduce_items,
+                                       const int* seg_q_start, const int* seg_q_len, const int* seg_ctx_len, void* out,
+                                       float* partial_o, float* partial_ml, int num_heads, int num_kv_heads,
+                                       int head_dim, int page_size, int max_pages, float scale, int window,
+                                       hipStream_t stream) {
+    if (head_dim % 32 != 0 || head_dim < 32 || head_dim > 256 || page_size % 4 != 0 || num_heads % num_kv_heads != 0)
+        return -1;
+    const float scale_log2e = scale * 1.4426950408889634f;
+    const bool v16 = page_size % 8 == 0;
+#define LAUNCH(HD, V16)                                                                                              \
+    paged_attention_mfma_kernel<HD, V16><<<num_items, 256, 0, stream>>>(                                            \
+        static_cast<const bf16*>(qkv), static_cast<const bf16*>(cache), block_tables, items, seg_q_start, seg_q_len, \
+        seg_ctx_len, static_cast<bf16*>(out), partial_o, partial_ml, num_heads, num_kv_heads, page_size, max_pages,  \
+        scale_log2e, window)
+#define LAUNCH_R(HD)                                                                                                 \
+    attention_reduce_kernel<HD><<<num_reduce_items, 256, 0, stream>>>(reduce_items, partial_o, partial_ml, seg_q_start, \
+                                                                      seg_q_len, static_cast<bf16*>(out), num_heads,  \
+                                                                      num_kv_heads, scale_log2e)
+#define CASE(HD)                                   \
+    case HD:                                       \
+        if (num_items > 0) {                       \
+            if (v16) LAUNCH(HD, true);             \
+            else LAUNCH(HD, false);                \
+        }                                          \
+        if (num_reduce_items > 0) LAUNCH_R(HD);    \
+        break;
+    switch (head_dim) {
+        CASE(32)
+        CASE(64)
+        CASE(96)
+        CASE(128)
+        CASE(160)
+        CASE(192)
+        CASE(224)
+        CASE(256)
+        default:
+            return -1;
+    }
+#undef CASE
+#undef LAUNCH
+#undef LAUNCH_R
+    return launch_status();
+}

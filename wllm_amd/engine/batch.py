@@ -86,6 +86,17 @@ class StepContext:
         self.requests = requests
         self.max_q_len = int(host_q_len.max()) if num_segments else 0
         self.max_ctx_len = int(host_ctx_len.max()) if num_segments else 0
+        self._attention_plans: dict = {}
+
+    def attention_plan(self, *, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, window: int):
+        """The step's work items for attention of this shape; made once, shared by all layers."""
+        from wllm_amd.kernels import ops
+        key = (num_heads, num_kv_heads, head_dim, page_size, window)
+        if key not in self._attention_plans:
+            self._attention_plans[key] = ops.plan_paged_attention(
+                self.host_q_len, self.host_ctx_len, num_heads=num_heads, num_kv_heads=num_kv_heads,
+                head_dim=head_dim, page_size=page_size, window=window, dtype=self.dtype, device=self.device)
+        return self._attention_plans[key]
 
     def buffer(self, name: str, shape: tuple, dtype: torch.dtype) -> torch.Tensor:
         return self._workspace.get(name, shape, dtype)

@@ -1,0 +1,107 @@
+"""How a step's attention is cut into work items for the matrix-core kernel.
+
+For one request (segment) and one key/value head the query rows are the pairs (token, query
+head of the group): rows = q_len * group.  A segment of at most 16 rows (a decoded token) is one
+tile of rows whose keys are split over workgroups in fixed chunks of `KEY_CHUNK` keys, the
+partial results combined by a second kernel; chunk boundaries are multiples of the chunk size
+counted from key 0, so they depend on the key index only.  Longer segments are cut into
+workgroups of up to four tiles of 16 rows that each walk all their keys.
+
+A work item is 8 int32: segment, key/value head, first row, row tiles (1, 2 or 4), first key,
+end key, partial slot (-1: the workgroup writes the final result), unused.  A reduce item is
+4 int32: segment, key/value head, first partial slot, number of splits.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+import numpy as np
+import torch
+
+KEY_CHUNK = 256
+ROWS_PER_TILE = 16
+ITEM_INTS = 8
+
+
+@dataclass
+class AttentionPlan:
+    items: torch.Tensor                 # int32 [num_items, 8] on the device
+    reduce_items: Optional[torch.Tensor]  # int32 [num_reduce, 4] or None
+    num_items: int
+    num_reduce: int
+    num_partial_slots: int
+
+
+def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_heads: int, window: int,
+                     fixed_splits: int = 0):
+    """Returns (items [n, 8], reduce_items [m, 4], partial slots) as int32 arrays.
+
+    `fixed_splits` > 0 gives every short segment exactly that many items per key/value head
+    (items beyond the segment's keys are padding that the kernel skips), so that the number
+    of items depends on the number of segments only: the shape a captured graph needs.
+    """
+    q_len = np.asarray(q_len, dtype=np.int64)
+    ctx_len = np.asarray(ctx_len, dtype=np.int64)
+    rows = q_len * group
+    short = rows <= ROWS_PER_TILE
+    items, reduces = [], []
+    slots = 0
+    kv = np.arange(num_kv_heads, dtype=np.int64)
+    # ---- short segments, vectorised over segments ----
+    idx = np.nonzero(short)[0]
+    if idx.size:
+        first_pos = ctx_len[idx] - q_len[idx]
+        lo = np.maximum(0, first_pos - window + 1) if window > 0 else np.zeros_like(first_pos)
+        c0 = lo // KEY_CHUNK
+        c1 = (ctx_len[idx] - 1) // KEY_CHUNK
+        ns = c1 - c0 + 1
+        width = int(fixed_splits) if fixed_splits > 0 else int(ns.max())
+        if fixed_splits > 0 and int(ns.max()) > fixed_splits:
+            raise ValueError(f"a segment needs {int(ns.max())} key chunks, the plan is fixed at {fixed_splits}")
+        j = np.arange(width, dtype=np.int64)
+        chunk = c0[:, None] + j[None, :]                       # [S, width]
+        live = j[None, :] < ns[:, None]
+        kb = np.maximum(lo[:, None], chunk * KEY_CHUNK)
+        ke = np.minimum(ctx_len[idx][:, None], (chunk + 1) * KEY_CHUNK)
+        single = (ns == 1) & (fixed_splits <= 0)
+        # partial slots: one per (segment, kv head, split) for segments that are split
+        n_split_seg = np.where(single, 0, width if fixed_splits > 0 else ns)
+        seg_base = np.concatenate([[0], np.cumsum(n_split_seg * num_kv_heads)])[:-1]
+        S = idx.size
+        it = np.zeros((S, num_kv_heads, width, ITEM_INTS), dtype=np.int32)
+        it[..., 0] = np.where(live, idx[:, None], -1)[:, None, :]
+        it[..., 1] = kv[None, :, None]
+        it[..., 2] = 0
+        it[..., 3] = 1
+        it[..., 4] = kb[:, None, :]
+        it[..., 5] = ke[:, None, :]
+        slot = seg_base[:, None, None] + kv[None, :, None] * n_split_seg[:, None, None] + j[None, None, :]
+        it[..., 6] = np.where(single[:, None, None], -1, slot)
+        if fixed_splits > 0:
+            keep = np.ones((S, num_kv_heads, width), dtype=bool)
+        else:
+            keep = np.broadcast_to(live[:, None, :], (S, num_kv_heads, width))
+        items.append(it[keep].reshape(-1, ITEM_INTS))
+        split_seg = ~single
+        if split_seg.any():
+            rs = np.zeros((S, num_kv_heads, 4), dtype=np.int32)
+            rs[..., 0] = idx[:, None]
+            rs[..., 1] = kv[None, :]
+            rs[..., 2] = seg_base[:, None] + kv[None, :] * n_split_seg[:, None]
+            rs[..., 3] = ns[:, None]
+            reduces.append(rs[split_seg].reshape(-1, 4))
+        slots = int((n_split_seg * num_kv_heads).sum())
+    # ---- long segments: workgroups of up to four row tiles over all keys ----
+    for s in np.nonzero(~short)[0]:
+        tiles = -(-int(rows[s]) // ROWS_PER_TILE)
+        t = 0
+        while t < tiles:
+            left = tiles - t
+            rt = 4 if left >= 3 else left          # 3 tiles run as 4 with one idle wavefront
+            for h in range(num_kv_heads):
+                items.append(np.array([[s, h, t * ROWS_PER_TILE, rt, 0, int(ctx_len[s]), -1, 0]], dtype=np.int32))
+            t += rt
+    items = np.concatenate(items) if items else np.zeros((0, ITEM_INTS), np.int32)
+    reduces = np.concatenate(reduces) if reduces else np.zeros((0, 4), np.int32)
+    return items, reduces, slots

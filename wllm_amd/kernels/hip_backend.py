@@ -6,8 +6,10 @@ from __future__ import annotations
 import ctypes
 from ctypes import c_float, c_int, c_longlong, c_void_p
 
+import numpy as np
 import torch
 
+from wllm_amd.kernels.attention_plan import AttentionPlan, build_work_items
 from wllm_amd.kernels.library import load
 
 
@@ -28,6 +30,9 @@ _SIGNATURES = {
     "wllm_gated_activation": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_paged_attention_generic": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+    "wllm_paged_attention_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
+                                  c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
+                                  c_int, c_void_p],
     "wllm_gemm_generic": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_argmax_rows": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "wllm_sample_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
@@ -39,6 +44,8 @@ class HipBackend:
         if not torch.cuda.is_available():
             raise KernelError("no GPU is visible; the kernels run on gfx950 only and there is no other path")
         self.lib = load()
+        self._partial_o = None
+        self._partial_ml = None
         for name, argtypes in _SIGNATURES.items():
             fn = getattr(self.lib, name)
             fn.argtypes = argtypes
@@ -82,9 +89,44 @@ class HipBackend:
             _ptr(cache), cache.shape[0] if cache is not None else 0, qkv.shape[0], num_heads, num_kv_heads, head_dim,
             rotary_dim, page_size, self._stream()), "rope_and_cache_write")
 
+    @staticmethod
+    def mfma_attention_takes(dtype, head_dim: int, page_size: int) -> bool:
+        """The matrix-core kernel: bfloat16, head sizes 32..256 in steps of 32, pages of a multiple of 4."""
+        return dtype == torch.bfloat16 and head_dim % 32 == 0 and 32 <= head_dim <= 256 and page_size % 4 == 0
+
+    def plan_paged_attention(self, host_q_len, host_ctx_len, num_heads, num_kv_heads, head_dim, page_size, window,
+                             dtype, device, fixed_splits: int = 0):
+        if not self.mfma_attention_takes(dtype, head_dim, page_size):
+            return None
+        items, reduces, slots = build_work_items(host_q_len, host_ctx_len, num_heads // num_kv_heads, num_kv_heads,
+                                                 window, fixed_splits)
+        flat = np.concatenate([items.reshape(-1), reduces.reshape(-1)])
+        dev = torch.from_numpy(flat).to(device, non_blocking=True)
+        n_i, n_r = items.shape[0], reduces.shape[0]
+        self._ensure_partials(slots, head_dim, device)
+        return AttentionPlan(dev[:n_i * 8].view(n_i, 8), dev[n_i * 8:].view(n_r, 4) if n_r else None, n_i, n_r, slots)
+
+    def _ensure_partials(self, slots: int, head_dim: int, device) -> None:
+        need = max(1, slots) * 16 * head_dim
+        if self._partial_o is None or self._partial_o.numel() < need or self._partial_o.device != torch.device(device):
+            self._partial_o = torch.empty(need, dtype=torch.float32, device=device)
+        need = max(1, slots) * 16 * 2
+        if self._partial_ml is None or self._partial_ml.numel() < need or self._partial_ml.device != torch.device(device):
+            self._partial_ml = torch.empty(need, dtype=torch.float32, device=device)
+
     def paged_attention(self, qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len, out,
-                        num_heads, num_kv_heads, head_dim, page_size, scale, window, max_q_len, max_ctx_len):
+                        num_heads, num_kv_heads, head_dim, page_size, scale, window, max_q_len, max_ctx_len,
+                        plan=None):
         self._on_gpu(qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len, out)
+        if plan is not None:
+            if not self.mfma_attention_takes(qkv.dtype, head_dim, page_size):
+                raise KernelError("paged_attention: a plan was given for sizes the matrix-core kernel does not take")
+            self._check(self.lib.wllm_paged_attention_mfma(
+                _ptr(qkv), _ptr(cache), _ptr(block_tables), _ptr(plan.items), plan.num_items, _ptr(plan.reduce_items),
+                plan.num_reduce, _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out),
+                _ptr(self._partial_o), _ptr(self._partial_ml), num_heads, num_kv_heads, head_dim, page_size,
+                block_tables.shape[1], scale, window, self._stream()), "paged_attention (matrix cores)")
+            return
         if head_dim % 4 or head_dim > 256:
             raise KernelError(f"paged_attention: head_dim {head_dim} is not a multiple of 4 up to 256")
         self._check(self.lib.wllm_paged_attention_generic(

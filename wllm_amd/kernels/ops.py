@@ -139,7 +139,7 @@ def paged_attention(qkv: torch.Tensor, cache: torch.Tensor, block_tables: torch.
                     token_segment: torch.Tensor, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor,
                     seg_ctx_len: torch.Tensor, out: torch.Tensor, *, num_heads: int, num_kv_heads: int,
                     head_dim: int, page_size: int, scale: float, window: int = 0,
-                    max_q_len: int = 0, max_ctx_len: int = 0) -> None:
+                    max_q_len: int = 0, max_ctx_len: int = 0, plan=None) -> None:
     """Softmax attention of every query over the keys of its own request in the paged cache.
 
     The batch is a row of segments; segment s holds tokens seg_q_start[s] .. +seg_q_len[s],
@@ -150,6 +150,7 @@ def paged_attention(qkv: torch.Tensor, cache: torch.Tensor, block_tables: torch.
     weighted sum accumulate in float32.  qkv as in `rope_and_cache_write` (only the queries
     are read); block_tables int32 [S, max_pages]; out T [n, num_heads*head_dim].
     max_q_len / max_ctx_len are host-side bounds of the segment arrays (0: unknown).
+    `plan`: what `plan_paged_attention` returned for these segments and sizes, or None.
     """
     width = (num_heads + 2 * num_kv_heads) * head_dim
     _dense(qkv, "qkv", _ACT)
@@ -170,7 +171,17 @@ def paged_attention(qkv: torch.Tensor, cache: torch.Tensor, block_tables: torch.
     if n:
         backend().paged_attention(qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len,
                                   out, num_heads, num_kv_heads, head_dim, page_size, float(scale), int(window),
-                                  int(max_q_len), int(max_ctx_len))
+                                  int(max_q_len), int(max_ctx_len), plan)
+
+
+def plan_paged_attention(host_q_len, host_ctx_len, *, num_heads: int, num_kv_heads: int, head_dim: int,
+                         page_size: int, window: int, dtype: torch.dtype, device):
+    """Cuts a step's attention into work items for the kernels that want them, once per step
+    and attention shape (all layers of that shape share it).  Returns an opaque plan, or None
+    when the kernel that will run needs none.  host_q_len / host_ctx_len: the segment arrays
+    on the host."""
+    return backend().plan_paged_attention(host_q_len, host_ctx_len, num_heads, num_kv_heads, head_dim, page_size,
+                                          int(window), dtype, device)
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> None:

@@ -87,7 +87,9 @@ class PagedAttention:
             qkv, pages.storage, pages.block_tables, ctx.token_segment, ctx.seg_q_start, ctx.seg_q_len,
             ctx.seg_ctx_len, attn, num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim,
             page_size=pages.page_size, scale=s.scale, window=s.window or 0,
-            max_q_len=ctx.max_q_len, max_ctx_len=ctx.max_ctx_len)
+            max_q_len=ctx.max_q_len, max_ctx_len=ctx.max_ctx_len,
+            plan=ctx.attention_plan(num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim,
+                                    page_size=pages.page_size, window=s.window or 0))
         y = ctx.buffer("mixer_out", (n, s.hidden_size), h.dtype)
         ops.linear(attn, self.w_o, y)
         return y
