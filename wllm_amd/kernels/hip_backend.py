@@ -35,6 +35,7 @@ _SIGNATURES = {
                                   c_int, c_void_p],
     "wllm_gemm_generic": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_argmax_rows": [c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "wllm_gemm_skinny": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_sample_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
 
@@ -45,6 +46,7 @@ class HipBackend:
             raise KernelError("no GPU is visible; the kernels run on gfx950 only and there is no other path")
         self.lib = load()
         self._partial_o = None
+        self._gemm_partials = None
         self._partial_ml = None
         for name, argtypes in _SIGNATURES.items():
             fn = getattr(self.lib, name)
@@ -134,12 +136,47 @@ class HipBackend:
             _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out), qkv.shape[0], num_heads, num_kv_heads,
             head_dim, page_size, block_tables.shape[1], scale, window, self._stream()), "paged_attention")
 
+    @staticmethod
+    def skinny_split(n: int, k: int) -> int:
+        """Over how many workgroups the K axis of a few-row product is split: enough that about
+        2,000 wavefronts stream weights at once, a function of the weight's shape only."""
+        tiles = -(-n // 16)
+        splits = 1
+        while tiles * splits < 1536 and k % (splits * 2) == 0 and (k // (splits * 2)) % 32 == 0 \
+                and k // (splits * 2) >= 256:
+            splits *= 2
+        return splits
+
+    def _gemm_partial(self, count: int, device) -> torch.Tensor:
+        if self._gemm_partials is None or self._gemm_partials.numel() < count or self._gemm_partials.device != device:
+            self._gemm_partials = torch.empty(count, dtype=torch.float32, device=device)
+        return self._gemm_partials
+
+    def _skinny(self, x, weight, out) -> None:
+        m, k = x.shape
+        n = weight.shape[0]
+        splits = self.skinny_split(n, k)
+        mt = -(-m // 16)
+        chunk = {1: 1024, 2: 512, 3: 256, 4: 256}[mt]
+        partial = self._gemm_partial(splits * m * n, x.device) if splits > 1 else None
+        self._check(self.lib.wllm_gemm_skinny(_ptr(x), _ptr(weight), _ptr(out), int(out.dtype == torch.bfloat16),
+                                              _ptr(partial), m, n, k, splits, chunk, self._stream()),
+                    "linear (few rows, matrix cores)")
+
     def linear(self, x, weight, out):
         self._on_gpu(x, weight, out)
-        if x.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and x.shape[0] > 64:
-            # many rows, bfloat16: the library's matrix-core product (float32 accumulation)
-            torch.mm(x, weight.t(), out=out)
-            return
+        m, k = x.shape
+        if x.dtype == torch.bfloat16:
+            if k % 32 == 0 and (m <= 64 or out.dtype == torch.float32):
+                # few rows: the weight-streaming kernel; float32 results from bfloat16 operands
+                # (logits) take it in blocks of 64 rows
+                for r in range(0, m, 64):
+                    self._skinny(x[r:r + 64], weight, out[r:r + 64])
+                return
+            if out.dtype == torch.bfloat16 and m > 64:
+                # many rows: the library's matrix-core product (float32 accumulation)
+                torch.mm(x, weight.t(), out=out)
+                return
         self._check(self.lib.wllm_gemm_generic(
             _ptr(x), _ptr(weight), int(x.dtype == torch.bfloat16), _ptr(out), int(out.dtype == torch.bfloat16),
             x.shape[0], weight.shape[0], x.shape[1], self._stream()), "linear")
