@@ -92,7 +92,7 @@ def measure_decode(model, batch: int, context: int, steps: int, warmup: int, blo
 
     from wllm_amd.engine import ModelRunner, Request, Scheduler
     total_new = warmup + steps + 1
-    pages = batch * (-(-(context + total_new) // block_size))
+    pages = batch * (-(-(context + total_new) // block_size)) + 2
     runner = ModelRunner.create(model, num_pages=pages, page_size=block_size, max_requests=batch)
     if hip_graphs and hasattr(runner, "enable_graphs"):
         runner.enable_graphs()

@@ -147,3 +147,33 @@ def test_trace_run_program(model_folders, tmp_path, dtype):
         got = torch.from_numpy(np.fromfile(out / f"{step}.f32", dtype="<f4").reshape(len(rows), 512))
         ref = torch.stack(rows)
         assert ((got.double() - ref.double()).abs() <= atol + rtol * ref.double().abs()).all(), f"step {step}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_graphs_give_what_eager_steps_give(model_folders, dtype):
+    """Decode steps replayed from captured graphs against the same steps run kernel by kernel:
+    several replays with eager work (prompt portions of newly admitted requests) between them,
+    batches that grow and shrink through the buckets, every replay checked."""
+    folder = model_folders["M"]
+    model = load_model(folder, dtype, "cuda")
+    prompts = [random_ids(40 + i, n, 1000) for i, n in enumerate([9, 33, 17, 70, 5, 41])]
+    news = [30, 12, 25, 8, 40, 18]
+
+    def run(graphs):
+        runner = ModelRunner.create(model, num_pages=40, page_size=16, max_requests=4)
+        if graphs:
+            runner.enable_graphs(buckets=(1, 2, 4))
+        s = Scheduler(runner, max_prefill_tokens_per_step=16)
+        reqs = [Request(i, p, n) for i, (p, n) in enumerate(zip(prompts, news))]
+        for r in reqs:
+            s.add_request(r)
+        s.run_to_completion()
+        runner.cache.check()
+        return reqs, runner
+
+    eager, _ = run(False)
+    graphed, runner = run(True)
+    assert runner.graph_steps > 20 and len(runner.graphs) >= 2
+    for a, b in zip(eager, graphed):
+        assert a.output_token_ids == b.output_token_ids
+        assert torch.allclose(torch.tensor(a.logprobs), torch.tensor(b.logprobs), atol=1e-5 if dtype == "float32" else 2e-2)

@@ -31,6 +31,9 @@ import torch
 from wllm_amd.cache.pages import OutOfPages, PageAccountingError, PagePool
 
 
+_SET_ASIDE = "(set aside)"
+
+
 class OutOfSlots(RuntimeError):
     """More live requests than state slots."""
 
@@ -99,6 +102,7 @@ class CacheManager:
                 self.group_of_entry[e] = len(self.groups)
             self.groups.append(g)
         self.requests: dict = {}
+        self._set_aside: dict = {}
         self._free_slots = list(range(max_requests - 1, -1, -1))
         self.state: dict = {}
         for entry, shape in (state_shapes or {}).items():
@@ -155,6 +159,13 @@ class CacheManager:
 
     def num_free_pages(self, group_index: int = 0) -> int:
         return self.groups[group_index].pool.num_free
+
+    def set_aside_page(self, group_index: int) -> int:
+        """Takes one page of a group out of circulation for good (captured graphs point
+        their padding rows at it) and returns its id."""
+        page = self.groups[group_index].pool.allocate(_SET_ASIDE)
+        self._set_aside.setdefault(group_index, []).append(page)
+        return page
 
     def reserve(self, request, num_new_tokens: int) -> list:
         """Makes room for the next `num_new_tokens` tokens of a request in every
@@ -247,7 +258,7 @@ class CacheManager:
                     seen[page] = request
                     if g.pool.holder(page) != request:
                         raise PageAccountingError(f"page {page} in the table of {request!r} is held by {g.pool.holder(page)!r}")
-            if set(seen) != set(g.pool.held_pages()):
+            if set(seen) | set(self._set_aside.get(gi, [])) != set(g.pool.held_pages()):
                 raise PageAccountingError("a held page is in no table")
         slots = [rc.slot for rc in self.requests.values()]
         if len(set(slots)) != len(slots) or set(slots) & set(self._free_slots):

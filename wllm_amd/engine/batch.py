@@ -87,11 +87,22 @@ class StepContext:
         self.max_q_len = int(host_q_len.max()) if num_segments else 0
         self.max_ctx_len = int(host_ctx_len.max()) if num_segments else 0
         self._attention_plans: dict = {}
+        # set by a captured graph: plans of fixed shape, refreshed in place before each replay
+        self.static_plans = False
+        self.static_max_context = 0
+        self.static_max_total_keys = 0
 
     def attention_plan(self, *, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, window: int):
         """The step's work items for attention of this shape; made once, shared by all layers."""
         from wllm_amd.kernels import ops
         key = (num_heads, num_kv_heads, head_dim, page_size, window)
+        if key not in self._attention_plans and self.static_plans:
+            plan = ops.backend().static_attention_plan(
+                self.num_segments, num_heads, num_kv_heads, head_dim, page_size, window, self.dtype, self.device,
+                self.static_max_context, self.static_max_total_keys)
+            if plan is not None:
+                plan.update(self.host_q_len, self.host_ctx_len)
+            self._attention_plans[key] = plan
         if key not in self._attention_plans:
             self._attention_plans[key] = ops.plan_paged_attention(
                 self.host_q_len, self.host_ctx_len, num_heads=num_heads, num_kv_heads=num_kv_heads,

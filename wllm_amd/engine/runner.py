@@ -30,6 +30,37 @@ class ModelRunner:
         self.workspace = Workspace(self.device)
         self.steps_run = 0
         self.tokens_run = 0
+        self.graphs: dict = {}             # bucket -> DecodeGraph
+        self.graph_buckets: tuple = ()
+        self.graph_max_context = 0
+        self.dummy_pages: list = []
+        self.graph_steps = 0
+
+    def enable_graphs(self, buckets=(1, 2, 4, 8, 16, 32, 64), max_context=None) -> None:
+        """Decode-only steps of up to max(buckets) requests replay a captured graph of the
+        smallest bucket that holds them.  One page per group is set aside for padding rows."""
+        if self.graph_buckets:
+            return
+        if not self.model.graph_capturable():
+            raise ValueError("a part of this model reads the step's arrays on the host; its steps cannot be captured")
+        limit = min(self.model.plan.max_positions, min(g.pool.num_pages - 1 for g in self.cache.groups) * self.cache.page_size)
+        self.graph_max_context = min(max_context or limit, limit)
+        self.graph_buckets = tuple(sorted(b for b in buckets if b <= self.cache.max_requests)) or (self.cache.max_requests,)
+        self.dummy_pages = [self.cache.set_aside_page(gi) for gi in range(len(self.cache.groups))]
+
+    def _graph_for(self, entries: list):
+        if not self.graph_buckets or len(entries) > self.graph_buckets[-1]:
+            return None
+        for e in entries:
+            if len(e.tokens) != 1 or list(e.want) != [0]:
+                return None
+            if self.cache.context_len(e.request) + 1 > self.graph_max_context:
+                return None
+        bucket = next(b for b in self.graph_buckets if b >= len(entries))
+        if bucket not in self.graphs:
+            from wllm_amd.engine.graphs import DecodeGraph
+            self.graphs[bucket] = DecodeGraph(self, bucket, self.graph_max_context)
+        return self.graphs[bucket]
 
     @classmethod
     def create(cls, model, *, num_pages: int, page_size: int, max_requests: int, **cache_options):
@@ -46,8 +77,15 @@ class ModelRunner:
     def step(self, entries: list) -> torch.Tensor:
         """Returns float32 logits [wanted, vocab] in the order of the entries and of
         each entry's `want`.  The tensor is a view of a buffer the next step reuses."""
-        ctx = self.prepare(entries)
-        logits = self.model.forward(ctx)
+        graph = self._graph_for(entries) if entries else None
+        if graph is not None:
+            self._validate(entries)
+            reserved = self._reserve(entries)
+            logits = graph.run(entries, reserved)
+            self.graph_steps += 1
+        else:
+            ctx = self.prepare(entries)
+            logits = self.model.forward(ctx)
         self.commit(entries)
         return logits
 
@@ -61,6 +99,12 @@ class ModelRunner:
     def prepare(self, entries: list) -> StepContext:
         """Checks the entries, takes room for them in the cache (all or none) and builds
         the step's index tensors."""
+        self._validate(entries)
+        cache = self.cache
+        reserved = self._reserve(entries)
+        return self._build_context(entries, reserved)
+
+    def _validate(self, entries: list) -> None:
         cache = self.cache
         max_pos = self.model.plan.max_positions
         seen = set()
@@ -78,17 +122,26 @@ class ModelRunner:
             for w in e.want:
                 if not 0 <= w < len(e.tokens):
                     raise StepError(f"request {e.request!r}: wanted place {w} is not among its {len(e.tokens)} tokens")
-        vocab = self.model.plan.embedding.vocab_size
-        num_groups = len(cache.groups)
-        # room first: all entries or none
+            vocab = self.model.plan.embedding.vocab_size
+            if min(e.tokens) < 0 or max(e.tokens) >= vocab:
+                raise StepError(f"request {e.request!r}: token id outside 0..{vocab - 1}")
+
+    def _reserve(self, entries: list) -> list:
+        """Room for every entry, or for none."""
+        cache = self.cache
         reserved = []
         try:
             for e in entries:
                 reserved.append(cache.reserve(e.request, len(e.tokens)))
         except OutOfPages:
-            for e in entries[:len(reserved)]:
+            for e in entries[:len(reserved) + 1]:
                 cache.trim(e.request)
             raise
+        return reserved
+
+    def _build_context(self, entries: list, reserved: list) -> StepContext:
+        cache = self.cache
+        num_groups = len(cache.groups)
         s = len(entries)
         q_len = np.array([len(e.tokens) for e in entries], dtype=np.int32)
         q_start = np.zeros(s, dtype=np.int32)
@@ -98,8 +151,6 @@ class ModelRunner:
         old_len = np.array([cache.context_len(e.request) for e in entries], dtype=np.int32)
         ctx_len = old_len + q_len
         token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries]) if s else np.zeros(0, np.int64)
-        if n and (token_ids.min() < 0 or token_ids.max() >= vocab):
-            raise StepError(f"token id outside 0..{vocab - 1}")
         token_ids = token_ids.astype(np.int32)
         token_segment = np.repeat(np.arange(s, dtype=np.int32), q_len)
         positions = (np.arange(n, dtype=np.int32) - q_start[token_segment] + old_len[token_segment]).astype(np.int32)

@@ -31,6 +31,38 @@ class AttentionPlan:
     num_items: int
     num_reduce: int
     num_partial_slots: int
+    partial_o: Optional[torch.Tensor] = None    # float32 [slots * 16 * head_dim]
+    partial_ml: Optional[torch.Tensor] = None   # float32 [slots * 16 * 2]
+
+
+class StaticAttentionPlan(AttentionPlan):
+    """A plan of fixed shape for a captured graph: always `segments * kv_heads * fixed_splits`
+    work items in the same device tensors, whose contents `update` rewrites before each replay.
+    Partial slots are numbered over the live chunks only, so the partial buffers are as large
+    as the most keys the cache pool can hold needs, not as the fixed shape."""
+
+    def __init__(self, segments: int, group: int, num_kv_heads: int, window: int, fixed_splits: int,
+                 max_slots: int, head_dim: int, device):
+        n_i, n_r = segments * num_kv_heads * fixed_splits, segments * num_kv_heads
+        self._host = torch.empty(n_i * ITEM_INTS + n_r * 4, dtype=torch.int32, pin_memory=True)
+        self._dev = torch.empty_like(self._host, device=device)
+        self._args = (group, num_kv_heads, window, fixed_splits)
+        self.max_slots = max_slots
+        super().__init__(self._dev[:n_i * ITEM_INTS].view(n_i, ITEM_INTS), self._dev[n_i * ITEM_INTS:].view(n_r, 4),
+                         n_i, n_r, max_slots,
+                         torch.empty(max(1, max_slots) * ROWS_PER_TILE * head_dim, dtype=torch.float32, device=device),
+                         torch.empty(max(1, max_slots) * ROWS_PER_TILE * 2, dtype=torch.float32, device=device))
+
+    def update(self, q_len: np.ndarray, ctx_len: np.ndarray) -> None:
+        group, nkv, window, fixed = self._args
+        items, reduces, slots = build_work_items(q_len, ctx_len, group, nkv, window, fixed)
+        if slots > self.max_slots:
+            raise ValueError(f"the step needs {slots} partial slots, the graph's plan has {self.max_slots}")
+        assert items.shape[0] == self.num_items and reduces.shape[0] == self.num_reduce
+        buf = self._host.numpy()
+        buf[:items.size] = items.reshape(-1)
+        buf[items.size:] = reduces.reshape(-1)
+        self._dev.copy_(self._host, non_blocking=True)
 
 
 def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_heads: int, window: int,
@@ -66,7 +98,7 @@ def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_
         ke = np.minimum(ctx_len[idx][:, None], (chunk + 1) * KEY_CHUNK)
         single = (ns == 1) & (fixed_splits <= 0)
         # partial slots: one per (segment, kv head, split) for segments that are split
-        n_split_seg = np.where(single, 0, width if fixed_splits > 0 else ns)
+        n_split_seg = np.where(single, 0, ns)
         seg_base = np.concatenate([[0], np.cumsum(n_split_seg * num_kv_heads)])[:-1]
         S = idx.size
         it = np.zeros((S, num_kv_heads, width, ITEM_INTS), dtype=np.int32)

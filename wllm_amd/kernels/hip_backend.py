@@ -106,7 +106,19 @@ class HipBackend:
         dev = torch.from_numpy(flat).to(device, non_blocking=True)
         n_i, n_r = items.shape[0], reduces.shape[0]
         self._ensure_partials(slots, head_dim, device)
-        return AttentionPlan(dev[:n_i * 8].view(n_i, 8), dev[n_i * 8:].view(n_r, 4) if n_r else None, n_i, n_r, slots)
+        return AttentionPlan(dev[:n_i * 8].view(n_i, 8), dev[n_i * 8:].view(n_r, 4) if n_r else None, n_i, n_r, slots,
+                             self._partial_o, self._partial_ml)
+
+    def static_attention_plan(self, segments, num_heads, num_kv_heads, head_dim, page_size, window, dtype, device,
+                              max_context: int, max_total_keys: int):
+        """A plan of fixed shape for a captured decode graph of `segments` requests of one token."""
+        if not self.mfma_attention_takes(dtype, head_dim, page_size):
+            return None
+        from wllm_amd.kernels.attention_plan import KEY_CHUNK, StaticAttentionPlan
+        fixed = -(-max_context // KEY_CHUNK)
+        max_slots = (max_total_keys // KEY_CHUNK + 2 * segments) * num_kv_heads
+        return StaticAttentionPlan(segments, num_heads // num_kv_heads, num_kv_heads, window, fixed, max_slots,
+                                   head_dim, device)
 
     def _ensure_partials(self, slots: int, head_dim: int, device) -> None:
         need = max(1, slots) * 16 * head_dim
@@ -126,7 +138,7 @@ class HipBackend:
             self._check(self.lib.wllm_paged_attention_mfma(
                 _ptr(qkv), _ptr(cache), _ptr(block_tables), _ptr(plan.items), plan.num_items, _ptr(plan.reduce_items),
                 plan.num_reduce, _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out),
-                _ptr(self._partial_o), _ptr(self._partial_ml), num_heads, num_kv_heads, head_dim, page_size,
+                _ptr(plan.partial_o), _ptr(plan.partial_ml), num_heads, num_kv_heads, head_dim, page_size,
                 block_tables.shape[1], scale, window, self._stream()), "paged_attention (matrix cores)")
             return
         if head_dim % 4 or head_dim > 256:
@@ -147,9 +159,16 @@ class HipBackend:
             splits *= 2
         return splits
 
+    # splits * N stays below 3072 * 16 by the rule of `skinny_split`; 64 rows of float32 of that
+    GEMM_PARTIAL_FLOATS = 3072 * 16 * 64
+
     def _gemm_partial(self, count: int, device) -> torch.Tensor:
-        if self._gemm_partials is None or self._gemm_partials.numel() < count or self._gemm_partials.device != device:
-            self._gemm_partials = torch.empty(count, dtype=torch.float32, device=device)
+        """The buffer of split sums.  It is allocated once at its largest size and never again,
+        because captured graphs hold its address."""
+        if count > self.GEMM_PARTIAL_FLOATS:
+            raise KernelError(f"split-sum buffer: {count} floats needed, {self.GEMM_PARTIAL_FLOATS} reserved")
+        if self._gemm_partials is None or self._gemm_partials.device != device:
+            self._gemm_partials = torch.empty(self.GEMM_PARTIAL_FLOATS, dtype=torch.float32, device=device)
         return self._gemm_partials
 
     def _skinny(self, x, weight, out) -> None:

@@ -24,6 +24,8 @@ from wllm_amd.weights.checkpoint import ExpectedTensor
 
 @register_mixer("attention")
 class PagedAttention:
+    graph_capturable = True     # everything it does reads the step's device arrays
+
     def __init__(self, spec: AttentionSpec):
         if spec.num_heads % spec.num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")

@@ -73,6 +73,11 @@ class CausalLM:
                 shapes[i] = tuple(shape)
         return shapes
 
+    def graph_capturable(self) -> bool:
+        """True if every part runs from the step's device arrays alone, so that a step can be
+        captured once and replayed with other contents.  A mixer says so with an attribute."""
+        return all(getattr(b.mixer, "graph_capturable", False) for b in self.blocks)
+
     # ---- weights ---------------------------------------------------------------
     def expected_tensors(self) -> dict:
         emb, head = self.plan.embedding, self.plan.head
