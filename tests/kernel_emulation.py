@@ -15,9 +15,10 @@ import torch
 
 
 class EmulatedKernels:
-    def __init__(self, precise: bool = False):
+    def __init__(self, precise: bool = False, splits: int = 1):
         self.acc = torch.float64 if precise else torch.float32
         self.calls = {}
+        self.splits = splits        # into how many partial sums `linear` is asked to split
 
     def _count(self, name):
         self.calls[name] = self.calls.get(name, 0) + 1
@@ -28,6 +29,11 @@ class EmulatedKernels:
 
     def rms_norm(self, x, weight, eps, offset, out, delta, rows):
         self._count("rms_norm")
+        if delta is not None and delta.dim() == 3:
+            total = delta[0].to(torch.float32)
+            for p in range(1, delta.shape[0]):
+                total = total + delta[p]
+            delta = total
         if rows is None:
             v = x.to(self.acc)
             if delta is not None:
@@ -44,11 +50,17 @@ class EmulatedKernels:
         out.copy_(y.to(out.dtype))
 
     def rope_and_cache_write(self, qkv, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads,
-                             head_dim, rotary_dim, page_size):
+                             head_dim, rotary_dim, page_size, parts=None):
         self._count("rope_and_cache_write")
         n = qkv.shape[0]
         heads = num_heads + 2 * num_kv_heads
-        v = qkv.to(self.acc)
+        if parts is not None:
+            total = parts[0]
+            for p in range(1, parts.shape[0]):
+                total = total + parts[p]
+            v = total.to(self.acc)
+        else:
+            v = qkv.to(self.acc)
         if bias is not None:
             v = v + bias.to(self.acc)
         v = v.view(n, heads, head_dim).clone()
@@ -110,9 +122,24 @@ class EmulatedKernels:
     def plan_paged_attention(self, *args):
         return None
 
+    def linear_splits(self, rows, out_features, in_features, dtype):
+        return self.splits
+
     def linear(self, x, weight, out):
         self._count("linear")
+        if out.dim() == 3:
+            k = x.shape[1]
+            edges = [round(i * k / out.shape[0]) for i in range(out.shape[0] + 1)]
+            for p in range(out.shape[0]):
+                a, b = edges[p], edges[p + 1]
+                out[p].copy_((x[:, a:b].to(self.acc) @ weight[:, a:b].to(self.acc).T).to(out.dtype))
+            return
         out.copy_((x.to(self.acc) @ weight.to(self.acc).T).to(out.dtype))
+
+    def gated_linear(self, x, weight, out, activation, scratch):
+        self._count("gated_linear")
+        gu = (x.to(self.acc) @ weight.to(self.acc).T)
+        self.gated_activation(gu, out, activation)
 
     def gated_activation(self, gate_up, out, activation):
         self._count("gated_activation")

@@ -63,3 +63,17 @@ def test_mixed_trace_reuses_pages(model_folders):
     assert max(len(s["entries"]) for s in trace) == 4
     assert any(len(e["tokens"]) > 1 for s in trace for e in s["entries"] if len(s["entries"]) > 1)
     assert any(len(e["tokens"]) == 1 for s in trace for e in s["entries"] if len(s["entries"]) > 1)
+
+
+def test_partial_sums_of_split_products_reach_the_consumers(model_folders, plain_logits):
+    """With a product kernel that splits its sums, the stacks must be added by the next norm and by
+    the rotation: same logits."""
+    requests = _requests("C")
+    trace = trace_mixed(requests)
+    emu = EmulatedKernels(splits=3)
+    with ops.use_backend(emu):
+        model = load_model(model_folders["C"], "float32", "cpu")
+        runner = ModelRunner.create(model, num_pages=pages_for_max_tokens(max_live_tokens(trace), 16), page_size=16,
+                                    max_requests=4)
+        got = replay_and_collect(TraceReplayer(runner), trace)
+    compare_with_plain(got, plain_logits["C"], atol=2e-5, rtol=1e-4)

@@ -106,6 +106,48 @@ def test_rope_and_cache_write(dtype, nh, nkv, d, rot, ps, bias):
     assert (vview.permute(0, 3, 1, 2).reshape(pages * ps, -1)[untouched] == 7.0).all()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_norm_and_rotation_add_stacks_of_partial_sums(dtype):
+    torch.manual_seed(7)
+    n, hidden = 6, 200
+    x = torch.randn(n, hidden, device=DEV)
+    w = torch.randn(hidden, device=DEV) * 0.1
+    stack = torch.randn(3, n, hidden, device=DEV)
+    out = torch.zeros(n, hidden, device=DEV, dtype=dtype)
+    x_ref, out_ref = x.clone(), out.clone()
+    ops.rms_norm(x, w, 1e-6, 1.0, out, delta=stack)
+    ops.rms_norm(x_ref, w, 1e-6, 1.0, out_ref, delta=((stack[0] + stack[1]) + stack[2]))
+    assert torch.equal(x, x_ref) and torch.equal(out, out_ref)
+    rows = torch.tensor([4, 0], device=DEV, dtype=torch.int32)
+    o2, o2_ref = torch.zeros(2, hidden, device=DEV, dtype=dtype), torch.zeros(2, hidden, device=DEV, dtype=dtype)
+    ops.rms_norm(x, w, 1e-6, 1.0, o2, delta=stack, rows=rows)
+    ops.rms_norm(x, w, 1e-6, 1.0, o2_ref, delta=((stack[0] + stack[1]) + stack[2]), rows=rows)
+    assert torch.equal(o2, o2_ref)
+    # rotation: the sum of the parts replaces the row
+    nh, nkv, d, ps = 3, 1, 40, 8
+    width = (nh + 2 * nkv) * d
+    parts = torch.randn(4, n, width, device=DEV)
+    summed = (((parts[0] + parts[1]) + parts[2]) + parts[3]).to(dtype)
+    positions = torch.arange(n, device=DEV, dtype=torch.int32) * 3
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, 24, 2, dtype=torch.float32) / 24))).to(DEV)
+    slots = torch.arange(n, device=DEV, dtype=torch.int32)
+    kw = dict(num_heads=nh, num_kv_heads=nkv, head_dim=d, page_size=ps)
+    for bias in (None, torch.randn(width, device=DEV) * 0.1):
+        qkv = torch.full((n, width), 9.0, device=DEV, dtype=dtype)
+        cache, cache_ref = (torch.zeros(2, 2, nkv, ps * d, device=DEV, dtype=dtype) for _ in range(2))
+        ops.rope_and_cache_write(qkv, bias, positions, inv_freq, slots, cache, parts=parts, **kw)
+        ref = summed.clone()
+        if dtype == torch.float32:
+            ops.rope_and_cache_write(ref, bias, positions, inv_freq, slots, cache_ref, **kw)
+            assert torch.equal(qkv, ref) and torch.equal(cache, cache_ref)
+        else:
+            # the parts are added in float32 and rounded once, after the rotation
+            with ops.use_backend(EmulatedKernels(precise=True)):
+                ops.rope_and_cache_write(ref, bias, positions, inv_freq, slots, cache_ref, parts=parts, **kw)
+            close(qkv, ref, dtype)
+            close(cache, cache_ref, dtype)
+
+
 def test_rope_position_zero_is_identity_and_no_cache():
     nh, nkv, d = 2, 1, 16
     qkv = torch.randn(3, (nh + 2 * nkv) * d, device=DEV)
@@ -245,6 +287,43 @@ def test_linear(dtype, m, n, k):
         torch.manual_seed(4)
         g, r = both("linear", make, dtype)
         close(g[2], r[2], out_dtype, f"product to {out_dtype}")
+
+
+@pytest.mark.parametrize("m,n,k", [(8, 2048, 16384), (5, 2560, 2048), (64, 1000, 1024), (1, 777, 512)])
+def test_linear_leaves_partial_sums_to_the_caller(m, n, k):
+    torch.manual_seed(8)
+    x = torch.randn(m, k, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(n, k, device=DEV) / math.sqrt(k)).to(torch.bfloat16)
+    s = ops.linear_splits(m, n, k, torch.bfloat16)
+    whole = torch.zeros(m, n, device=DEV)
+    ops.linear(x, w, whole)
+    if s == 1:
+        with pytest.raises(ops.KernelShapeError):
+            ops.linear(x, w, torch.zeros(2, m, n, device=DEV))
+        return
+    stack = torch.full((s, m, n), 7.0, device=DEV)
+    ops.linear(x, w, stack)
+    total = stack[0].clone()
+    for p in range(1, s):
+        total += stack[p]
+    assert torch.equal(total, whole), "the partial sums add up, in order, to what the kernel gives unsplit"
+    close(whole, x.double() @ w.double().T, torch.float32, "product")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("act", ["gelu_tanh", "silu"])
+@pytest.mark.parametrize("m,inter,k", [(8, 16384, 2048), (3, 250, 96), (64, 777, 128), (100, 384, 96), (17, 112, 80)])
+def test_gated_linear(dtype, act, m, inter, k):
+    torch.manual_seed(9)
+
+    def make():
+        x = torch.randn(m, k, device=DEV).to(dtype)
+        w = (torch.randn(2 * inter, k, device=DEV) / math.sqrt(k)).to(dtype)
+        return [x, w, torch.zeros(m, inter, device=DEV, dtype=dtype), act, torch.zeros(m, 2 * inter, device=DEV, dtype=dtype)], {}
+
+    torch.manual_seed(9)
+    g, r = both("gated_linear", make, dtype)
+    close(g[2], r[2], dtype)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

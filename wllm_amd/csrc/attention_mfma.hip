@@ -263,32 +263,33 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
 // Combines the partial results of a (segment, key/value head) whose keys were split over workgroups.
 // reduce items: seg, kvh, first partial slot, number of splits.
 template <int HD>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(HD)
 attention_reduce_kernel(const int* __restrict__ reduce_items, const float* __restrict__ partial_o,
                         const float* __restrict__ partial_ml, const int* __restrict__ seg_q_start,
                         const int* __restrict__ seg_q_len, bf16* __restrict__ out, int num_heads, int num_kv_heads,
                         float scale_log2e) {
+    // one workgroup per (item, row); one thread per element of the head; the loads of the
+    // splits do not depend on each other
     const int* item = reduce_items + static_cast<size_t>(blockIdx.x) * 4;
     const int seg = item[0], kvh = item[1], first = item[2], splits = item[3];
     if (seg < 0) return;
     const int group = num_heads / num_kv_heads;
-    const int rows = seg_q_len[seg] * group;      // at most 16
-    const int q_start = seg_q_start[seg];
-    for (int idx = threadIdx.x; idx < rows * HD; idx += blockDim.x) {
-        const int r = idx / HD, d = idx % HD;
-        float m = -INFINITY;
-        for (int s = 0; s < splits; ++s) m = fmaxf(m, partial_ml[(static_cast<size_t>(first + s) * kRowsPerTile + r) * 2]);
-        float num = 0.f, den = 0.f;
-        for (int s = 0; s < splits; ++s) {
-            const size_t prow = static_cast<size_t>(first + s) * kRowsPerTile + r;
-            const float ms = partial_ml[prow * 2];
-            const float f = ms == -INFINITY ? 0.f : exp2f((ms - m) * scale_log2e);
-            num = fmaf(partial_o[prow * HD + d], f, num);
-            den = fmaf(partial_ml[prow * 2 + 1], f, den);
-        }
-        const int tok = r / group, head = kvh * group + r % group;
-        out[(static_cast<size_t>(q_start + tok) * num_heads + head) * HD + d] = from_float<bf16>(num / den);
+    const int r = blockIdx.y, d = threadIdx.x;
+    if (r >= seg_q_len[seg] * group) return;       // at most 16 rows
+    const float* ml = partial_ml + (static_cast<size_t>(first) * kRowsPerTile + r) * 2;
+    const float* po = partial_o + (static_cast<size_t>(first) * kRowsPerTile + r) * HD + d;
+    float m = -INFINITY;
+    for (int s = 0; s < splits; ++s) m = fmaxf(m, ml[static_cast<size_t>(s) * kRowsPerTile * 2]);
+    float num = 0.f, den = 0.f;
+#pragma unroll 4
+    for (int s = 0; s < splits; ++s) {
+        const float ms = ml[static_cast<size_t>(s) * kRowsPerTile * 2];
+        const float f = ms == -INFINITY ? 0.f : exp2f((ms - m) * scale_log2e);
+        num = fmaf(po[static_cast<size_t>(s) * kRowsPerTile * HD], f, num);
+        den = fmaf(ml[static_cast<size_t>(s) * kRowsPerTile * 2 + 1], f, den);
     }
+    const int tok = r / group, head = kvh * group + r % group;
+    out[(static_cast<size_t>(seg_q_start[seg] + tok) * num_heads + head) * HD + d] = from_float<bf16>(num / den);
 }
 
 // Returns 0, a HIP error code, or -1 for sizes these kernels do not take.
@@ -308,7 +309,7 @@ WLLM_API int wllm_paged_attention_mfma(const void* qkv, const void* cache, const
         seg_ctx_len, static_cast<bf16*>(out), partial_o, partial_ml, num_heads, num_kv_heads, page_size, max_pages,  \
         scale_log2e, window)
 #define LAUNCH_R(HD)                                                                                                 \
-    attention_reduce_kernel<HD><<<num_reduce_items, 256, 0, stream>>>(reduce_items, partial_o, partial_ml, seg_q_start, \
+    attention_reduce_kernel<HD><<<dim3(num_reduce_items, kRowsPerTile), HD, 0, stream>>>(reduce_items, partial_o, partial_ml, seg_q_start, \
                                                                       seg_q_len, static_cast<bf16*>(out), num_heads,  \
                                                                       num_kv_heads, scale_log2e)
 #define CASE(HD)                                   \

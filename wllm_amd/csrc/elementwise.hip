@@ -30,11 +30,13 @@ WLLM_API int wllm_embed_lookup(const int* ids, const void* table, int is_bf16, f
 }
 
 // ---- RMS norm: out = v * rsqrt(mean(v^2) + eps) * (offset + w), v = x (+ delta) ------------
-// One workgroup per output row.  Without `rows` the sum x + delta is written back to x.
+// One workgroup per output row.  Without `rows` the sum x + delta is written back to x.  `delta`
+// may be a stack of `splits` partial sums (a product split over K), `split_stride` elements apart;
+// they are added in stack order.
 template <typename TD, typename TO>
-__global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ delta, const float* __restrict__ weight,
-                                const int* __restrict__ rows, TO* __restrict__ out, int hidden, float eps,
-                                float offset) {
+__global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ delta, int splits, size_t split_stride,
+                                const float* __restrict__ weight, const int* __restrict__ rows, TO* __restrict__ out,
+                                int hidden, float eps, float offset) {
     __shared__ float scratch[16];
     const int orow = blockIdx.x;
     const int irow = rows ? rows[orow] : orow;
@@ -44,7 +46,9 @@ __global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ de
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         float v = xr[i];
         if (dr) {
-            v += to_float(dr[i]);
+            float d = to_float(dr[i]);
+            for (int p = 1; p < splits; ++p) d += to_float(dr[p * split_stride + i]);
+            v += d;
             if (!rows) xr[i] = v;
         }
         ss += v * v;
@@ -54,17 +58,22 @@ __global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ de
     TO* o = out + static_cast<size_t>(orow) * hidden;
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         float v = xr[i];
-        if (dr && rows) v += to_float(dr[i]);
+        if (dr && rows) {
+            float d = to_float(dr[i]);
+            for (int p = 1; p < splits; ++p) d += to_float(dr[p * split_stride + i]);
+            v += d;
+        }
         o[i] = from_float<TO>(v * inv * (offset + weight[i]));
     }
 }
 
-WLLM_API int wllm_rms_norm(float* x, const void* delta, int delta_bf16, const float* weight, const int* rows,
-                           void* out, int out_bf16, int num_out_rows, int hidden, float eps, float offset,
-                           hipStream_t stream) {
+WLLM_API int wllm_rms_norm(float* x, const void* delta, int delta_bf16, int splits, long long split_stride,
+                           const float* weight, const int* rows, void* out, int out_bf16, int num_out_rows,
+                           int hidden, float eps, float offset, hipStream_t stream) {
     const int threads = hidden >= 1024 ? 256 : (hidden >= 256 ? 128 : 64);
-#define LAUNCH(TD, TO)                                                                                         \
-    rms_norm_kernel<TD, TO><<<num_out_rows, threads, 0, stream>>>(x, static_cast<const TD*>(delta), weight, rows, \
+#define LAUNCH(TD, TO)                                                                                          \
+    rms_norm_kernel<TD, TO><<<num_out_rows, threads, 0, stream>>>(x, static_cast<const TD*>(delta), splits,      \
+                                                                  static_cast<size_t>(split_stride), weight, rows, \
                                                                   static_cast<TO*>(out), hidden, eps, offset)
     if (delta_bf16 && out_bf16) LAUNCH(bf16, bf16);
     else if (delta_bf16) LAUNCH(bf16, float);
@@ -80,13 +89,23 @@ WLLM_API int wllm_rms_norm(float* x, const void* delta, int delta_bf16, const fl
 // the pair is turned by position * inv_freq[j]; angle, sine and cosine are float32.  Keys go to
 // the cache as [page_size, head_dim], values transposed as [head_dim, page_size].
 template <typename T>
-__global__ void rope_cache_kernel(T* __restrict__ qkv, const float* __restrict__ bias, const int* __restrict__ positions,
+__global__ void rope_cache_kernel(T* __restrict__ qkv, const float* __restrict__ parts, int splits, size_t split_stride,
+                                  const float* __restrict__ bias, const int* __restrict__ positions,
                                   const float* __restrict__ inv_freq, const int* __restrict__ slots,
                                   T* __restrict__ cache, int num_heads, int num_kv_heads, int head_dim, int rotary_dim,
                                   int page_size, long long num_pages) {
     const int token = blockIdx.x;
     const int width = (num_heads + 2 * num_kv_heads) * head_dim;
     T* row = qkv + static_cast<size_t>(token) * width;
+    const float* prow = parts ? parts + static_cast<size_t>(token) * width : nullptr;
+    // a value of the projection: the row itself, or the sum of the partial sums of a split product
+    auto value = [&](int idx) -> float {
+        if (!prow) return to_float(row[idx]);
+        float v = prow[idx];
+        for (int p = 1; p < splits; ++p) v += prow[p * split_stride + idx];
+        return v;
+    };
+    const bool rewrite = bias || prow;      // every element of the row must be written
     const float pos = static_cast<float>(positions[token]);
     const int half = rotary_dim / 2;
     const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * head_dim;
@@ -107,7 +126,7 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, const float* __restrict__
     for (int idx = threadIdx.x; idx < rot_heads * half; idx += blockDim.x) {
         const int head = idx / half, j = idx % half;
         const int ia = head * head_dim + j, ib = ia + half;
-        float a = to_float(row[ia]), b = to_float(row[ib]);
+        float a = value(ia), b = value(ib);
         if (bias) {
             a += bias[ia];
             b += bias[ib];
@@ -125,13 +144,13 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, const float* __restrict__
     }
     // the part of query and key heads that is not rotated
     const int rest = head_dim - rotary_dim;
-    if (rest > 0 && (bias || kpage)) {
+    if (rest > 0 && (rewrite || kpage)) {
         for (int idx = threadIdx.x; idx < rot_heads * rest; idx += blockDim.x) {
             const int head = idx / rest, j = rotary_dim + idx % rest;
             const int i = head * head_dim + j;
             T v = row[i];
-            if (bias) {
-                v = from_float<T>(to_float(v) + bias[i]);
+            if (rewrite) {
+                v = from_float<T>(value(i) + (bias ? bias[i] : 0.f));
                 row[i] = v;
             }
             if (kpage && head >= num_heads)
@@ -139,13 +158,13 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, const float* __restrict__
         }
     }
     // values
-    if (bias || vpage) {
+    if (rewrite || vpage) {
         const int vbase = rot_heads * head_dim;
         for (int idx = threadIdx.x; idx < num_kv_heads * head_dim; idx += blockDim.x) {
             const int head = idx / head_dim, j = idx % head_dim;
             T v = row[vbase + idx];
-            if (bias) {
-                v = from_float<T>(to_float(v) + bias[vbase + idx]);
+            if (rewrite) {
+                v = from_float<T>(value(vbase + idx) + (bias ? bias[vbase + idx] : 0.f));
                 row[vbase + idx] = v;
             }
             if (vpage) vpage[(static_cast<size_t>(head) * head_dim + j) * page_size + off] = v;
@@ -153,18 +172,20 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, const float* __restrict__
     }
 }
 
-WLLM_API int wllm_rope_cache_write(void* qkv, int is_bf16, const float* bias, const int* positions,
-                                   const float* inv_freq, const int* slots, void* cache, long long num_pages, int n,
-                                   int num_heads, int num_kv_heads, int head_dim, int rotary_dim, int page_size,
-                                   hipStream_t stream) {
+WLLM_API int wllm_rope_cache_write(void* qkv, int is_bf16, const float* parts, int splits, long long split_stride,
+                                   const float* bias, const int* positions, const float* inv_freq, const int* slots,
+                                   void* cache, long long num_pages, int n, int num_heads, int num_kv_heads,
+                                   int head_dim, int rotary_dim, int page_size, hipStream_t stream) {
     if (is_bf16)
-        rope_cache_kernel<bf16><<<n, 256, 0, stream>>>(static_cast<bf16*>(qkv), bias, positions, inv_freq, slots,
-                                                       static_cast<bf16*>(cache), num_heads, num_kv_heads, head_dim,
-                                                       rotary_dim, page_size, num_pages);
+        rope_cache_kernel<bf16><<<n, 256, 0, stream>>>(static_cast<bf16*>(qkv), parts, splits,
+                                                       static_cast<size_t>(split_stride), bias, positions, inv_freq,
+                                                       slots, static_cast<bf16*>(cache), num_heads, num_kv_heads,
+                                                       head_dim, rotary_dim, page_size, num_pages);
     else
-        rope_cache_kernel<float><<<n, 256, 0, stream>>>(static_cast<float*>(qkv), bias, positions, inv_freq, slots,
-                                                        static_cast<float*>(cache), num_heads, num_kv_heads, head_dim,
-                                                        rotary_dim, page_size, num_pages);
+        rope_cache_kernel<float><<<n, 256, 0, stream>>>(static_cast<float*>(qkv), parts, splits,
+                                                        static_cast<size_t>(split_stride), bias, positions, inv_freq,
+                                                        slots, static_cast<float*>(cache), num_heads, num_kv_heads,
+                                                        head_dim, rotary_dim, page_size, num_pages);
     return launch_status();
 }
 

@@ -2,20 +2,35 @@
 #include "common.h"
 
 // ---- argmax: the largest value of a row, the lowest index among equals -------------------------
-__global__ void __launch_bounds__(256) argmax_rows_kernel(const float* __restrict__ logits, int* __restrict__ out,
-                                                         int vocab) {
-    __shared__ float best_v[4];
-    __shared__ int best_i[4];
+constexpr int kArgmaxThreads = 1024;
+
+__device__ __forceinline__ void argmax_take(float v, int i, float& bv, int& bi) {
+    // NaN never wins; among equals the lowest index
+    if (v > bv || (v == bv && i < bi) || bi == 0x7fffffff) {
+        bv = v == v ? v : -INFINITY;
+        bi = i;
+    }
+}
+
+__global__ void __launch_bounds__(kArgmaxThreads) argmax_rows_kernel(const float* __restrict__ logits,
+                                                                   int* __restrict__ out, int vocab) {
+    __shared__ float best_v[kArgmaxThreads / kWave];
+    __shared__ int best_i[kArgmaxThreads / kWave];
     const float* row = logits + static_cast<size_t>(blockIdx.x) * vocab;
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-        const float v = row[i];
-        // NaN never wins; ascending i per thread, so ">" keeps the lowest index
-        if (v > bv || bi == 0x7fffffff) {
-            bv = v == v ? v : -INFINITY;
-            bi = i;
+    if (vocab % 4 == 0) {
+        // rows are 16-byte aligned: four values per load
+        const float4* row4 = reinterpret_cast<const float4*>(row);
+        for (int q = threadIdx.x; q < vocab / 4; q += blockDim.x) {
+            const float4 v = row4[q];
+            argmax_take(v.x, 4 * q, bv, bi);
+            argmax_take(v.y, 4 * q + 1, bv, bi);
+            argmax_take(v.z, 4 * q + 2, bv, bi);
+            argmax_take(v.w, 4 * q + 3, bv, bi);
         }
+    } else {
+        for (int i = threadIdx.x; i < vocab; i += blockDim.x) argmax_take(row[i], i, bv, bi);
     }
 #pragma unroll
     for (int off = kWave / 2; off > 0; off >>= 1) {
@@ -33,7 +48,7 @@ __global__ void __launch_bounds__(256) argmax_rows_kernel(const float* __restric
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int w = 1; w < 4; ++w)
+        for (int w = 1; w < kArgmaxThreads / kWave; ++w)
             if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) {
                 bv = best_v[w];
                 bi = best_i[w];
@@ -43,7 +58,7 @@ __global__ void __launch_bounds__(256) argmax_rows_kernel(const float* __restric
 }
 
 WLLM_API int wllm_argmax_rows(const float* logits, int* out, int rows, int vocab, hipStream_t stream) {
-    argmax_rows_kernel<<<rows, 256, 0, stream>>>(logits, out, vocab);
+    argmax_rows_kernel<<<rows, kArgmaxThreads, 0, stream>>>(logits, out, vocab);
     return launch_status();
 }
 

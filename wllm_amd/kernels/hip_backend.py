@@ -23,10 +23,11 @@ def _ptr(t):
 
 _SIGNATURES = {
     "wllm_embed_lookup": [c_void_p, c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
-    "wllm_rms_norm": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float,
-                      c_void_p],
-    "wllm_rope_cache_write": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong, c_int,
-                              c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "wllm_rms_norm": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                      c_float, c_float, c_void_p],
+    "wllm_rope_cache_write": [c_void_p, c_int, c_void_p, c_int, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p,
+                              c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "wllm_gemm_skinny_gated": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_gated_activation": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_paged_attention_generic": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
@@ -78,16 +79,21 @@ class HipBackend:
 
     def rms_norm(self, x, weight, eps, offset, out, delta, rows):
         self._on_gpu(x, weight, out, delta, rows)
+        splits, stride = 1, 0
+        if delta is not None and delta.dim() == 3:
+            splits, stride = delta.shape[0], delta.shape[1] * delta.shape[2]
         self._check(self.lib.wllm_rms_norm(
-            _ptr(x), _ptr(delta), int(delta is not None and delta.dtype == torch.bfloat16), _ptr(weight), _ptr(rows),
-            _ptr(out), int(out.dtype == torch.bfloat16), out.shape[0], x.shape[1], eps, offset, self._stream()),
-            "rms_norm")
+            _ptr(x), _ptr(delta), int(delta is not None and delta.dtype == torch.bfloat16), splits, stride,
+            _ptr(weight), _ptr(rows), _ptr(out), int(out.dtype == torch.bfloat16), out.shape[0], x.shape[1], eps,
+            offset, self._stream()), "rms_norm")
 
     def rope_and_cache_write(self, qkv, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads, head_dim,
-                             rotary_dim, page_size):
-        self._on_gpu(qkv, bias, positions, inv_freq, slots, cache)
+                             rotary_dim, page_size, parts=None):
+        self._on_gpu(qkv, bias, positions, inv_freq, slots, cache, parts)
+        splits, stride = (parts.shape[0], parts.shape[1] * parts.shape[2]) if parts is not None else (0, 0)
         self._check(self.lib.wllm_rope_cache_write(
-            _ptr(qkv), int(qkv.dtype == torch.bfloat16), _ptr(bias), _ptr(positions), _ptr(inv_freq), _ptr(slots),
+            _ptr(qkv), int(qkv.dtype == torch.bfloat16), _ptr(parts), splits, stride, _ptr(bias), _ptr(positions),
+            _ptr(inv_freq), _ptr(slots),
             _ptr(cache), cache.shape[0] if cache is not None else 0, qkv.shape[0], num_heads, num_kv_heads, head_dim,
             rotary_dim, page_size, self._stream()), "rope_and_cache_write")
 
@@ -171,12 +177,26 @@ class HipBackend:
             self._gemm_partials = torch.empty(self.GEMM_PARTIAL_FLOATS, dtype=torch.float32, device=device)
         return self._gemm_partials
 
+    SKINNY_CHUNK = {1: 1024, 2: 512, 3: 256, 4: 256}     # K elements of x staged at a time, by row tiles
+
+    @staticmethod
+    def skinny_takes(dtype, rows: int, in_features: int) -> bool:
+        return dtype == torch.bfloat16 and rows <= 64 and in_features % 32 == 0
+
+    def linear_splits(self, rows, out_features, in_features, dtype) -> int:
+        if self.skinny_takes(dtype, rows, in_features):
+            return self.skinny_split(out_features, in_features)
+        return 1
+
     def _skinny(self, x, weight, out) -> None:
         m, k = x.shape
         n = weight.shape[0]
         splits = self.skinny_split(n, k)
-        mt = -(-m // 16)
-        chunk = {1: 1024, 2: 512, 3: 256, 4: 256}[mt]
+        chunk = self.SKINNY_CHUNK[-(-m // 16)]
+        if out.dim() == 3:      # the caller adds the partial sums later
+            self._check(self.lib.wllm_gemm_skinny(_ptr(x), _ptr(weight), c_void_p(0), 0, _ptr(out), m, n, k, splits,
+                                                  chunk, self._stream()), "linear (few rows, partial sums)")
+            return
         partial = self._gemm_partial(splits * m * n, x.device) if splits > 1 else None
         self._check(self.lib.wllm_gemm_skinny(_ptr(x), _ptr(weight), _ptr(out), int(out.dtype == torch.bfloat16),
                                               _ptr(partial), m, n, k, splits, chunk, self._stream()),
@@ -186,9 +206,12 @@ class HipBackend:
         self._on_gpu(x, weight, out)
         m, k = x.shape
         if x.dtype == torch.bfloat16:
-            if k % 32 == 0 and (m <= 64 or out.dtype == torch.float32):
-                # few rows: the weight-streaming kernel; float32 results from bfloat16 operands
-                # (logits) take it in blocks of 64 rows
+            if self.skinny_takes(x.dtype, m, k):
+                self._skinny(x, weight, out)
+                return
+            if k % 32 == 0 and out.dtype == torch.float32:
+                # float32 results from bfloat16 operands (logits at many rows): the few-row kernel
+                # in blocks of 64 rows
                 for r in range(0, m, 64):
                     self._skinny(x[r:r + 64], weight, out[r:r + 64])
                 return
@@ -199,6 +222,17 @@ class HipBackend:
         self._check(self.lib.wllm_gemm_generic(
             _ptr(x), _ptr(weight), int(x.dtype == torch.bfloat16), _ptr(out), int(out.dtype == torch.bfloat16),
             x.shape[0], weight.shape[0], x.shape[1], self._stream()), "linear")
+
+    def gated_linear(self, x, weight, out, activation, scratch):
+        self._on_gpu(x, weight, out, scratch)
+        m, k = x.shape
+        if self.skinny_takes(x.dtype, m, k):
+            self._check(self.lib.wllm_gemm_skinny_gated(
+                _ptr(x), _ptr(weight), _ptr(out), m, out.shape[1], k, 0 if activation == "gelu_tanh" else 1,
+                self.SKINNY_CHUNK[-(-m // 16)], self._stream()), "gated_linear (few rows, matrix cores)")
+            return
+        self.linear(x, weight, scratch)
+        self.gated_activation(scratch, out, activation)
 
     def gated_activation(self, gate_up, out, activation):
         self._on_gpu(gate_up, out)

@@ -75,8 +75,9 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, offset: float, o
              delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None) -> None:
     """out = x * rsqrt(mean(x^2) + eps) * (offset + weight), all in float32, cast to out's dtype.
 
-    x float32 [n, H]; weight float32 [H]; out T [m, H].  With `delta` (T [n, H]) the
-    row normalised is x + delta.  Without `rows`, m = n and the sum is written back
+    x float32 [n, H]; weight float32 [H]; out T [m, H].  With `delta` (T [n, H], or a stack
+    float32 [S, n, H] of partial sums that are added in order) the row normalised is
+    x + delta.  Without `rows`, m = n and the sum is written back
     to x (the residual stream moves on).  With `rows` (int32 [m]) only those rows are
     read, x is left alone and out[i] belongs to row rows[i].
     """
@@ -85,7 +86,11 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, offset: float, o
     n, h = x.shape
     _dense(weight, "weight", torch.float32, (h,))
     if delta is not None:
-        _dense(delta, "delta", _ACT, (n, h))
+        if delta.dim() == 3:
+            _dense(delta, "delta", torch.float32, (delta.shape[0], n, h))
+            _need(delta.shape[0] >= 1, "delta: an empty stack")
+        else:
+            _dense(delta, "delta", _ACT, (n, h))
     m = n
     if rows is not None:
         _dense(rows, "rows", torch.int32)
@@ -99,7 +104,7 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, offset: float, o
 def rope_and_cache_write(qkv: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
                          inv_freq: Optional[torch.Tensor], slots: Optional[torch.Tensor],
                          cache: Optional[torch.Tensor], *, num_heads: int, num_kv_heads: int,
-                         head_dim: int, page_size: int) -> None:
+                         head_dim: int, page_size: int, parts: Optional[torch.Tensor] = None) -> None:
     """Adds `bias`, rotates queries and keys in place and stores keys and values in pages.
 
     qkv T [n, (num_heads + 2*num_kv_heads) * head_dim]: queries, then keys, then values.
@@ -109,7 +114,9 @@ def rope_and_cache_write(qkv: torch.Tensor, bias: Optional[torch.Tensor], positi
     float32.  slots int32 [n]: page * page_size + offset for each token; cache
     T [pages, 2, num_kv_heads, page_size*head_dim] holds a page's keys as [page_size,
     head_dim] and its values as [head_dim, page_size].  slots and cache None: nothing is
-    stored (the layer reads another layer's cache).
+    stored (the layer reads another layer's cache).  `parts` (float32 [S, n, width]): the
+    projection arrives as a stack of partial sums; their sum in order replaces what qkv holds
+    on entry.
     """
     width = (num_heads + 2 * num_kv_heads) * head_dim
     _dense(qkv, "qkv", _ACT)
@@ -117,6 +124,9 @@ def rope_and_cache_write(qkv: torch.Tensor, bias: Optional[torch.Tensor], positi
     n = qkv.shape[0]
     if bias is not None:
         _dense(bias, "bias", torch.float32, (width,))
+    if parts is not None:
+        _need(parts.dim() == 3 and parts.shape[0] >= 1, "parts: expected [S, n, width]")
+        _dense(parts, "parts", torch.float32, (parts.shape[0], n, width))
     _dense(positions, "positions", torch.int32, (n,))
     rotary_dim = 0
     if inv_freq is not None:
@@ -132,7 +142,7 @@ def rope_and_cache_write(qkv: torch.Tensor, bias: Optional[torch.Tensor], positi
               f"cache: shape {tuple(cache.shape)}, expected [pages, 2, {num_kv_heads}, {page_size * head_dim}]")
     if n:
         backend().rope_and_cache_write(qkv, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads,
-                                       head_dim, rotary_dim, page_size)
+                                       head_dim, rotary_dim, page_size, parts)
 
 
 def paged_attention(qkv: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor,
@@ -184,15 +194,28 @@ def plan_paged_attention(host_q_len, host_ctx_len, *, num_heads: int, num_kv_hea
                                           int(window), dtype, device)
 
 
+def linear_splits(rows: int, out_features: int, in_features: int, dtype: torch.dtype) -> int:
+    """Into how many partial sums over the input axis the product kernel for these sizes splits
+    its work (1: it does not).  A caller that can take the sum later (the next norm, the rotation)
+    hands `linear` an output of shape [S, rows, out_features] and saves the pass that adds them."""
+    return int(backend().linear_splits(rows, out_features, in_features, dtype))
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> None:
-    """out = x @ weight^T.  x T [m, k]; weight T [n, k]; out T or float32 [m, n].
-    Products of bfloat16 accumulate in float32; float32 stays float32 throughout."""
+    """out = x @ weight^T.  x T [m, k]; weight T [n, k]; out T or float32 [m, n], or float32
+    [S, m, n] with S = linear_splits(m, n, k, T): then the S slices are partial sums whose sum in
+    order is the product.  Products of bfloat16 accumulate in float32; float32 stays float32."""
     _dense(x, "x", _ACT)
     _need(x.dim() == 2, "x: expected [rows, in]")
     _dense(weight, "weight", x.dtype)
     _need(weight.dim() == 2 and weight.shape[1] == x.shape[1],
           f"weight: shape {tuple(weight.shape)}, expected [out, {x.shape[1]}]")
-    _dense(out, "out", (x.dtype, torch.float32), (x.shape[0], weight.shape[0]))
+    if out.dim() == 3:
+        s = linear_splits(x.shape[0], weight.shape[0], x.shape[1], x.dtype)
+        _dense(out, "out", torch.float32, (s, x.shape[0], weight.shape[0]))
+        _need(s > 1, "out: a stack of partial sums where the product is not split")
+    else:
+        _dense(out, "out", (x.dtype, torch.float32), (x.shape[0], weight.shape[0]))
     if x.shape[0]:
         backend().linear(x, weight, out)
 
@@ -208,6 +231,23 @@ def gated_activation(gate_up: torch.Tensor, out: torch.Tensor, activation: str) 
     _dense(out, "out", gate_up.dtype, (gate_up.shape[0], gate_up.shape[1] // 2))
     if gate_up.shape[0]:
         backend().gated_activation(gate_up, out, activation)
+
+
+def gated_linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, activation: str,
+                 scratch: torch.Tensor) -> None:
+    """out = act(x @ Wg^T) * (x @ Wu^T) with weight = [Wg; Wu] stacked, T [2I, k]; x T [m, k];
+    out T [m, I]; scratch T [m, 2I] may be used for the unfused product."""
+    _need(activation in ACTIVATIONS, f"activation {activation!r}: expected one of {ACTIVATIONS}")
+    _dense(x, "x", _ACT)
+    _need(x.dim() == 2, "x: expected [rows, in]")
+    _dense(weight, "weight", x.dtype)
+    _need(weight.dim() == 2 and weight.shape[1] == x.shape[1] and weight.shape[0] % 2 == 0,
+          f"weight: shape {tuple(weight.shape)}, expected [2*intermediate, {x.shape[1]}]")
+    inter = weight.shape[0] // 2
+    _dense(out, "out", x.dtype, (x.shape[0], inter))
+    _dense(scratch, "scratch", x.dtype, (x.shape[0], 2 * inter))
+    if x.shape[0]:
+        backend().gated_linear(x, weight, out, activation, scratch)
 
 
 def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> None:

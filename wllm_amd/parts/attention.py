@@ -17,6 +17,7 @@ import torch
 
 from wllm_amd.cache.manager import CacheNeed
 from wllm_amd.kernels import ops
+from wllm_amd.parts.common import project
 from wllm_amd.parts.registry import build_position, register_mixer
 from wllm_amd.parts.specs import AttentionSpec
 from wllm_amd.weights.checkpoint import ExpectedTensor
@@ -78,12 +79,15 @@ class PagedAttention:
         s = self.spec
         n = h.shape[0]
         qkv = ctx.buffer("qkv", (n, self.qkv_width), h.dtype)
-        ops.linear(h, self.w_qkv, qkv)
+        # where the product kernel splits its sums, the rotation kernel adds them as it reads
+        projected = project(ctx, "qkv", h, self.w_qkv, qkv)
+        parts = projected if projected.dim() == 3 else None
         pages = ctx.pages(entry)
         ops.rope_and_cache_write(
             qkv, self.b_qkv, ctx.positions, self.position.inv_freq,
             pages.slots if pages.writes else None, pages.storage if pages.writes else None,
-            num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim, page_size=pages.page_size)
+            num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim, page_size=pages.page_size,
+            parts=parts)
         attn = ctx.buffer("attn", (n, s.num_heads * s.head_dim), h.dtype)
         ops.paged_attention(
             qkv, pages.storage, pages.block_tables, ctx.token_segment, ctx.seg_q_start, ctx.seg_q_len,
@@ -92,6 +96,5 @@ class PagedAttention:
             max_q_len=ctx.max_q_len, max_ctx_len=ctx.max_ctx_len,
             plan=ctx.attention_plan(num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim,
                                     page_size=pages.page_size, window=s.window or 0))
-        y = ctx.buffer("mixer_out", (n, s.hidden_size), h.dtype)
-        ops.linear(attn, self.w_o, y)
-        return y
+        # the next norm adds the contribution to the residual stream, partial sums and all
+        return project(ctx, "mixer_out", attn, self.w_o)

@@ -7,6 +7,7 @@ from __future__ import annotations
 import torch
 
 from wllm_amd.kernels import ops
+from wllm_amd.parts.common import project
 from wllm_amd.parts.registry import register_feed_forward
 from wllm_amd.parts.specs import GatedMLPSpec
 from wllm_amd.weights.checkpoint import ExpectedTensor
@@ -38,9 +39,6 @@ class GatedMLP:
         s = self.spec
         n = h.shape[0]
         gate_up = ctx.buffer("gate_up", (n, 2 * s.intermediate_size), h.dtype)
-        ops.linear(h, self.w_gate_up, gate_up)
         act = ctx.buffer("ffn_act", (n, s.intermediate_size), h.dtype)
-        ops.gated_activation(gate_up, act, s.activation)
-        y = ctx.buffer("ffn_out", (n, s.hidden_size), h.dtype)
-        ops.linear(act, self.w_down, y)
-        return y
+        ops.gated_linear(h, self.w_gate_up, act, s.activation, gate_up)
+        return project(ctx, "ffn_out", act, self.w_down)
