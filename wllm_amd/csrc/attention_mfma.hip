@@ -113,23 +113,55 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
         for (int blk = blk_first + ks; blk < blk_end; blk += key_splits) {
             const int kbase = blk * kKeysPerBlock;
             const bool edge = kbase < seg_lo || kbase + kKeysPerBlock > ctx;
+            // ---- addresses of the keys and values of this block; all loads are issued before
+            //      the first product needs one, so the block costs one trip to memory ----
+            const bf16* krow[2];
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2) {
+                // which key the A row i of the score product is; see the header for why
+                int kk = kbase + (V16 ? 8 * (i / 4) + 4 * t2 + (i % 4) : 16 * t2 + i);
+                kk = min(kk, ctx - 1);
+                const int page = table[kk / page_size];
+                krow[t2] = cache + static_cast<size_t>(page) * page_elems + k_off +
+                           static_cast<size_t>(kk % page_size) * HD + 8 * g;
+            }
+            int vpage0, vslot0, vpage1 = 0, vslot1 = 0;
+            if (V16) {
+                const int kk = min(kbase + 8 * g, ctx - 1) & ~7;
+                vpage0 = table[kk / page_size];
+                vslot0 = kk % page_size;
+            } else {
+                const int ka = min(kbase + 4 * g, ctx - 1) & ~3, kb = min(kbase + 16 + 4 * g, ctx - 1) & ~3;
+                vpage0 = table[ka / page_size];
+                vslot0 = ka % page_size;
+                vpage1 = table[kb / page_size];
+                vslot1 = kb % page_size;
+            }
+            const bf16* vbase0 = cache + static_cast<size_t>(vpage0) * page_elems + v_off + vslot0;
+            const bf16* vbase1 = cache + static_cast<size_t>(vpage1) * page_elems + v_off + vslot1;
+            Pack16 ka_[2][DC], va_[DT];
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+                for (int c = 0; c < DC; ++c) ka_[t2][c].u = *reinterpret_cast<const uint4*>(krow[t2] + c * 32);
+#pragma unroll
+            for (int t = 0; t < DT; ++t) {
+                const size_t drow = static_cast<size_t>(t * 16 + i) * page_size;
+                if (V16) {
+                    va_[t].u = *reinterpret_cast<const uint4*>(vbase0 + drow);
+                } else {
+                    va_[t].half[0] = *reinterpret_cast<const uint2*>(vbase0 + drow);
+                    va_[t].half[1] = *reinterpret_cast<const uint2*>(vbase1 + drow);
+                }
+            }
             // ---- scores of two tiles of 16 keys ----
             float4_t s[2];
 #pragma unroll
             for (int t2 = 0; t2 < 2; ++t2) {
-                // which key the A row i of this product is; see the header for why
-                int kk = kbase + (V16 ? 8 * (i / 4) + 4 * t2 + (i % 4) : 16 * t2 + i);
-                kk = min(kk, ctx - 1);
-                const int page = table[kk / page_size];
-                const bf16* krow = cache + static_cast<size_t>(page) * page_elems + k_off +
-                                   static_cast<size_t>(kk % page_size) * HD;
                 float4_t sc = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int c = 0; c < DC; ++c) {
-                    Pack16 a;
-                    a.u = *reinterpret_cast<const uint4*>(krow + c * 32 + 8 * g);
-                    sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qreg[c], sc, 0, 0, 0);
-                }
+                for (int c = 0; c < DC; ++c)
+                    sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka_[t2][c].v, qreg[c], sc, 0, 0, 0);
                 s[t2] = sc;
             }
             // ---- mask, running maximum, probabilities ----
@@ -160,30 +192,9 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
             l_run = l_run * alpha + psum;      // per lane; the four lanes of a row are added at the end
             m_run = m_new;
             // ---- out^T += V^T . P^T ----
-            int vpage0, vslot0, vpage1 = 0, vslot1 = 0;
-            if (V16) {
-                const int kk = min(kbase + 8 * g, ctx - 1) & ~7;
-                vpage0 = table[kk / page_size];
-                vslot0 = kk % page_size;
-            } else {
-                const int ka = min(kbase + 4 * g, ctx - 1) & ~3, kb = min(kbase + 16 + 4 * g, ctx - 1) & ~3;
-                vpage0 = table[ka / page_size];
-                vslot0 = ka % page_size;
-                vpage1 = table[kb / page_size];
-                vslot1 = kb % page_size;
-            }
-            const bf16* vbase0 = cache + static_cast<size_t>(vpage0) * page_elems + v_off + vslot0;
-            const bf16* vbase1 = cache + static_cast<size_t>(vpage1) * page_elems + v_off + vslot1;
 #pragma unroll
             for (int t = 0; t < DT; ++t) {
-                const size_t drow = static_cast<size_t>(t * 16 + i) * page_size;
-                Pack16 a;
-                if (V16) {
-                    a.u = *reinterpret_cast<const uint4*>(vbase0 + drow);
-                } else {
-                    a.half[0] = *reinterpret_cast<const uint2*>(vbase0 + drow);
-                    a.half[1] = *reinterpret_cast<const uint2*>(vbase1 + drow);
-                }
+                Pack16 a = va_[t];
                 if (edge) {
                     // keys outside the request (stale slots, pages given back) may hold anything,
                     // NaN included; 0 * NaN would poison the sum, so they are cleared

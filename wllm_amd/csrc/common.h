@@ -52,5 +52,19 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
     return total;
 }
 
+// The sum of `splits` partial sums `stride` elements apart, added in stack order.  The loads of
+// eight slices are issued before the first addition needs one.
+__device__ __forceinline__ float stack_sum(const float* __restrict__ p, int splits, size_t stride) {
+    float total = p[0];
+    for (int s0 = 1; s0 < splits; s0 += 8) {
+        float t[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) t[j] = s0 + j < splits ? p[(s0 + j) * stride] : 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) total += t[j];
+    }
+    return total;
+}
+
 // The error a launch left, as an int for the caller (0 = hipSuccess).
 __host__ inline int launch_status() { return static_cast<int>(hipGetLastError()); }

@@ -33,6 +33,13 @@ WLLM_API int wllm_embed_lookup(const int* ids, const void* table, int is_bf16, f
 // One workgroup per output row.  Without `rows` the sum x + delta is written back to x.  `delta`
 // may be a stack of `splits` partial sums (a product split over K), `split_stride` elements apart;
 // they are added in stack order.
+__device__ __forceinline__ float delta_value(const bf16* p, int, size_t) { return to_float(*p); }
+__device__ __forceinline__ float delta_value(const float* p, int splits, size_t stride) {
+    return splits > 1 ? stack_sum(p, splits, stride) : *p;
+}
+
+constexpr int kNormPerThread = 8;    // elements a thread may keep in registers between the passes
+
 template <typename TD, typename TO>
 __global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ delta, int splits, size_t split_stride,
                                 const float* __restrict__ weight, const int* __restrict__ rows, TO* __restrict__ out,
@@ -42,35 +49,56 @@ __global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ de
     const int irow = rows ? rows[orow] : orow;
     float* xr = x + static_cast<size_t>(irow) * hidden;
     const TD* dr = delta ? delta + static_cast<size_t>(irow) * hidden : nullptr;
+    TO* o = out + static_cast<size_t>(orow) * hidden;
+    const bool in_registers = hidden <= static_cast<int>(blockDim.x) * kNormPerThread;
+    float keep[kNormPerThread];
     float ss = 0.f;
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-        float v = xr[i];
-        if (dr) {
-            float d = to_float(dr[i]);
-            for (int p = 1; p < splits; ++p) d += to_float(dr[p * split_stride + i]);
-            v += d;
-            if (!rows) xr[i] = v;
+    if (in_registers) {
+#pragma unroll
+        for (int e = 0; e < kNormPerThread; ++e) {
+            const int i = threadIdx.x + e * blockDim.x;
+            float v = 0.f;
+            if (i < hidden) {
+                v = xr[i];
+                if (dr) {
+                    v += delta_value(dr + i, splits, split_stride);
+                    if (!rows) xr[i] = v;
+                }
+            }
+            keep[e] = v;
+            ss += v * v;
         }
-        ss += v * v;
+    } else {
+        for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+            float v = xr[i];
+            if (dr) {
+                v += delta_value(dr + i, splits, split_stride);
+                if (!rows) xr[i] = v;
+            }
+            ss += v * v;
+        }
     }
     ss = block_sum(ss, scratch);
     const float inv = rsqrtf(ss / static_cast<float>(hidden) + eps);
-    TO* o = out + static_cast<size_t>(orow) * hidden;
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-        float v = xr[i];
-        if (dr && rows) {
-            float d = to_float(dr[i]);
-            for (int p = 1; p < splits; ++p) d += to_float(dr[p * split_stride + i]);
-            v += d;
+    if (in_registers) {
+#pragma unroll
+        for (int e = 0; e < kNormPerThread; ++e) {
+            const int i = threadIdx.x + e * blockDim.x;
+            if (i < hidden) o[i] = from_float<TO>(keep[e] * inv * (offset + weight[i]));
         }
-        o[i] = from_float<TO>(v * inv * (offset + weight[i]));
+    } else {
+        for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+            float v = xr[i];
+            if (dr && rows) v += delta_value(dr + i, splits, split_stride);
+            o[i] = from_float<TO>(v * inv * (offset + weight[i]));
+        }
     }
 }
 
 WLLM_API int wllm_rms_norm(float* x, const void* delta, int delta_bf16, int splits, long long split_stride,
                            const float* weight, const int* rows, void* out, int out_bf16, int num_out_rows,
                            int hidden, float eps, float offset, hipStream_t stream) {
-    const int threads = hidden >= 1024 ? 256 : (hidden >= 256 ? 128 : 64);
+    const int threads = hidden >= 4096 ? 1024 : (hidden >= 1024 ? 512 : (hidden >= 256 ? 128 : 64));
 #define LAUNCH(TD, TO)                                                                                          \
     rms_norm_kernel<TD, TO><<<num_out_rows, threads, 0, stream>>>(x, static_cast<const TD*>(delta), splits,      \
                                                                   static_cast<size_t>(split_stride), weight, rows, \
@@ -101,9 +129,7 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, const float* __restrict__
     // a value of the projection: the row itself, or the sum of the partial sums of a split product
     auto value = [&](int idx) -> float {
         if (!prow) return to_float(row[idx]);
-        float v = prow[idx];
-        for (int p = 1; p < splits; ++p) v += prow[p * split_stride + idx];
-        return v;
+        return stack_sum(prow + idx, splits, split_stride);
     };
     const bool rewrite = bias || prow;      // every element of the row must be written
     const float pos = static_cast<float>(positions[token]);
@@ -176,13 +202,15 @@ WLLM_API int wllm_rope_cache_write(void* qkv, int is_bf16, const float* parts, i
                                    const float* bias, const int* positions, const float* inv_freq, const int* slots,
                                    void* cache, long long num_pages, int n, int num_heads, int num_kv_heads,
                                    int head_dim, int rotary_dim, int page_size, hipStream_t stream) {
+    const int pairs = (num_heads + num_kv_heads) * (rotary_dim / 2);
+    const int threads = pairs >= 1024 ? 1024 : (pairs >= 512 ? 512 : 256);
     if (is_bf16)
-        rope_cache_kernel<bf16><<<n, 256, 0, stream>>>(static_cast<bf16*>(qkv), parts, splits,
+        rope_cache_kernel<bf16><<<n, threads, 0, stream>>>(static_cast<bf16*>(qkv), parts, splits,
                                                        static_cast<size_t>(split_stride), bias, positions, inv_freq,
                                                        slots, static_cast<bf16*>(cache), num_heads, num_kv_heads,
                                                        head_dim, rotary_dim, page_size, num_pages);
     else
-        rope_cache_kernel<float><<<n, 256, 0, stream>>>(static_cast<float*>(qkv), parts, splits,
+        rope_cache_kernel<float><<<n, threads, 0, stream>>>(static_cast<float*>(qkv), parts, splits,
                                                         static_cast<size_t>(split_stride), bias, positions, inv_freq,
                                                         slots, static_cast<float*>(cache), num_heads, num_kv_heads,
                                                         head_dim, rotary_dim, page_size, num_pages);

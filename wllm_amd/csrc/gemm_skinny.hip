@@ -45,6 +45,21 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* _
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
 
+    // The weight stream is read in batches of kBatch 16-byte loads per lane; the next batch is
+    // in flight while the products of this one are made, the first before x is staged at all.
+    constexpr int kBatch = 16;
+    const bool live = n0 < N;
+    const int steps = (k_end - k_begin) / 32;
+    const bf16* wp = wrow + k_begin + 8 * g;
+    Frag cur[kBatch], nxt[kBatch];
+    auto fetch = [&](Frag* dst, int step0) {
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u)
+            dst[u].u = (live && step0 + u < steps) ? *reinterpret_cast<const uint4*>(wp + (step0 + u) * 32)
+                                                   : make_uint4(0, 0, 0, 0);
+    };
+    fetch(cur, 0);
+    int step = 0;
     for (int kc = k_begin; kc < k_end; kc += chunk) {
         const int len = min(chunk, k_end - kc);   // a multiple of 32
         const int vecs = len / 8;
@@ -56,34 +71,23 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* _
             xs[m * stride + c] = v;
         }
         __syncthreads();
-        if (n0 < N) {
-            const bf16* wp = wrow + kc + 8 * g;
-            int k = 0;
-            // four weight loads in flight per lane before the first product needs one
-            for (; k + 128 <= len; k += 128) {
-                Frag a[4];
+        for (int k = 0; k < len; k += 32 * kBatch) {
+            const int used = min(kBatch, (len - k) / 32);      // steps of this batch that lie in the chunk
+            fetch(nxt, step + used);
 #pragma unroll
-                for (int u = 0; u < 4; ++u) a[u].u = *reinterpret_cast<const uint4*>(wp + k + 32 * u);
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < kBatch; ++u) {
+                if (k + 32 * u < len) {
 #pragma unroll
                     for (int t = 0; t < MT; ++t) {
                         Frag b;
-                        b.u = xs[(t * 16 + i) * stride + (k + 32 * u) / 8 + g];
-                        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u].v, b.v, acc[t], 0, 0, 0);
+                        b.u = xs[(t * 16 + i) * stride + k / 8 + 4 * u + g];
+                        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[u].v, b.v, acc[t], 0, 0, 0);
                     }
                 }
             }
-            for (; k < len; k += 32) {
-                Frag a;
-                a.u = *reinterpret_cast<const uint4*>(wp + k);
 #pragma unroll
-                for (int t = 0; t < MT; ++t) {
-                    Frag b;
-                    b.u = xs[(t * 16 + i) * stride + k / 8 + g];
-                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc[t], 0, 0, 0);
-                }
-            }
+            for (int u = 0; u < kBatch; ++u) cur[u] = nxt[u];
+            step += used;
         }
     }
     if (n0 >= N) return;
@@ -173,71 +177,94 @@ __device__ __forceinline__ float act_gelu_tanh(float z) {
 }
 __device__ __forceinline__ float act_silu(float z) { return z / (1.f + expf(-z)); }
 
+// A workgroup is 8 wavefronts: 4 tiles of 16 gate rows (with their up rows) times 2 halves of the
+// K axis, so that two wavefronts per SIMD keep loads in flight; the halves are added through shared
+// memory in a fixed order before the activation.
 template <int MT, int ACT>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(512)
 gemm_skinny_gated_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, bf16* __restrict__ out, int M,
                          int inter, int K, int chunk) {
-    extern __shared__ uint4 xs[];
+    extern __shared__ uint4 xs[];                 // two halves of [MT*16][chunk/8 + 1]
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const int i = lane % 16, g = lane / 16;
-    const int n0 = (blockIdx.x * 4 + wave) * 16;
+    const int tile = wave % 4, half = wave / 4;
+    const int n0 = (blockIdx.x * 4 + tile) * 16;
     const int stride = chunk / 8 + 1;
+    const int half_k = K / 2;                     // a multiple of 32
+    const int k_begin = half * half_k;
+    uint4* xh = xs + half * (MT * 16 * stride);
     const int nrow = min(n0 + i, inter - 1);
-    const bf16* grow = w + static_cast<size_t>(nrow) * K;
-    const bf16* urow = w + static_cast<size_t>(inter + nrow) * K;
+    const bf16* gp = w + static_cast<size_t>(nrow) * K + k_begin + 8 * g;
+    const bf16* up = w + static_cast<size_t>(inter + nrow) * K + k_begin + 8 * g;
     float4_t accg[MT], accu[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         accg[t] = float4_t{0.f, 0.f, 0.f, 0.f};
         accu[t] = float4_t{0.f, 0.f, 0.f, 0.f};
     }
-    for (int kc = 0; kc < K; kc += chunk) {
-        const int len = min(chunk, K - kc);
+    constexpr int kBatch = 8;       // per stream; two streams
+    const bool live = n0 < inter;
+    const int steps = half_k / 32;
+    Frag curg[kBatch], curu[kBatch], nxtg[kBatch], nxtu[kBatch];
+    auto fetch = [&](Frag* dg, Frag* du, int step0) {
+#pragma unroll
+        for (int u = 0; u < kBatch; ++u) {
+            const bool ok = live && step0 + u < steps;
+            dg[u].u = ok ? *reinterpret_cast<const uint4*>(gp + (step0 + u) * 32) : make_uint4(0, 0, 0, 0);
+            du[u].u = ok ? *reinterpret_cast<const uint4*>(up + (step0 + u) * 32) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    fetch(curg, curu, 0);
+    int step = 0;
+    const int tid_half = threadIdx.x % 256;
+    for (int kc = 0; kc < half_k; kc += chunk) {
+        const int len = min(chunk, half_k - kc);
         const int vecs = len / 8;
         __syncthreads();
-        for (int idx = threadIdx.x; idx < MT * 16 * vecs; idx += blockDim.x) {
+        for (int idx = tid_half; idx < MT * 16 * vecs; idx += 256) {
             const int m = idx / vecs, c = idx % vecs;
             uint4 v = make_uint4(0, 0, 0, 0);
-            if (m < M) v = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(m) * K + kc + c * 8);
-            xs[m * stride + c] = v;
+            if (m < M) v = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(m) * K + k_begin + kc + c * 8);
+            xh[m * stride + c] = v;
         }
         __syncthreads();
-        if (n0 < inter) {
-            const bf16* gp = grow + kc + 8 * g;
-            const bf16* up = urow + kc + 8 * g;
-            int k = 0;
-            for (; k + 64 <= len; k += 64) {
-                Frag a[4];
-                a[0].u = *reinterpret_cast<const uint4*>(gp + k);
-                a[1].u = *reinterpret_cast<const uint4*>(up + k);
-                a[2].u = *reinterpret_cast<const uint4*>(gp + k + 32);
-                a[3].u = *reinterpret_cast<const uint4*>(up + k + 32);
+        for (int k = 0; k < len; k += 32 * kBatch) {
+            const int used = min(kBatch, (len - k) / 32);
+            fetch(nxtg, nxtu, step + used);
 #pragma unroll
-                for (int u2 = 0; u2 < 2; ++u2) {
+            for (int u = 0; u < kBatch; ++u) {
+                if (k + 32 * u < len) {
 #pragma unroll
                     for (int t = 0; t < MT; ++t) {
                         Frag b;
-                        b.u = xs[(t * 16 + i) * stride + (k + 32 * u2) / 8 + g];
-                        accg[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[2 * u2].v, b.v, accg[t], 0, 0, 0);
-                        accu[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[2 * u2 + 1].v, b.v, accu[t], 0, 0, 0);
+                        b.u = xh[(t * 16 + i) * stride + k / 8 + 4 * u + g];
+                        accg[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(curg[u].v, b.v, accg[t], 0, 0, 0);
+                        accu[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(curu[u].v, b.v, accu[t], 0, 0, 0);
                     }
                 }
             }
-            for (; k < len; k += 32) {
-                Frag ag, au;
-                ag.u = *reinterpret_cast<const uint4*>(gp + k);
-                au.u = *reinterpret_cast<const uint4*>(up + k);
 #pragma unroll
-                for (int t = 0; t < MT; ++t) {
-                    Frag b;
-                    b.u = xs[(t * 16 + i) * stride + k / 8 + g];
-                    accg[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ag.v, b.v, accg[t], 0, 0, 0);
-                    accu[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(au.v, b.v, accu[t], 0, 0, 0);
-                }
+            for (int u = 0; u < kBatch; ++u) {
+                curg[u] = nxtg[u];
+                curu[u] = nxtu[u];
             }
+            step += used;
         }
     }
-    if (n0 >= inter) return;
+    // the second half hands its sums to the first through shared memory
+    __syncthreads();
+    float* red = reinterpret_cast<float*>(xs) + (tile * kWave + lane) * (MT * 8);
+    if (half == 1) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                red[t * 8 + v] = accg[t][v];
+                red[t * 8 + 4 + v] = accu[t][v];
+            }
+    }
+    __syncthreads();
+    if (half == 1 || n0 >= inter) return;
     const int n = n0 + 4 * g;
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
@@ -245,7 +272,10 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
         if (m >= M) continue;
         float4_t r;
 #pragma unroll
-        for (int v = 0; v < 4; ++v) r[v] = (ACT == 0 ? act_gelu_tanh(accg[t][v]) : act_silu(accg[t][v])) * accu[t][v];
+        for (int v = 0; v < 4; ++v) {
+            const float gate = accg[t][v] + red[t * 8 + v], upv = accu[t][v] + red[t * 8 + 4 + v];
+            r[v] = (ACT == 0 ? act_gelu_tanh(gate) : act_silu(gate)) * upv;
+        }
         bf16* o = out + static_cast<size_t>(m) * inter + n;
         if (n + 3 < inter && (inter % 4 == 0)) {
             store4<bf16>(o, r);
@@ -259,14 +289,16 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
 
 WLLM_API int wllm_gemm_skinny_gated(const void* x, const void* w, void* out, int M, int inter, int K, int activation,
                                     int chunk, hipStream_t stream) {
-    if (M < 1 || M > 64 || K % 32 != 0 || chunk % 32 != 0 || activation < 0 || activation > 1) return -1;
+    if (M < 1 || M > 64 || K % 64 != 0 || chunk % 32 != 0 || activation < 0 || activation > 1) return -1;
     const int mt = (M + 15) / 16;
-    if (chunk > K) chunk = K;
-    const size_t smem = static_cast<size_t>(mt) * 16 * (chunk / 8 + 1) * sizeof(uint4);
+    if (chunk > K / 2) chunk = K / 2;
+    size_t smem = static_cast<size_t>(2) * mt * 16 * (chunk / 8 + 1) * sizeof(uint4);
+    const size_t red = static_cast<size_t>(4) * kWave * mt * 8 * sizeof(float);
+    if (red > smem) smem = red;
     if (smem > 65536) return -1;
     const dim3 grid((inter + 63) / 64);
 #define LAUNCH(MT, A)                                                                                              \
-    gemm_skinny_gated_kernel<MT, A><<<grid, 256, smem, stream>>>(static_cast<const bf16*>(x), static_cast<const bf16*>(w), \
+    gemm_skinny_gated_kernel<MT, A><<<grid, 512, smem, stream>>>(static_cast<const bf16*>(x), static_cast<const bf16*>(w), \
                                                                  static_cast<bf16*>(out), M, inter, K, chunk)
 #define BY_MT(A)                     \
     switch (mt) {                    \

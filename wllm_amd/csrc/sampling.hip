@@ -2,7 +2,10 @@
 #include "common.h"
 
 // ---- argmax: the largest value of a row, the lowest index among equals -------------------------
-constexpr int kArgmaxThreads = 1024;
+// Two stages, so that a handful of rows still use many compute units: a row is cut into
+// kArgmaxSplits segments, one workgroup each, then one wavefront per row picks among them.
+constexpr int kArgmaxThreads = 256;
+constexpr int kArgmaxSplits = 32;
 
 __device__ __forceinline__ void argmax_take(float v, int i, float& bv, int& bi) {
     // NaN never wins; among equals the lowest index
@@ -12,26 +15,7 @@ __device__ __forceinline__ void argmax_take(float v, int i, float& bv, int& bi) 
     }
 }
 
-__global__ void __launch_bounds__(kArgmaxThreads) argmax_rows_kernel(const float* __restrict__ logits,
-                                                                   int* __restrict__ out, int vocab) {
-    __shared__ float best_v[kArgmaxThreads / kWave];
-    __shared__ int best_i[kArgmaxThreads / kWave];
-    const float* row = logits + static_cast<size_t>(blockIdx.x) * vocab;
-    float bv = -INFINITY;
-    int bi = 0x7fffffff;
-    if (vocab % 4 == 0) {
-        // rows are 16-byte aligned: four values per load
-        const float4* row4 = reinterpret_cast<const float4*>(row);
-        for (int q = threadIdx.x; q < vocab / 4; q += blockDim.x) {
-            const float4 v = row4[q];
-            argmax_take(v.x, 4 * q, bv, bi);
-            argmax_take(v.y, 4 * q + 1, bv, bi);
-            argmax_take(v.z, 4 * q + 2, bv, bi);
-            argmax_take(v.w, 4 * q + 3, bv, bi);
-        }
-    } else {
-        for (int i = threadIdx.x; i < vocab; i += blockDim.x) argmax_take(row[i], i, bv, bi);
-    }
+__device__ __forceinline__ void argmax_wave(float& bv, int& bi) {
 #pragma unroll
     for (int off = kWave / 2; off > 0; off >>= 1) {
         const float ov = __shfl_xor(bv, off, kWave);
@@ -41,6 +25,31 @@ __global__ void __launch_bounds__(kArgmaxThreads) argmax_rows_kernel(const float
             bi = oi;
         }
     }
+}
+
+__global__ void __launch_bounds__(kArgmaxThreads)
+argmax_partial_kernel(const float* __restrict__ logits, float* __restrict__ part_v, int* __restrict__ part_i,
+                      int vocab, int segment) {
+    __shared__ float best_v[kArgmaxThreads / kWave];
+    __shared__ int best_i[kArgmaxThreads / kWave];
+    const float* row = logits + static_cast<size_t>(blockIdx.x) * vocab;
+    const int begin = blockIdx.y * segment, end = min(vocab, begin + segment);
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    if (vocab % 4 == 0) {
+        // rows and segments are 16-byte aligned: four values per load
+        const float4* row4 = reinterpret_cast<const float4*>(row);
+        for (int q = begin / 4 + threadIdx.x; q < end / 4; q += blockDim.x) {
+            const float4 v = row4[q];
+            argmax_take(v.x, 4 * q, bv, bi);
+            argmax_take(v.y, 4 * q + 1, bv, bi);
+            argmax_take(v.z, 4 * q + 2, bv, bi);
+            argmax_take(v.w, 4 * q + 3, bv, bi);
+        }
+    } else {
+        for (int i = begin + threadIdx.x; i < end; i += blockDim.x) argmax_take(row[i], i, bv, bi);
+    }
+    argmax_wave(bv, bi);
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     if (lane == 0) {
         best_v[wave] = bv;
@@ -53,12 +62,28 @@ __global__ void __launch_bounds__(kArgmaxThreads) argmax_rows_kernel(const float
                 bv = best_v[w];
                 bi = best_i[w];
             }
-        out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+        part_v[blockIdx.x * kArgmaxSplits + blockIdx.y] = bv;
+        part_i[blockIdx.x * kArgmaxSplits + blockIdx.y] = bi;
     }
 }
 
-WLLM_API int wllm_argmax_rows(const float* logits, int* out, int rows, int vocab, hipStream_t stream) {
-    argmax_rows_kernel<<<rows, kArgmaxThreads, 0, stream>>>(logits, out, vocab);
+__global__ void __launch_bounds__(kWave)
+argmax_final_kernel(const float* __restrict__ part_v, const int* __restrict__ part_i, int* __restrict__ out) {
+    const int lane = threadIdx.x;
+    float bv = lane < kArgmaxSplits ? part_v[blockIdx.x * kArgmaxSplits + lane] : -INFINITY;
+    int bi = lane < kArgmaxSplits ? part_i[blockIdx.x * kArgmaxSplits + lane] : 0x7fffffff;
+    argmax_wave(bv, bi);
+    if (lane == 0) out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+}
+
+// `scratch` holds rows * 64 four-byte words.
+WLLM_API int wllm_argmax_rows(const float* logits, int* out, void* scratch, int rows, int vocab, hipStream_t stream) {
+    float* part_v = static_cast<float*>(scratch);
+    int* part_i = reinterpret_cast<int*>(part_v + static_cast<size_t>(rows) * kArgmaxSplits);
+    int segment = (vocab + kArgmaxSplits - 1) / kArgmaxSplits;
+    segment = (segment + 3) / 4 * 4;
+    argmax_partial_kernel<<<dim3(rows, kArgmaxSplits), kArgmaxThreads, 0, stream>>>(logits, part_v, part_i, vocab, segment);
+    argmax_final_kernel<<<rows, kWave, 0, stream>>>(part_v, part_i, out);
     return launch_status();
 }
 

@@ -19,7 +19,7 @@ from typing import Optional
 import numpy as np
 import torch
 
-KEY_CHUNK = 256
+KEY_CHUNK = 128
 ROWS_PER_TILE = 16
 ITEM_INTS = 8
 

@@ -35,7 +35,7 @@ _SIGNATURES = {
                                   c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
                                   c_int, c_void_p],
     "wllm_gemm_generic": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
-    "wllm_argmax_rows": [c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "wllm_argmax_rows": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "wllm_gemm_skinny": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_sample_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
@@ -48,6 +48,7 @@ class HipBackend:
         self.lib = load()
         self._partial_o = None
         self._gemm_partials = None
+        self._argmax_scratch = None
         self._partial_ml = None
         for name, argtypes in _SIGNATURES.items():
             fn = getattr(self.lib, name)
@@ -226,10 +227,10 @@ class HipBackend:
     def gated_linear(self, x, weight, out, activation, scratch):
         self._on_gpu(x, weight, out, scratch)
         m, k = x.shape
-        if self.skinny_takes(x.dtype, m, k):
+        if self.skinny_takes(x.dtype, m, k) and k % 64 == 0:
             self._check(self.lib.wllm_gemm_skinny_gated(
                 _ptr(x), _ptr(weight), _ptr(out), m, out.shape[1], k, 0 if activation == "gelu_tanh" else 1,
-                self.SKINNY_CHUNK[-(-m // 16)], self._stream()), "gated_linear (few rows, matrix cores)")
+                self.SKINNY_CHUNK[-(-m // 16)] // 2, self._stream()), "gated_linear (few rows, matrix cores)")
             return
         self.linear(x, weight, scratch)
         self.gated_activation(scratch, out, activation)
@@ -240,10 +241,17 @@ class HipBackend:
             _ptr(gate_up), _ptr(out), int(gate_up.dtype == torch.bfloat16), 0 if activation == "gelu_tanh" else 1,
             gate_up.shape[0], out.shape[1], self._stream()), "gated_activation")
 
+    ARGMAX_ROWS = 4096       # rows per launch; the scratch (64 words a row) is allocated once
+
     def argmax_rows(self, logits, out):
         self._on_gpu(logits, out)
-        self._check(self.lib.wllm_argmax_rows(_ptr(logits), _ptr(out), logits.shape[0], logits.shape[1],
-                                              self._stream()), "argmax_rows")
+        if self._argmax_scratch is None or self._argmax_scratch.device != logits.device:
+            self._argmax_scratch = torch.empty(self.ARGMAX_ROWS * 64, dtype=torch.int32, device=logits.device)
+        for r in range(0, logits.shape[0], self.ARGMAX_ROWS):
+            rows = min(self.ARGMAX_ROWS, logits.shape[0] - r)
+            self._check(self.lib.wllm_argmax_rows(_ptr(logits[r:r + rows]), _ptr(out[r:r + rows]),
+                                                  _ptr(self._argmax_scratch), rows, logits.shape[1], self._stream()),
+                        "argmax_rows")
 
     def sample_rows(self, logits, params, seeds, penalty_ids, penalty_offsets, out_tokens, out_logprobs):
         self._on_gpu(logits, params, seeds, penalty_ids, penalty_offsets, out_tokens, out_logprobs)
