@@ -91,7 +91,8 @@ def measure_decode(model, batch: int, context: int, steps: int, warmup: int, blo
     import torch
 
     from wllm_amd.engine import ModelRunner, Request, Scheduler
-    total_new = warmup + steps + 1
+    # requests admitted first decode while the later ones are still prefilled, one prompt a step
+    total_new = batch + warmup + steps + 2
     pages = batch * (-(-(context + total_new) // block_size)) + 2
     runner = ModelRunner.create(model, num_pages=pages, page_size=block_size, max_requests=batch)
     if hip_graphs and hasattr(runner, "enable_graphs"):
@@ -106,14 +107,15 @@ def measure_decode(model, batch: int, context: int, steps: int, warmup: int, blo
     for _ in range(warmup):
         sched.step()
     assert len(sched.running) == batch and all(r.status.value == "running" for r in sched.running)
-    first_len = sched.running[0].num_computed
+    len_before = sum(r.num_computed for r in sched.running) / batch
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
         sched.step()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    mean_ctx = first_len + (steps + 1) / 2.0
+    assert len(sched.running) == batch, "a request finished inside the timed steps"
+    mean_ctx = (len_before + sum(r.num_computed for r in sched.running) / batch) / 2.0
     del sched, runner
     torch.cuda.empty_cache()
     return dt, mean_ctx
