@@ -183,12 +183,15 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
             const float alpha = exp2f((m_run - m_use) * scale_log2e);    // 0 while nothing was seen
             Pack16 pv;
             float psum = 0.f;
+            const float mc = m_use * scale_log2e;
+            float pe[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float p = ok[e] ? exp2f((sv[e] - m_use) * scale_log2e) : 0.f;
-                psum += p;
-                pv.s[e] = bf16_bits(p);
+                pe[e] = ok[e] ? exp2f(fmaf(sv[e], scale_log2e, -mc)) : 0.f;
+                psum += pe[e];
             }
+            pv.u = make_uint4(pack2_bf16(pe[0], pe[1]), pack2_bf16(pe[2], pe[3]), pack2_bf16(pe[4], pe[5]),
+                              pack2_bf16(pe[6], pe[7]));
             l_run = l_run * alpha + psum;      // per lane; the four lanes of a row are added at the end
             m_run = m_new;
             // ---- out^T += V^T . P^T ----
@@ -254,8 +257,8 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
 #pragma unroll
         for (int t = 0; t < DT; ++t) {
             uint2 w;
-            w.x = bf16_bits(acc[t][0] * inv) | (static_cast<uint32_t>(bf16_bits(acc[t][1] * inv)) << 16);
-            w.y = bf16_bits(acc[t][2] * inv) | (static_cast<uint32_t>(bf16_bits(acc[t][3] * inv)) << 16);
+            w.x = pack2_bf16(acc[t][0] * inv, acc[t][1] * inv);
+            w.y = pack2_bf16(acc[t][2] * inv, acc[t][3] * inv);
             *reinterpret_cast<uint2*>(orow + t * 16 + 4 * g) = w;
         }
     } else {

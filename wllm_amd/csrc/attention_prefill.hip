@@ -1,0 +1,329 @@
+// Paged attention for long segments (prompt portions) on the matrix cores, bfloat16: the keys
+// and values of a block of 32 keys are staged through shared memory once per workgroup and read
+// by all four wavefronts; a wavefront owns 32 query rows (two tiles of 16), so every fragment it
+// reads from shared memory feeds two products.  A workgroup is 128 rows of one (segment, key/value
+// head): rows are (token, query head of the group) pairs, row r = token * G + head.
+//
+// The products are those of `attention_mfma.hip` (v_mfma_f32_16x16x32_bf16, scores transposed so
+// that a lane's values all belong to one query row, probabilities fed to the second product from
+// the registers they were computed in).  Staging: while the products of block b run from shared
+// memory, the global loads of block b+1 are in flight into registers; they are written to shared
+// memory after a barrier.  Keys land as [32][HD] rows (padded), values as [HD][32] rows whose 32
+// keys are permuted so that the 8 keys a lane needs are contiguous.  Keys outside the request
+// (stale slots of the last page, pages a window gave back) are cleared while staging, so that a
+// NaN there cannot meet a zero probability.
+#include "common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kPrefillWaves = 4;       // wavefronts per workgroup
+constexpr int kPrefillThreads = kPrefillWaves * 64;
+constexpr int kBlockKeys = 32;
+constexpr int kMaxTablePages = 4096;
+
+union PPack {
+    uint4 u;
+    bf16x8_t v;
+    uint2 half[2];
+    uint16_t s[8];
+};
+
+template <int HD>
+struct PrefillSmem {
+    static constexpr int kStrideK = HD + 8;            // elements; the pad spreads rows over banks
+    static constexpr int kStrideV = kBlockKeys + 8;
+    static constexpr int kBytes = (kBlockKeys * kStrideK + HD * kStrideV) * 2;
+};
+
+// prefill items: seg, kvh, first row, unused
+template <int HD, int RTW>      // RTW: tiles of 16 rows per wavefront (1 or 2)
+__global__ void __launch_bounds__(kPrefillThreads)
+paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restrict__ cache,
+                               const int* __restrict__ block_tables, const int* __restrict__ items,
+                               const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
+                               const int* __restrict__ seg_ctx_len, bf16* __restrict__ out, int num_heads,
+                               int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window) {
+    constexpr int DC = HD / 32, DT = HD / 16;
+    constexpr int SK = PrefillSmem<HD>::kStrideK, SV = PrefillSmem<HD>::kStrideV;
+    __shared__ __align__(16) uint16_t k_s[kBlockKeys * SK];
+    __shared__ __align__(16) uint16_t v_s[HD * SV];
+    __shared__ int table_s[kMaxTablePages];     // the request's block table: page lookups never leave the CU
+
+    const int* item = items + static_cast<size_t>(blockIdx.x) * 4;
+    const int seg = item[0], kvh = item[1], row_begin = item[2];
+    if (seg < 0) return;
+    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const int i = lane % 16, g = lane / 16;
+    const int group = num_heads / num_kv_heads;
+    const int q_start = seg_q_start[seg], q_len = seg_q_len[seg], ctx = seg_ctx_len[seg];
+    const int total_rows = q_len * group;
+    const int first_pos = ctx - q_len;
+    const int seg_lo = window > 0 ? max(0, first_pos - window + 1) : 0;
+    const int width = (num_heads + 2 * num_kv_heads) * HD;
+    const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * HD;
+    const size_t k_off = static_cast<size_t>(kvh) * page_size * HD;
+    const size_t v_off = (static_cast<size_t>(num_kv_heads) + kvh) * page_size * HD;
+    {
+        const int* table_g = block_tables + static_cast<size_t>(seg) * max_pages;
+        const int pages_used = min(max_pages, (ctx + page_size - 1) / page_size);
+        for (int p = tid; p < pages_used; p += kPrefillThreads) table_s[p] = table_g[p];
+    }
+    const int* table = table_s;
+
+    // this wavefront's two tiles of rows
+    constexpr int kWaveRows = 16 * RTW, kPrefillRows = kPrefillWaves * kWaveRows;
+    const int wr0 = row_begin + wave * kWaveRows;
+    int row[RTW], tok[RTW], head[RTW], pos[RTW], lo[RTW];
+    bool row_valid[RTW];
+    bf16x8_t qreg[RTW][DC];
+#pragma unroll
+    for (int rt = 0; rt < RTW; ++rt) {
+        row[rt] = wr0 + rt * 16 + i;
+        row_valid[rt] = row[rt] < total_rows;
+        tok[rt] = row_valid[rt] ? row[rt] / group : 0;
+        head[rt] = kvh * group + (row_valid[rt] ? row[rt] % group : 0);
+        pos[rt] = first_pos + tok[rt];
+        lo[rt] = window > 0 ? max(0, pos[rt] - window + 1) : 0;
+        const bf16* qrow = qkv + static_cast<size_t>(q_start + tok[rt]) * width + static_cast<size_t>(head[rt]) * HD;
+#pragma unroll
+        for (int c = 0; c < DC; ++c) {
+            PPack p;
+            p.u = row_valid[rt] ? *reinterpret_cast<const uint4*>(qrow + c * 32 + 8 * g) : make_uint4(0, 0, 0, 0);
+            qreg[rt][c] = p.v;
+        }
+    }
+    // per row tile: the lowest position and the highest window start of its rows (wavefront-wide)
+    int t_pos_min[RTW], t_lo_max[RTW];
+#pragma unroll
+    for (int rt = 0; rt < RTW; ++rt) {
+        const int first = wr0 + rt * 16, last = min(total_rows - 1, first + 15);
+        t_pos_min[rt] = first < total_rows ? first_pos + first / group : -1;
+        const int pmax = first_pos + max(last, 0) / group;
+        t_lo_max[rt] = window > 0 ? max(0, pmax - window + 1) : 0;
+        if (last < first + 15) t_pos_min[rt] = -1;      // a tile with rows beyond the segment always masks
+    }
+    // keys the wavefront's rows can need
+    const bool wave_active = wr0 < total_rows;
+    const int w_last_row = min(total_rows - 1, wr0 + kWaveRows - 1);
+    const int w_hi = wave_active ? first_pos + w_last_row / group + 1 : 0;                       // exclusive
+    const int w_lo = window > 0 ? max(0, first_pos + wr0 / group - window + 1) : 0;
+    // keys the workgroup stages: from the first wavefront's lowest to the last row's highest
+    const int b_last_row = min(total_rows - 1, row_begin + kPrefillRows - 1);
+    const int b_hi = first_pos + b_last_row / group + 1;
+    const int b_lo = window > 0 ? max(0, first_pos + row_begin / group - window + 1) : 0;
+    const int blk_first = b_lo / kBlockKeys, blk_end = (b_hi + kBlockKeys - 1) / kBlockKeys;
+
+    float4_t acc[RTW][DT];
+    float m_run[RTW], l_run[RTW];
+#pragma unroll
+    for (int rt = 0; rt < RTW; ++rt) {
+        m_run[rt] = -INFINITY;
+        l_run[rt] = 0.f;
+#pragma unroll
+        for (int t = 0; t < DT; ++t) acc[rt][t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // ---- staging.  Keys: kTPK threads share a key row and take its 16-byte chunks in turn, so a
+    //      thread looks up one page per block.  Values: a thread keeps one group of 4 keys (j) and
+    //      walks the rows d of the transposed page, again one page lookup per block. ----
+    constexpr int kTPK = kPrefillThreads / kBlockKeys;              // threads per key row
+    constexpr int KCH = (HD / 8 + kTPK - 1) / kTPK;
+    constexpr int kRowsPerPass = kPrefillThreads / 8;               // value rows staged per pass
+    constexpr int VCH = (HD + kRowsPerPass - 1) / kRowsPerPass;
+    const int k_key = tid / kTPK, k_lane = tid % kTPK;
+    const int v_j = tid % 8, v_d0 = tid / 8;
+    uint4 kreg_a[KCH];
+    uint2 vreg_a[VCH];
+    const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
+    auto page_of = [&](int key, int& slot) -> int {
+        if (page_shift >= 0) {
+            slot = key & (page_size - 1);
+            return table[key >> page_shift];
+        }
+        slot = key % page_size;
+        return table[key / page_size];
+    };
+    auto fetch = [&](uint4* kreg, uint2* vreg, int kbase) {
+        {
+            const int key = kbase + k_key;
+            const bool ok = key < ctx && key >= seg_lo;
+            const int kk = min(key, ctx - 1);
+            int slot;
+            const int page = page_of(kk, slot);
+            const bf16* src = cache + static_cast<size_t>(page) * page_elems + k_off + static_cast<size_t>(slot) * HD;
+#pragma unroll
+            for (int u = 0; u < KCH; ++u) {
+                const int chunk = k_lane + u * kTPK;
+                kreg[u] = (ok && chunk < HD / 8) ? *reinterpret_cast<const uint4*>(src + chunk * 8)
+                                                 : make_uint4(0, 0, 0, 0);
+            }
+        }
+        {
+            const int key = kbase + 4 * v_j;                 // group v_j: keys key .. key + 3
+            const int kk = min(key, ctx - 1) & ~3;
+            int slot;
+            const int page = page_of(kk, slot);
+            const bf16* src = cache + static_cast<size_t>(page) * page_elems + v_off + slot;
+            // keys of the group that are not the request's are cleared
+            uint2 keep = make_uint2(0xffffffffu, 0xffffffffu);
+            if (key + 3 >= ctx || key < seg_lo) {
+                const bool k0 = key < ctx && key >= seg_lo, k1 = key + 1 < ctx && key + 1 >= seg_lo;
+                const bool k2 = key + 2 < ctx && key + 2 >= seg_lo, k3 = key + 3 < ctx && key + 3 >= seg_lo;
+                keep.x = (k0 ? 0x0000ffffu : 0u) | (k1 ? 0xffff0000u : 0u);
+                keep.y = (k2 ? 0x0000ffffu : 0u) | (k3 ? 0xffff0000u : 0u);
+            }
+#pragma unroll
+            for (int u = 0; u < VCH; ++u) {
+                const int d = min(v_d0 + u * kRowsPerPass, HD - 1);
+                uint2 v = *reinterpret_cast<const uint2*>(src + static_cast<size_t>(d) * page_size);
+                v.x &= keep.x;
+                v.y &= keep.y;
+                vreg[u] = v;
+            }
+        }
+    };
+    auto stage = [&](const uint4* kreg, const uint2* vreg) {
+#pragma unroll
+        for (int u = 0; u < KCH; ++u) {
+            const int chunk = k_lane + u * kTPK;
+            if (chunk < HD / 8) *reinterpret_cast<uint4*>(&k_s[k_key * SK + chunk * 8]) = kreg[u];
+        }
+#pragma unroll
+        for (int u = 0; u < VCH; ++u) {
+            const int d = v_d0 + u * kRowsPerPass;
+            // keys 4j..4j+3 go to positions 8*(j%4) + 4*(j/4): a lane's keys {4g..4g+3, 16+4g..} become contiguous
+            if (d < HD) *reinterpret_cast<uint2*>(&v_s[d * SV + 8 * (v_j % 4) + 4 * (v_j / 4)]) = vreg[u];
+        }
+    };
+
+    __syncthreads();      // the block table is in shared memory
+    // the loads of the next block are in flight while the products of this one run
+    if (blk_first < blk_end) fetch(kreg_a, vreg_a, blk_first * kBlockKeys);
+    for (int blk = blk_first; blk < blk_end; ++blk) {
+        const int kbase = blk * kBlockKeys;
+        __syncthreads();                 // everyone is done with the previous block's tiles
+        stage(kreg_a, vreg_a);
+        __syncthreads();
+        if (blk + 1 < blk_end) fetch(kreg_a, vreg_a, kbase + kBlockKeys);
+        if (!wave_active || kbase >= w_hi || kbase + kBlockKeys <= w_lo) continue;
+        // ---- scores: tile t2 holds keys kbase + 16*t2 + (0..15); lane (i, g) gets keys 16*t2 + 4g + v ----
+        float4_t s[RTW][2];
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2) {
+            float4_t sc[RTW];
+#pragma unroll
+            for (int rt = 0; rt < RTW; ++rt) sc[rt] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < DC; ++c) {
+                PPack a;
+                a.u = *reinterpret_cast<const uint4*>(&k_s[(16 * t2 + i) * SK + c * 32 + 8 * g]);
+#pragma unroll
+                for (int rt = 0; rt < RTW; ++rt)
+                    sc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qreg[rt][c], sc[rt], 0, 0, 0);
+            }
+#pragma unroll
+            for (int rt = 0; rt < RTW; ++rt) s[rt][t2] = sc[rt];
+        }
+        // ---- softmax bookkeeping per row tile ----
+        PPack pv[RTW];
+        float alpha[RTW];
+        bool rescale[RTW];
+#pragma unroll
+        for (int rt = 0; rt < RTW; ++rt) {
+            float sv[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sv[e] = s[rt][e / 4][e % 4];
+            // blocks that lie wholly inside every row's range need no mask (a wavefront-wide decision)
+            const bool inside = kbase + kBlockKeys - 1 <= t_pos_min[rt] && kbase >= t_lo_max[rt];
+            if (!inside) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int key = kbase + 16 * (e / 4) + 4 * g + (e % 4);
+                    if (!(row_valid[rt] && key <= pos[rt] && key >= lo[rt])) sv[e] = -INFINITY;
+                }
+            }
+            float tile_max = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
+                                   fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
+            const float m_new = fmaxf(m_run[rt], tile_max);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            const float mc = m_use * scale_log2e;
+            alpha[rt] = exp2f(fmaf(m_run[rt], scale_log2e, -mc));
+            float pe[8], psum = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                pe[e] = exp2f(fmaf(sv[e], scale_log2e, -mc));       // exp2(-inf) = 0 for masked keys
+                psum += pe[e];
+            }
+            pv[rt].u = make_uint4(pack2_bf16(pe[0], pe[1]), pack2_bf16(pe[2], pe[3]), pack2_bf16(pe[4], pe[5]),
+                                  pack2_bf16(pe[6], pe[7]));
+            l_run[rt] = l_run[rt] * alpha[rt] + psum;
+            m_run[rt] = m_new;
+            rescale[rt] = __any(alpha[rt] != 1.f);
+        }
+        // ---- out^T += V^T . P^T; the accumulators are rescaled only when some row's maximum moved ----
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+            PPack a;
+            a.u = *reinterpret_cast<const uint4*>(&v_s[(16 * t + i) * SV + 8 * g]);
+#pragma unroll
+            for (int rt = 0; rt < RTW; ++rt) {
+                if (rescale[rt]) acc[rt][t] *= alpha[rt];
+                acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pv[rt].v, acc[rt][t], 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int rt = 0; rt < RTW; ++rt) {
+        float l = l_run[rt];
+        l += __shfl_xor(l, 16, kWave);
+        l += __shfl_xor(l, 32, kWave);
+        if (!row_valid[rt]) continue;
+        const float inv = 1.f / l;
+        bf16* orow = out + (static_cast<size_t>(q_start + tok[rt]) * num_heads + head[rt]) * HD;
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+            uint2 w;
+            w.x = pack2_bf16(acc[rt][t][0] * inv, acc[rt][t][1] * inv);
+            w.y = pack2_bf16(acc[rt][t][2] * inv, acc[rt][t][3] * inv);
+            *reinterpret_cast<uint2*>(orow + t * 16 + 4 * g) = w;
+        }
+    }
+}
+
+// Returns 0, a HIP error code, or -1 for sizes this kernel does not take.
+WLLM_API int wllm_paged_attention_prefill(const void* qkv, const void* cache, const int* block_tables,
+                                          const int* items, int num_items, int rows_per_item, const int* seg_q_start,
+                                          const int* seg_q_len, const int* seg_ctx_len, void* out, int num_heads,
+                                          int num_kv_heads, int head_dim, int page_size, int max_pages, float scale,
+                                          int window, hipStream_t stream) {
+    if (head_dim % 32 != 0 || head_dim < 32 || head_dim > 256 || page_size % 4 != 0 || num_heads % num_kv_heads != 0)
+        return -1;
+    if (max_pages > kMaxTablePages) return -1;       // the block table must fit the kernel's shared copy
+    if (rows_per_item != 64 && rows_per_item != 128) return -1;
+    if (num_items <= 0) return 0;
+    const float scale_log2e = scale * 1.4426950408889634f;
+#define LAUNCH_RTW(HD, RTW)                                                                                         \
+    paged_attention_prefill_kernel<HD, RTW><<<num_items, kPrefillThreads, 0, stream>>>(                             \
+        static_cast<const bf16*>(qkv), static_cast<const bf16*>(cache), block_tables, items, seg_q_start, seg_q_len, \
+        seg_ctx_len, static_cast<bf16*>(out), num_heads, num_kv_heads, page_size, max_pages, scale_log2e, window)
+#define LAUNCH(HD)                            \
+    if (rows_per_item == 64) LAUNCH_RTW(HD, 1); \
+    else LAUNCH_RTW(HD, 2)
+    switch (head_dim) {
+        case 32: LAUNCH(32); break;
+        case 64: LAUNCH(64); break;
+        case 96: LAUNCH(96); break;
+        case 128: LAUNCH(128); break;
+        case 160: LAUNCH(160); break;
+        case 192: LAUNCH(192); break;
+        case 224: LAUNCH(224); break;
+        case 256: LAUNCH(256); break;
+        default: return -1;
+    }
+#undef LAUNCH
+#undef LAUNCH_RTW
+    return launch_status();
+}

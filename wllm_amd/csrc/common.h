@@ -19,11 +19,18 @@ __device__ __forceinline__ float to_float(bf16 v) { return __uint_as_float(stati
 template <typename T> __device__ __forceinline__ T from_float(float v);
 template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
 template <> __device__ __forceinline__ bf16 from_float<bf16>(float v) {
-    // round to nearest, ties to even; NaN stays NaN
-    uint32_t x = __float_as_uint(v);
-    if ((x & 0x7fffffffu) > 0x7f800000u) return bf16{static_cast<uint16_t>((x >> 16) | 0x0040u)};
-    x += 0x7fffu + ((x >> 16) & 1u);
-    return bf16{static_cast<uint16_t>(x >> 16)};
+    // round to nearest, ties to even, NaN stays NaN: gfx950 converts in hardware (v_cvt_pk_bf16_f32)
+    const __bf16 h = static_cast<__bf16>(v);
+    return bf16{*reinterpret_cast<const uint16_t*>(&h)};
+}
+
+// Two floats to two bfloat16 in one word, the first in the low half (one v_cvt_pk_bf16_f32).
+__device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    typedef float float2_t __attribute__((ext_vector_type(2)));
+    const float2_t f = {lo, hi};
+    const bf16x2_t r = __builtin_convertvector(f, bf16x2_t);
+    return *reinterpret_cast<const uint32_t*>(&r);
 }
 
 __device__ __forceinline__ float wave_sum(float v) {

@@ -25,8 +25,8 @@ template <typename TO> __device__ __forceinline__ void store4(TO* p, float4_t v)
 template <> __device__ __forceinline__ void store4<float>(float* p, float4_t v) { *reinterpret_cast<float4_t*>(p) = v; }
 template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float4_t v) {
     uint2 w;
-    w.x = from_float<bf16>(v[0]).bits | (static_cast<uint32_t>(from_float<bf16>(v[1]).bits) << 16);
-    w.y = from_float<bf16>(v[2]).bits | (static_cast<uint32_t>(from_float<bf16>(v[3]).bits) << 16);
+    w.x = pack2_bf16(v[0], v[1]);
+    w.y = pack2_bf16(v[2], v[3]);
     *reinterpret_cast<uint2*>(p) = w;
 }
 

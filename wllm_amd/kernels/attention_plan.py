@@ -9,7 +9,9 @@ workgroups of up to four tiles of 16 rows that each walk all their keys.
 
 A work item is 8 int32: segment, key/value head, first row, row tiles (1, 2 or 4), first key,
 end key, partial slot (-1: the workgroup writes the final result), unused.  A reduce item is
-4 int32: segment, key/value head, first partial slot, number of splits.
+4 int32: segment, key/value head, first partial slot, number of splits.  A prefill item (long
+segments, 64 or 128 rows each, for the kernel that stages keys and values through shared memory) is
+4 int32: segment, key/value head, first row, unused.
 """
 from __future__ import annotations
 
@@ -33,6 +35,9 @@ class AttentionPlan:
     num_partial_slots: int
     partial_o: Optional[torch.Tensor] = None    # float32 [slots * 16 * head_dim]
     partial_ml: Optional[torch.Tensor] = None   # float32 [slots * 16 * 2]
+    prefill_items: Optional[torch.Tensor] = None  # int32 [num_prefill, 4]
+    num_prefill: int = 0
+    prefill_rows: int = 64
 
 
 class StaticAttentionPlan(AttentionPlan):
@@ -55,7 +60,8 @@ class StaticAttentionPlan(AttentionPlan):
 
     def update(self, q_len: np.ndarray, ctx_len: np.ndarray) -> None:
         group, nkv, window, fixed = self._args
-        items, reduces, slots = build_work_items(q_len, ctx_len, group, nkv, window, fixed)
+        items, reduces, slots, prefill, _ = build_work_items(q_len, ctx_len, group, nkv, window, fixed)
+        assert prefill.shape[0] == 0, "a captured decode graph holds no long segment"
         if slots > self.max_slots:
             raise ValueError(f"the step needs {slots} partial slots, the graph's plan has {self.max_slots}")
         assert items.shape[0] == self.num_items and reduces.shape[0] == self.num_reduce
@@ -67,7 +73,7 @@ class StaticAttentionPlan(AttentionPlan):
 
 def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_heads: int, window: int,
                      fixed_splits: int = 0):
-    """Returns (items [n, 8], reduce_items [m, 4], partial slots) as int32 arrays.
+    """Returns (items [n, 8], reduce_items [m, 4], partial slots, prefill items [p, 4]) as int32 arrays.
 
     `fixed_splits` > 0 gives every short segment exactly that many items per key/value head
     (items beyond the segment's keys are padding that the kernel skips), so that the number
@@ -124,16 +130,20 @@ def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_
             rs[..., 3] = ns[:, None]
             reduces.append(rs[split_seg].reshape(-1, 4))
         slots = int((n_split_seg * num_kv_heads).sum())
-    # ---- long segments: workgroups of up to four row tiles over all keys ----
+    # ---- long segments: workgroups of 64 or 128 rows that walk all their keys ----
+    prefill = []
+    long_rows = rows[~short]
+    # 128 rows a workgroup when that still gives every compute unit two workgroups, else 64
+    prefill_rows = 128 if int((-(-long_rows // 128)).sum()) * num_kv_heads >= 512 else 64
     for s in np.nonzero(~short)[0]:
-        tiles = -(-int(rows[s]) // ROWS_PER_TILE)
-        t = 0
-        while t < tiles:
-            left = tiles - t
-            rt = 4 if left >= 3 else left          # 3 tiles run as 4 with one idle wavefront
-            for h in range(num_kv_heads):
-                items.append(np.array([[s, h, t * ROWS_PER_TILE, rt, 0, int(ctx_len[s]), -1, 0]], dtype=np.int32))
-            t += rt
+        blocks = -(-int(rows[s]) // prefill_rows)
+        it = np.zeros((blocks, num_kv_heads, 4), dtype=np.int32)
+        it[..., 0] = s
+        it[..., 1] = kv[None, :]
+        it[..., 2] = (np.arange(blocks, dtype=np.int32) * prefill_rows)[:, None]
+        # the last rows see the most keys: start them first
+        prefill.append(it[::-1].reshape(-1, 4))
+    prefill = np.concatenate(prefill) if prefill else np.zeros((0, 4), np.int32)
     items = np.concatenate(items) if items else np.zeros((0, ITEM_INTS), np.int32)
     reduces = np.concatenate(reduces) if reduces else np.zeros((0, 4), np.int32)
-    return items, reduces, slots
+    return items, reduces, slots, prefill, prefill_rows
