@@ -331,16 +331,17 @@ def test_gated_linear(dtype, act, m, inter, k):
 def test_gated_activation(dtype, act):
     torch.manual_seed(5)
 
-    def make():
-        gu = (torch.randn(13, 2 * 250, device=DEV) * 3).to(dtype)
-        return [gu, torch.zeros(13, 250, device=DEV, dtype=dtype), act], {}
+    for inter in (250, 256, 1032):
+        def make():
+            gu = (torch.randn(13, 2 * inter, device=DEV) * 3).to(dtype)
+            return [gu, torch.zeros(13, inter, device=DEV, dtype=dtype), act], {}
 
-    torch.manual_seed(5)
-    g, r = both("gated_activation", make, dtype)
-    close(g[1], r[1], dtype)
-    if act == "gelu_tanh":
-        ref = torch.nn.functional.gelu(g[0][:, :250].float(), approximate="tanh") * g[0][:, 250:].float()
-        close(g[1], ref, dtype, "against the library's gelu")
+        torch.manual_seed(5)
+        g, r = both("gated_activation", make, dtype)
+        close(g[1], r[1], dtype)
+        if act == "gelu_tanh":
+            ref = torch.nn.functional.gelu(g[0][:, :inter].float(), approximate="tanh") * g[0][:, inter:].float()
+            close(g[1], ref, dtype, "against the library's gelu")
 
 
 def test_argmax_rows_lowest_index_among_equals():

@@ -30,90 +30,120 @@ template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float4_t v) {
     *reinterpret_cast<uint2*>(p) = w;
 }
 
-template <int MT, typename TO>
+// NT: tiles of 16 weight rows per wavefront.  With many rows of x (MT > 1) every fragment of x read
+// from shared memory then feeds NT products, and a workgroup stages x once for 64*NT weight rows.
+template <int MT, int NT, typename TO>
 __global__ void __launch_bounds__(256)
 gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* __restrict__ out,
                    float* __restrict__ partial, int M, int N, int K, int k_per_split, int chunk) {
     extern __shared__ uint4 xs[];                 // [MT*16][chunk/8 + 1]
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const int i = lane % 16, g = lane / 16;
-    const int n0 = (blockIdx.x * 4 + wave) * 16;
+    const int n0 = (blockIdx.x * 4 + wave) * 16 * NT;
     const int k_begin = blockIdx.y * k_per_split, k_end = min(K, k_begin + k_per_split);
     const int stride = chunk / 8 + 1;             // in uint4; the odd stride spreads rows over the banks
-    const bf16* wrow = w + static_cast<size_t>(min(n0 + i, N - 1)) * K;
-    float4_t acc[MT];
+    const bf16* wp[NT];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int nt = 0; nt < NT; ++nt)
+        wp[nt] = w + static_cast<size_t>(min(n0 + nt * 16 + i, N - 1)) * K + k_begin + 8 * g;
+    float4_t acc[NT][MT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[nt][t] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    // The weight stream is read in batches of kBatch 16-byte loads per lane; the next batch is
-    // in flight while the products of this one are made, the first before x is staged at all.
-    constexpr int kBatch = 16;
+    // The weight stream is read in batches of kBatch 16-byte loads per lane and tile; the next batch
+    // is in flight while the products of this one are made, the first before x is staged at all.
+    constexpr int kBatch = 16 / NT;
     const bool live = n0 < N;
     const int steps = (k_end - k_begin) / 32;
-    const bf16* wp = wrow + k_begin + 8 * g;
-    Frag cur[kBatch], nxt[kBatch];
-    auto fetch = [&](Frag* dst, int step0) {
+    Frag cur[NT][kBatch], nxt[NT][kBatch];
+    auto fetch = [&](Frag (&dst)[NT][kBatch], int step0) {
 #pragma unroll
-        for (int u = 0; u < kBatch; ++u)
-            dst[u].u = (live && step0 + u < steps) ? *reinterpret_cast<const uint4*>(wp + (step0 + u) * 32)
-                                                   : make_uint4(0, 0, 0, 0);
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u)
+                dst[nt][u].u = (live && step0 + u < steps) ? *reinterpret_cast<const uint4*>(wp[nt] + (step0 + u) * 32)
+                                                           : make_uint4(0, 0, 0, 0);
     };
     fetch(cur, 0);
+    // x is staged chunk by chunk; the loads of the next chunk are in flight during the products
+    constexpr int kXRegs = 8;                     // 16-byte pieces of a chunk per thread (MT*16*chunk/8 <= 2048)
+    uint4 xreg[kXRegs];
+    auto fetch_x = [&](int kc) {
+        const int vecs = min(chunk, k_end - kc) / 8;
+#pragma unroll
+        for (int u = 0; u < kXRegs; ++u) {
+            const int idx = threadIdx.x + u * 256;
+            const int m = idx / vecs, c = idx % vecs;
+            xreg[u] = (idx < MT * 16 * vecs && m < M) ? *reinterpret_cast<const uint4*>(x + static_cast<size_t>(m) * K + kc + c * 8)
+                                                      : make_uint4(0, 0, 0, 0);
+        }
+    };
+    fetch_x(k_begin);
     int step = 0;
     for (int kc = k_begin; kc < k_end; kc += chunk) {
         const int len = min(chunk, k_end - kc);   // a multiple of 32
         const int vecs = len / 8;
         __syncthreads();
-        for (int idx = threadIdx.x; idx < MT * 16 * vecs; idx += blockDim.x) {
-            const int m = idx / vecs, c = idx % vecs;
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (m < M) v = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(m) * K + kc + c * 8);
-            xs[m * stride + c] = v;
+#pragma unroll
+        for (int u = 0; u < kXRegs; ++u) {
+            const int idx = threadIdx.x + u * 256;
+            if (idx < MT * 16 * vecs) xs[(idx / vecs) * stride + idx % vecs] = xreg[u];
         }
         __syncthreads();
+        if (kc + chunk < k_end) fetch_x(kc + chunk);
         for (int k = 0; k < len; k += 32 * kBatch) {
             const int used = min(kBatch, (len - k) / 32);      // steps of this batch that lie in the chunk
             fetch(nxt, step + used);
 #pragma unroll
             for (int u = 0; u < kBatch; ++u) {
                 if (k + 32 * u < len) {
+                    Frag b[MT];
 #pragma unroll
-                    for (int t = 0; t < MT; ++t) {
-                        Frag b;
-                        b.u = xs[(t * 16 + i) * stride + k / 8 + 4 * u + g];
-                        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[u].v, b.v, acc[t], 0, 0, 0);
-                    }
+                    for (int t = 0; t < MT; ++t) b[t].u = xs[(t * 16 + i) * stride + k / 8 + 4 * u + g];
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                        for (int t = 0; t < MT; ++t)
+                            acc[nt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[nt][u].v, b[t].v, acc[nt][t], 0, 0, 0);
                 }
             }
 #pragma unroll
-            for (int u = 0; u < kBatch; ++u) cur[u] = nxt[u];
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u) cur[nt][u] = nxt[nt][u];
             step += used;
         }
     }
-    if (n0 >= N) return;
-    // lane (i, g) holds columns n0 + 4g .. +3 of row m = 16t + i
-    const int n = n0 + 4 * g;
+    if (!live) return;
+    // lane (i, g) holds columns n .. n + 3 of row m = 16t + i
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-        const int m = t * 16 + i;
-        if (m >= M) continue;
-        if (gridDim.y == 1) {
-            TO* o = out + static_cast<size_t>(m) * N + n;
-            if (n + 3 < N && (N % 4 == 0)) {
-                store4<TO>(o, acc[t]);
+    for (int nt = 0; nt < NT; ++nt) {
+        const int n = n0 + nt * 16 + 4 * g;
+        if (n >= N) continue;
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            const int m = t * 16 + i;
+            if (m >= M) continue;
+            if (gridDim.y == 1) {
+                TO* o = out + static_cast<size_t>(m) * N + n;
+                if (n + 3 < N && (N % 4 == 0)) {
+                    store4<TO>(o, acc[nt][t]);
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        if (n + v < N) o[v] = from_float<TO>(acc[nt][t][v]);
+                }
             } else {
+                float* o = partial + (static_cast<size_t>(blockIdx.y) * M + m) * N + n;
+                if (n + 3 < N && (N % 4 == 0)) {
+                    *reinterpret_cast<float4_t*>(o) = acc[nt][t];
+                } else {
 #pragma unroll
-                for (int v = 0; v < 4; ++v)
-                    if (n + v < N) o[v] = from_float<TO>(acc[t][v]);
-            }
-        } else {
-            float* o = partial + (static_cast<size_t>(blockIdx.y) * M + m) * N + n;
-            if (n + 3 < N && (N % 4 == 0)) {
-                *reinterpret_cast<float4_t*>(o) = acc[t];
-            } else {
-#pragma unroll
-                for (int v = 0; v < 4; ++v)
-                    if (n + v < N) o[v] = acc[t][v];
+                    for (int v = 0; v < 4; ++v)
+                        if (n + v < N) o[v] = acc[nt][t][v];
+                }
             }
         }
     }
@@ -140,20 +170,32 @@ WLLM_API int wllm_gemm_skinny(const void* x, const void* w, void* out, int out_b
     const int k_per_split = K / splits;
     if (chunk > k_per_split) chunk = k_per_split;
     const size_t smem = static_cast<size_t>(mt) * 16 * (chunk / 8 + 1) * sizeof(uint4);
-    if (smem > 65536) return -1;
-    const dim3 grid((N + 63) / 64, splits);
-#define LAUNCH(MT, TO)                                                                                       \
-    gemm_skinny_kernel<MT, TO><<<grid, 256, smem, stream>>>(static_cast<const bf16*>(x), static_cast<const bf16*>(w), \
-                                                            static_cast<TO*>(out), partial, M, N, K, k_per_split, chunk)
-#define BY_MT(TO)                    \
-    switch (mt) {                    \
-        case 1: LAUNCH(1, TO); break; \
-        case 2: LAUNCH(2, TO); break; \
-        case 3: LAUNCH(3, TO); break; \
-        default: LAUNCH(4, TO); break; \
+    if (smem > 65536 || mt * 16 * (chunk / 8) > 2048) return -1;     // 8 pieces of x per thread at most
+    // weight rows per wavefront: more when x has many rows, as long as about a thousand wavefronts remain
+    const long long tiles = (N + 15) / 16;
+    int nt = 1;
+    if (mt >= 2) {
+        if (tiles / 4 * splits >= 1024) nt = 4;
+        else if (tiles / 2 * splits >= 1024) nt = 2;
+    }
+    const dim3 grid((N + 64 * nt - 1) / (64 * nt), splits);
+#define LAUNCH(MT, NT, TO)                                                                                   \
+    gemm_skinny_kernel<MT, NT, TO><<<grid, 256, smem, stream>>>(static_cast<const bf16*>(x), static_cast<const bf16*>(w), \
+                                                                static_cast<TO*>(out), partial, M, N, K, k_per_split, chunk)
+#define BY_NT(MT, TO)                    \
+    if (nt == 4) LAUNCH(MT, 4, TO);      \
+    else if (nt == 2) LAUNCH(MT, 2, TO); \
+    else LAUNCH(MT, 1, TO)
+#define BY_MT(TO)                         \
+    switch (mt) {                         \
+        case 1: LAUNCH(1, 1, TO); break;  \
+        case 2: BY_NT(2, TO); break;      \
+        case 3: BY_NT(3, TO); break;      \
+        default: BY_NT(4, TO); break;     \
     }
     if (out_bf16) { BY_MT(bf16) } else { BY_MT(float) }
 #undef BY_MT
+#undef BY_NT
 #undef LAUNCH
     int err = launch_status();
     if (err) return err;
@@ -217,17 +259,32 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
     fetch(curg, curu, 0);
     int step = 0;
     const int tid_half = threadIdx.x % 256;
+    // x is staged chunk by chunk (per half of K); the next chunk's loads are in flight during the products
+    constexpr int kXRegs = 4;                     // MT*16*chunk/8 <= 1024 pieces for 256 threads
+    uint4 xreg[kXRegs];
+    auto fetch_x = [&](int kc) {
+        const int vecs = min(chunk, half_k - kc) / 8;
+#pragma unroll
+        for (int u = 0; u < kXRegs; ++u) {
+            const int idx = tid_half + u * 256;
+            const int m = idx / vecs, c = idx % vecs;
+            xreg[u] = (idx < MT * 16 * vecs && m < M)
+                          ? *reinterpret_cast<const uint4*>(x + static_cast<size_t>(m) * K + k_begin + kc + c * 8)
+                          : make_uint4(0, 0, 0, 0);
+        }
+    };
+    fetch_x(0);
     for (int kc = 0; kc < half_k; kc += chunk) {
         const int len = min(chunk, half_k - kc);
         const int vecs = len / 8;
         __syncthreads();
-        for (int idx = tid_half; idx < MT * 16 * vecs; idx += 256) {
-            const int m = idx / vecs, c = idx % vecs;
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (m < M) v = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(m) * K + k_begin + kc + c * 8);
-            xh[m * stride + c] = v;
+#pragma unroll
+        for (int u = 0; u < kXRegs; ++u) {
+            const int idx = tid_half + u * 256;
+            if (idx < MT * 16 * vecs) xh[(idx / vecs) * stride + idx % vecs] = xreg[u];
         }
         __syncthreads();
+        if (kc + chunk < half_k) fetch_x(kc + chunk);
         for (int k = 0; k < len; k += 32 * kBatch) {
             const int used = min(kBatch, (len - k) / 32);
             fetch(nxtg, nxtu, step + used);
@@ -295,7 +352,7 @@ WLLM_API int wllm_gemm_skinny_gated(const void* x, const void* w, void* out, int
     size_t smem = static_cast<size_t>(2) * mt * 16 * (chunk / 8 + 1) * sizeof(uint4);
     const size_t red = static_cast<size_t>(4) * kWave * mt * 8 * sizeof(float);
     if (red > smem) smem = red;
-    if (smem > 65536) return -1;
+    if (smem > 65536 || mt * 16 * (chunk / 8) > 1024) return -1;     // 4 pieces of x per thread at most
     const dim3 grid((inter + 63) / 64);
 #define LAUNCH(MT, A)                                                                                              \
     gemm_skinny_gated_kernel<MT, A><<<grid, 512, smem, stream>>>(static_cast<const bf16*>(x), static_cast<const bf16*>(w), \
