@@ -59,3 +59,47 @@ def test_replay_matches_plain(models, plain_logits, name, dtype, family):
     assert len(got) == sum(len(t) for t in requests.values())
     worst = compare_with_plain(got, plain_logits[name][dtype], **TOLERANCE[dtype])
     print(f"{name} {dtype} {family}: worst error {worst:.3f} x tolerance")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sharp_attention_over_hundreds_of_keys(model_folders, tmp_path_factory, dtype):
+    """Random weights of the usual size give nearly flat attention, which hides a lost or doubled key.
+    Here the query and key projections are scaled up until each query puts almost all its weight on
+    one or two keys, often far back, over sequences of several hundred tokens cut at page and chunk
+    edges; a wrong key then changes the logits by far more than the tolerance."""
+    import os
+    from wllm_amd.weights import Checkpoint, write_safetensors
+    src = model_folders["M"]
+    folder = str(tmp_path_factory.mktemp("sharp"))
+    ck = Checkpoint(src)
+    tensors = {n: ck.tensor(n) for n in ck.names()}
+    ck.close()
+    for n in tensors:
+        if n.endswith(("q_proj.weight", "k_proj.weight")):
+            tensors[n] = (tensors[n].float() * 6.0).to(torch.bfloat16)
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors)
+    with open(os.path.join(src, "config.json")) as f, open(os.path.join(folder, "config.json"), "w") as g:
+        g.write(f.read())
+    cfg = gemma_plain.read_config(folder)
+    w = gemma_plain.read_weights(folder, torch.float32)
+    requests = {"a": random_ids(71, 400, 1000), "b": random_ids(72, 333, 1000), "c": random_ids(73, 257, 1000)}
+    rounding = torch.bfloat16 if dtype == "bfloat16" else None
+    plain = {rid: gemma_plain.forward_logits(cfg, w, t, scale_rounding=rounding) for rid, t in requests.items()}
+    # the attention really is sharp: the largest probability of a late query is far from 1/400
+    h = gemma_plain.rms_norm_one_plus_w(gemma_plain.embed(torch.tensor(requests["a"]), w["model.embed_tokens.weight"], 128),
+                                        w["model.layers.0.input_layernorm.weight"], 1e-6)
+    q = (h @ w["model.layers.0.self_attn.q_proj.weight"].T).view(400, 8, 64)
+    k = (h @ w["model.layers.0.self_attn.k_proj.weight"].T).view(400, 2, 64)
+    probs = torch.softmax((q[-1, 0] @ k[:, 0].T) / 8.0, -1)
+    assert probs.max() > 0.2
+    model = load_model(folder, dtype, "cuda")
+    # float32 is the sharp comparison.  In bfloat16 the rounding of queries and keys (8 bits) is multiplied
+    # by scores of magnitude 20 before the exponential, so the bound is wider there; a lost key still moves
+    # logits of size 3 by far more.
+    tol = dict(atol=5e-5, rtol=2e-4) if dtype == "float32" else dict(atol=1e-1, rtol=5e-2)
+    for family in (trace_whole, trace_portions, trace_mixed, lambda r: trace_tail(r, tail=40)):
+        trace = family(requests)
+        pages = pages_for_max_tokens(max_live_tokens(trace), 16)
+        runner = ModelRunner.create(model, num_pages=pages, page_size=16, max_requests=4, poison_freed_pages=True)
+        got = replay_and_collect(TraceReplayer(runner), trace)
+        compare_with_plain(got, plain, **tol)

@@ -177,3 +177,18 @@ def test_captured_graphs_give_what_eager_steps_give(model_folders, dtype):
     for a, b in zip(eager, graphed):
         assert a.output_token_ids == b.output_token_ids
         assert torch.allclose(torch.tensor(a.logprobs), torch.tensor(b.logprobs), atol=1e-5 if dtype == "float32" else 2e-2)
+
+
+def test_command_line_generates_what_the_entry_point_generates(model_folders, tmp_path):
+    folder = model_folders["A"]
+    cfg, w = plain_model(folder)
+    prompts = [random_ids(5, 9, 512), random_ids(6, 14, 512)]
+    args = [sys.executable, "-m", "wllm_amd.cli", "generate", "--model", folder, "--dtype", "float32", "--num-blocks", "32",
+            "--block-size", "4", "--max-new-tokens", "6", "--chunked-prefill-tokens", "8"]
+    for p in prompts:
+        args += ["--prompt-ids", ",".join(str(t) for t in p)]
+    proc = subprocess.run(args, capture_output=True, text=True, timeout=300, cwd=ROOT)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = [json.loads(l) for l in proc.stdout.splitlines() if l.startswith("{")]
+    assert [l["token_ids"] for l in lines] == [gemma_plain.generate_greedy(cfg, w, p, 6) for p in prompts]
+    assert all(l["finish_reason"] == "length" for l in lines)

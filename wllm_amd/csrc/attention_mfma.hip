@@ -1,6 +1,7 @@
-// Paged attention on the matrix cores for bfloat16: head sizes 32..256 in steps of 32, pages
-// of a multiple of 4 tokens, any number of heads and groups, optional window.  One kernel serves
-// prompt portions and decoded tokens.
+// Paged attention on the matrix cores for bfloat16, for segments of at most 16 query rows (decoded
+// tokens, and portions short enough): head sizes 32..256 in steps of 32, pages of a multiple of 4
+// tokens, any number of heads and groups, optional window.  Longer segments take the kernel of
+// `attention_prefill.hip`, which shares the products' layout described here.
 //
 // Rows.  For one request (segment) and one key/value head, the query rows are the pairs (token,
 // query head of the group): row r = token * G + head.  All rows of a tile read the same keys and
@@ -9,10 +10,9 @@
 // src/wllm/kernels/csrc/paged_attention.cu:44-45,185).
 //
 // Work items.  The host cuts every (segment, key/value head) into work items, one workgroup of 4
-// wavefronts each: up to 4 tiles of 16 rows, and a range of keys.  With 4 row tiles each
-// wavefront owns a tile and walks all keys; with fewer, the spare wavefronts split the keys and
-// are merged through shared memory.  Segments of at most 16 rows (decoded tokens) are also split
-// over workgroups in fixed chunks of keys; those write partial results (running maximum, sum,
+// wavefronts each: the segment's one tile of 16 rows and a chunk of keys.  The four wavefronts
+// split the chunk's blocks of 32 keys and are merged through shared memory.  A segment with more
+// keys than a chunk is split over workgroups; those write partial results (running maximum, sum,
 // unnormalised accumulator) that `attention_reduce_kernel` combines.  Chunk boundaries depend
 // on the key index only, never on the batch.
 //
@@ -58,7 +58,8 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
     __shared__ float merge_s[2][kRowsPerTile * (HD + 2)];
 
     const int* item = items + static_cast<size_t>(blockIdx.x) * kItemInts;
-    const int seg = item[0], kvh = item[1], row_begin = item[2], row_tiles = item[3];
+    const int seg = item[0], kvh = item[1], row_begin = item[2];
+    constexpr int row_tiles = 1;            // one tile of 16 rows; the four wavefronts split the keys
     const int key_begin = item[4], key_end = item[5], partial_slot = item[6];
     if (seg < 0) return;    // padding item
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;

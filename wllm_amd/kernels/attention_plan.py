@@ -7,7 +7,7 @@ partial results combined by a second kernel; chunk boundaries are multiples of t
 counted from key 0, so they depend on the key index only.  Longer segments are cut into
 workgroups of up to four tiles of 16 rows that each walk all their keys.
 
-A work item is 8 int32: segment, key/value head, first row, row tiles (1, 2 or 4), first key,
+A work item is 8 int32: segment, key/value head, first row, 1 (reserved), first key,
 end key, partial slot (-1: the workgroup writes the final result), unused.  A reduce item is
 4 int32: segment, key/value head, first partial slot, number of splits.  A prefill item (long
 segments, 64 or 128 rows each, for the kernel that stages keys and values through shared memory) is
