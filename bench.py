@@ -121,6 +121,47 @@ def measure_decode(model, batch: int, context: int, steps: int, warmup: int, blo
     return dt, mean_ctx
 
 
+def run_stress(model, args) -> dict:
+    """Continuous batching under pressure: 64 requests at once, prompt lengths uniform in
+    [128, 4096], output lengths uniform in [16, 512] (seeded), prompt portions of at most 512
+    tokens a step beside the decoding requests, temperature 0.7 with per-request seeds, and a page
+    pool too small for all requests together, so that some wait for admission."""
+    import numpy as np
+    import torch
+
+    from wllm_amd.engine import ModelRunner, Request, Scheduler
+    from wllm_amd.sampling import SamplingParams
+    rng = np.random.default_rng(args.seed)
+    n = args.stress_requests
+    prompts = rng.integers(128, 4097, size=n)
+    outputs = rng.integers(16, 513, size=n)
+    vocab = model.plan.embedding.vocab_size
+    need = int(sum(-(-(int(p) + int(o)) // args.block_size) for p, o in zip(prompts, outputs)))
+    pages = max(int(need * args.stress_pool_fraction), -(-4608 // args.block_size) + 1)
+    runner = ModelRunner.create(model, num_pages=pages, page_size=args.block_size, max_requests=n)
+    if not args.no_graphs:
+        runner.enable_graphs()
+    sched = Scheduler(runner, max_prefill_tokens_per_step=512, seed=args.seed)
+    for i in range(n):
+        ids = rng.integers(0, vocab, size=int(prompts[i])).tolist()
+        sched.add_request(Request(i, ids, int(outputs[i]), sampling_params=SamplingParams(temperature=0.7, seed=1000 + i)))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    finished = sched.run_to_completion()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    runner.cache.check()
+    generated = sum(len(r.output_token_ids) for r in finished)
+    assert len(finished) == n and generated == int(outputs.sum())
+    return {"metric": "continuous-batching stress, Gemma-2B layer sizes", "value": round(generated / dt, 1),
+            "unit": "generated tokens/s", "seconds": round(dt, 3), "requests": n, "steps": sched.stats["steps"],
+            "prompt_tokens": int(prompts.sum()), "generated_tokens": generated,
+            "total_tokens_per_s": round((generated + int(prompts.sum())) / dt, 1),
+            "pool_pages": pages, "pages_all_requests_need": need, "peak_pages": sched.stats["peak_pages"],
+            "admission_waits": sched.stats["admission_waits"], "preemptions": sched.stats["preemptions"],
+            "graph_steps": runner.graph_steps, "dtype": args.dtype}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -136,6 +177,11 @@ def main() -> int:
     ap.add_argument("--no-graphs", action="store_true", help="do not replay captured graphs for decode")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--workload", default="decode", choices=["decode", "stress"],
+                    help="decode: the contract's line; stress: continuous batching of 64 mixed requests")
+    ap.add_argument("--stress-requests", type=int, default=64)
+    ap.add_argument("--stress-pool-fraction", type=float, default=0.5,
+                    help="page pool as a fraction of what all requests together would need")
     args = ap.parse_args()
     world = int(os.environ.get("WORLD_SIZE", "1"))
     if args.gpus != 1 or world != 1:
@@ -156,6 +202,9 @@ def main() -> int:
         shape["num_hidden_layers"] = args.layers
     with torch.inference_mode():
         model = build_model(shape, args.dtype, args.seed)
+        if args.workload == "stress":
+            print(json.dumps(run_stress(model, args)))
+            return 0
         graphs = not args.no_graphs
         weight_bytes = model.weight_bytes()
         kv_per_token = kv_bytes_per_token(model)
