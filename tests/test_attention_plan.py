@@ -1,0 +1,99 @@
+"""The host-side plan of the matrix-core attention kernels: every (query row, key) pair that the
+mask allows is covered by exactly one work item, partial slots are held once, and every partial
+result has exactly one reduce item that reads it.  Runs without a GPU: it follows the kernels'
+reading of the items (`wllm_amd/csrc/attention_mfma.hip`, `attention_prefill.hip`)."""
+import numpy as np
+import pytest
+
+from wllm_amd.kernels import attention_plan as ap
+
+
+def covered(q_len, ctx_len, group, nkv, window, page_size):
+    items, reduces, slots, prefill, prefill_rows = ap.build_work_items(
+        np.array(q_len), np.array(ctx_len), group, nkv, window, 0, page_size)
+    cover = {}          # (seg, kvh, row) -> list of (first key, end key, slot)
+    slot_users = {}
+    def hold(slot, who):
+        assert 0 <= slot < slots, (slot, slots)
+        assert slot not in slot_users, f"slot {slot} held by {slot_users[slot]} and {who}"
+        slot_users[slot] = who
+    for n, it in enumerate(items):
+        seg, kvh, row0, _, kb, ke, slot, _ = (int(v) for v in it)
+        rows = q_len[seg] * group
+        assert rows <= 16 and row0 == 0
+        if slot >= 0:
+            hold(slot, ("short", n))
+        for r in range(rows):
+            cover.setdefault((seg, kvh, r), []).append((kb, ke, slot))
+    for n, it in enumerate(prefill):
+        seg, kvh, row0, kb, ke, slot = (int(v) for v in it[:6])
+        rows = q_len[seg] * group
+        assert rows > 16 and row0 % prefill_rows == 0 and row0 < rows
+        first_pos = ctx_len[seg] - q_len[seg]
+        last = min(rows - 1, row0 + prefill_rows - 1)
+        b_hi = first_pos + last // group + 1
+        b_lo = max(0, first_pos + row0 // group - window + 1) if window > 0 else 0
+        lo, hi = max(b_lo, kb), min(b_hi, ke)
+        assert lo < hi, "an item without keys"
+        assert kb % 32 == 0 and ke % 32 == 0
+        first_page, last_page = (lo // 32 * 32) // page_size, (min(-(-hi // 32) * 32, ctx_len[seg]) - 1) // page_size
+        assert last_page - first_page + 1 <= ap.PREFILL_TABLE_PAGES
+        for tile in range(prefill_rows // 16):
+            if slot >= 0 and row0 + 16 * tile < rows:
+                hold(slot + tile, ("prefill", n, tile))
+        for r in range(row0, last + 1):
+            cover.setdefault((seg, kvh, r), []).append((lo, hi, slot + (r - row0) // 16 if slot >= 0 else -1))
+    reduce_of = {}
+    for it in reduces:
+        seg, kvh, first, splits, row0, stride = (int(v) for v in it[:6])
+        for r in range(row0, min(row0 + 16, q_len[seg] * group)):
+            assert (seg, kvh, r) not in reduce_of
+            reduce_of[(seg, kvh, r)] = {first + j * stride for j in range(splits)}
+    for seg in range(len(q_len)):
+        first_pos = ctx_len[seg] - q_len[seg]
+        for kvh in range(nkv):
+            for r in range(q_len[seg] * group):
+                pos = first_pos + r // group
+                lo = max(0, pos - window + 1) if window > 0 else 0
+                pieces = sorted(cover[(seg, kvh, r)])
+                # pieces are disjoint, in order, and hold every key lo..pos
+                assert pieces[0][0] <= lo and pieces[-1][1] > pos, (seg, kvh, r, pieces, lo, pos)
+                for a, b in zip(pieces, pieces[1:]):
+                    assert a[1] == b[0], (seg, kvh, r, pieces)
+                if len(pieces) == 1 and pieces[0][2] < 0:
+                    assert (seg, kvh, r) not in reduce_of
+                else:
+                    assert all(p[2] >= 0 for p in pieces)
+                    assert reduce_of[(seg, kvh, r)] == {p[2] for p in pieces}
+    assert len(slot_users) <= slots      # tiles beyond a segment's last row leave their slots unused
+    return items, reduces, slots, prefill
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_every_pair_is_covered_once(seed, monkeypatch):
+    rng = np.random.default_rng(seed)
+    # small targets so that small cases split the way large ones do
+    monkeypatch.setattr(ap, "PREFILL_MIN_CHUNK", 128)
+    monkeypatch.setattr(ap, "PREFILL_TARGET_ITEMS", int(rng.choice([1, 8, 64, 1024])))
+    monkeypatch.setattr(ap, "PREFILL_TABLE_PAGES", int(rng.choice([34, 1024])))
+    group, nkv = int(rng.choice([1, 2, 3, 8])), int(rng.choice([1, 2, 3]))
+    window = int(rng.choice([0, 0, 40, 300]))
+    page_size = int(rng.choice([4, 12, 16, 64]))
+    n = int(rng.integers(1, 5))
+    q_len = [int(rng.choice([1, 2, 5, 17, 70, 130, 400])) for _ in range(n)]
+    ctx_len = [q + int(rng.choice([0, 1, 31, 128, 500, 1500])) for q in q_len]
+    covered(q_len, ctx_len, group, nkv, window, page_size)
+
+
+def test_a_late_portion_of_a_long_prompt_is_split_over_the_keys():
+    # 512 tokens at the end of 2,560, 8 query heads on one key/value head: 64 blocks of rows alone
+    # would leave most compute units idle
+    _, reduces, slots, prefill = covered([512], [2560], 8, 1, 0, 16)
+    assert prefill.shape[0] >= 256
+    assert slots > 0 and reduces.shape[0] == 512 * 8 // 16
+
+
+def test_a_whole_prompt_of_many_heads_is_not_split():
+    _, reduces, slots, prefill = covered([300], [300], 1, 1, 0, 16)
+    assert slots == 0 and reduces.shape[0] == 0
+    assert (prefill[:, 5] == -1).all()

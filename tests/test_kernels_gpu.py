@@ -232,6 +232,27 @@ MFMA_SHAPES = ATTENTION_SHAPES + [
 @pytest.mark.parametrize("nh,nkv,d,ps,segs,window", MFMA_SHAPES)
 def test_paged_attention_matrix_cores(nh, nkv, d, ps, segs, window):
     """The bfloat16 kernel the engine uses for these sizes (with its plan of work items)."""
+    _check_matrix_cores(nh, nkv, d, ps, segs, window)
+
+
+@pytest.mark.parametrize("nh,nkv,d,ps,segs,window,small_pieces", [
+    (8, 1, 256, 16, [(512, 2560)], 0, False),          # a late portion of a long prompt: split as the engine splits it
+    (8, 1, 256, 16, [(200, 900), (1, 70)], 0, True),
+    (8, 2, 64, 8, [(40, 700), (1, 300), (70, 70)], 150, True),
+    (6, 2, 96, 4, [(100, 400), (9, 500)], 0, True),
+    (5, 5, 32, 12, [(130, 333)], 0, True),
+])
+def test_prompt_portions_whose_keys_are_split_over_workgroups(nh, nkv, d, ps, segs, window, small_pieces, monkeypatch):
+    """Blocks of rows whose keys are cut into pieces, each piece a workgroup, combined by the reduce kernel."""
+    from wllm_amd.kernels import attention_plan
+    if small_pieces:       # pieces of 128 keys, so that small cases are cut the way large ones are
+        monkeypatch.setattr(attention_plan, "PREFILL_MIN_CHUNK", 128)
+    plan = _check_matrix_cores(nh, nkv, d, ps, segs, window)
+    assert plan.num_prefill > 0 and plan.num_reduce > 0
+    assert int((plan.prefill_items[:, 5] >= 0).sum()) > 0, "no block of rows was split"
+
+
+def _check_matrix_cores(nh, nkv, d, ps, segs, window):
     dtype = torch.bfloat16
     args, kwargs = _attention_case(dtype, nh, nkv, d, ps, segs, window, seed=11)
     ref_args = [a.clone() for a in args]
@@ -254,6 +275,7 @@ def test_paged_attention_matrix_cores(nh, nkv, d, ps, segs, window):
         ops.paged_attention(*ref_args, **kwargs)
     assert torch.isfinite(args[7].float()).all()
     close(args[7], ref_args[7], dtype, "attention output")
+    return kw["plan"]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -276,7 +276,7 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
 }
 
 // Combines the partial results of a (segment, key/value head) whose keys were split over workgroups.
-// reduce items: seg, kvh, first partial slot, number of splits.
+// reduce items: seg, kvh, first partial slot, number of splits, first row, slots between splits, 2 unused.
 template <int HD>
 __global__ void __launch_bounds__(HD)
 attention_reduce_kernel(const int* __restrict__ reduce_items, const float* __restrict__ partial_o,
@@ -284,26 +284,29 @@ attention_reduce_kernel(const int* __restrict__ reduce_items, const float* __res
                         const int* __restrict__ seg_q_len, bf16* __restrict__ out, int num_heads, int num_kv_heads,
                         float scale_log2e) {
     // one workgroup per (item, row); one thread per element of the head; the loads of the
-    // splits do not depend on each other
-    const int* item = reduce_items + static_cast<size_t>(blockIdx.x) * 4;
-    const int seg = item[0], kvh = item[1], first = item[2], splits = item[3];
+    // splits do not depend on each other.  Reduce items are 8 int32: segment, key/value head, first
+    // slot, number of splits, first row of the tile within the segment, slots between two splits.
+    const int* item = reduce_items + static_cast<size_t>(blockIdx.x) * kItemInts;
+    const int seg = item[0], kvh = item[1], first = item[2], splits = item[3], row0 = item[4];
     if (seg < 0) return;
+    const size_t stride = static_cast<size_t>(item[5]) * kRowsPerTile;     // rows between two splits
     const int group = num_heads / num_kv_heads;
     const int r = blockIdx.y, d = threadIdx.x;
-    if (r >= seg_q_len[seg] * group) return;       // at most 16 rows
+    if (row0 + r >= seg_q_len[seg] * group) return;
     const float* ml = partial_ml + (static_cast<size_t>(first) * kRowsPerTile + r) * 2;
     const float* po = partial_o + (static_cast<size_t>(first) * kRowsPerTile + r) * HD + d;
     float m = -INFINITY;
-    for (int s = 0; s < splits; ++s) m = fmaxf(m, ml[static_cast<size_t>(s) * kRowsPerTile * 2]);
+    for (int s = 0; s < splits; ++s) m = fmaxf(m, ml[s * stride * 2]);
     float num = 0.f, den = 0.f;
 #pragma unroll 4
     for (int s = 0; s < splits; ++s) {
-        const float ms = ml[static_cast<size_t>(s) * kRowsPerTile * 2];
+        const float ms = ml[s * stride * 2];
         const float f = ms == -INFINITY ? 0.f : exp2f((ms - m) * scale_log2e);
-        num = fmaf(po[static_cast<size_t>(s) * kRowsPerTile * HD], f, num);
-        den = fmaf(ml[static_cast<size_t>(s) * kRowsPerTile * 2 + 1], f, den);
+        num = fmaf(po[s * stride * HD], f, num);
+        den = fmaf(ml[s * stride * 2 + 1], f, den);
     }
-    const int tok = r / group, head = kvh * group + r % group;
+    const int row = row0 + r;
+    const int tok = row / group, head = kvh * group + row % group;
     out[(static_cast<size_t>(seg_q_start[seg] + tok) * num_heads + head) * HD + d] = from_float<bf16>(num / den);
 }
 

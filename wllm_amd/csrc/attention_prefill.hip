@@ -20,7 +20,8 @@ typedef float float4_t __attribute__((ext_vector_type(4)));
 constexpr int kPrefillWaves = 4;       // wavefronts per workgroup
 constexpr int kPrefillThreads = kPrefillWaves * 64;
 constexpr int kBlockKeys = 32;
-constexpr int kMaxTablePages = 4096;
+constexpr int kMaxTablePages = 1024;     // pages one work item's keys may span (the host cuts items to fit)
+constexpr int kPrefillItemInts = 8;
 
 union PPack {
     uint4 u;
@@ -36,22 +37,27 @@ struct PrefillSmem {
     static constexpr int kBytes = (kBlockKeys * kStrideK + HD * kStrideV) * 2;
 };
 
-// prefill items: seg, kvh, first row, unused
+// prefill items: seg, kvh, first row, first key, end key, partial slot (-1: the workgroup walks all
+// the keys of its rows and writes the result itself), 2 unused.  Items that split the keys of a
+// block of rows write, per tile of 16 rows, an unnormalised accumulator and (maximum, sum) into
+// slot `partial slot + tile`, which `attention_reduce_kernel` combines.
 template <int HD, int RTW>      // RTW: tiles of 16 rows per wavefront (1 or 2)
 __global__ void __launch_bounds__(kPrefillThreads)
 paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restrict__ cache,
                                const int* __restrict__ block_tables, const int* __restrict__ items,
                                const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
-                               const int* __restrict__ seg_ctx_len, bf16* __restrict__ out, int num_heads,
+                               const int* __restrict__ seg_ctx_len, bf16* __restrict__ out,
+                               float* __restrict__ partial_o, float* __restrict__ partial_ml, int num_heads,
                                int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window) {
     constexpr int DC = HD / 32, DT = HD / 16;
     constexpr int SK = PrefillSmem<HD>::kStrideK, SV = PrefillSmem<HD>::kStrideV;
     __shared__ __align__(16) uint16_t k_s[kBlockKeys * SK];
     __shared__ __align__(16) uint16_t v_s[HD * SV];
-    __shared__ int table_s[kMaxTablePages];     // the request's block table: page lookups never leave the CU
+    __shared__ int table_s[kMaxTablePages];     // the pages of this item's keys: lookups never leave the CU
 
-    const int* item = items + static_cast<size_t>(blockIdx.x) * 4;
+    const int* item = items + static_cast<size_t>(blockIdx.x) * kPrefillItemInts;
     const int seg = item[0], kvh = item[1], row_begin = item[2];
+    const int key_begin = item[3], key_end = item[4], partial_slot = item[5];
     if (seg < 0) return;
     const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
     const int i = lane % 16, g = lane / 16;
@@ -64,12 +70,6 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
     const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * HD;
     const size_t k_off = static_cast<size_t>(kvh) * page_size * HD;
     const size_t v_off = (static_cast<size_t>(num_kv_heads) + kvh) * page_size * HD;
-    {
-        const int* table_g = block_tables + static_cast<size_t>(seg) * max_pages;
-        const int pages_used = min(max_pages, (ctx + page_size - 1) / page_size);
-        for (int p = tid; p < pages_used; p += kPrefillThreads) table_s[p] = table_g[p];
-    }
-    const int* table = table_s;
 
     // this wavefront's two tiles of rows
     constexpr int kWaveRows = 16 * RTW, kPrefillRows = kPrefillWaves * kWaveRows;
@@ -112,7 +112,16 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
     const int b_last_row = min(total_rows - 1, row_begin + kPrefillRows - 1);
     const int b_hi = first_pos + b_last_row / group + 1;
     const int b_lo = window > 0 ? max(0, first_pos + row_begin / group - window + 1) : 0;
-    const int blk_first = b_lo / kBlockKeys, blk_end = (b_hi + kBlockKeys - 1) / kBlockKeys;
+    const int blk_first = max(b_lo, key_begin) / kBlockKeys;
+    const int blk_end = (min(b_hi, key_end) + kBlockKeys - 1) / kBlockKeys;
+    // the pages of keys blk_first * 32 .. blk_end * 32 (clamped to the request's keys)
+    const int page_base = blk_first * kBlockKeys / page_size;
+    if (blk_first < blk_end) {
+        const int* table_g = block_tables + static_cast<size_t>(seg) * max_pages + page_base;
+        const int page_last = (min(blk_end * kBlockKeys, ctx) - 1) / page_size;
+        const int count = min(min(max_pages - 1, page_last) - page_base + 1, kMaxTablePages);
+        for (int p = tid; p < count; p += kPrefillThreads) table_s[p] = table_g[p];
+    }
 
     float4_t acc[RTW][DT];
     float m_run[RTW], l_run[RTW];
@@ -139,10 +148,10 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
     auto page_of = [&](int key, int& slot) -> int {
         if (page_shift >= 0) {
             slot = key & (page_size - 1);
-            return table[key >> page_shift];
+            return table_s[(key >> page_shift) - page_base];
         }
         slot = key % page_size;
-        return table[key / page_size];
+        return table_s[key / page_size - page_base];
     };
     auto fetch = [&](uint4* kreg, uint2* vreg, int kbase) {
         {
@@ -281,6 +290,17 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
         l += __shfl_xor(l, 16, kWave);
         l += __shfl_xor(l, 32, kWave);
         if (!row_valid[rt]) continue;
+        if (partial_slot >= 0) {
+            // one slot per tile of 16 rows: [16][HD] accumulators and [16][2] (maximum, sum)
+            const size_t slot = static_cast<size_t>(partial_slot) + wave * RTW + rt;
+            float* po = partial_o + (slot * 16 + i) * HD;
+#pragma unroll
+            for (int t = 0; t < DT; ++t)
+                *reinterpret_cast<float4*>(po + t * 16 + 4 * g) =
+                    make_float4(acc[rt][t][0], acc[rt][t][1], acc[rt][t][2], acc[rt][t][3]);
+            if (g == 0) *reinterpret_cast<float2*>(partial_ml + (slot * 16 + i) * 2) = make_float2(m_run[rt], l);
+            continue;
+        }
         const float inv = 1.f / l;
         bf16* orow = out + (static_cast<size_t>(q_start + tok[rt]) * num_heads + head[rt]) * HD;
 #pragma unroll
@@ -296,19 +316,20 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
 // Returns 0, a HIP error code, or -1 for sizes this kernel does not take.
 WLLM_API int wllm_paged_attention_prefill(const void* qkv, const void* cache, const int* block_tables,
                                           const int* items, int num_items, int rows_per_item, const int* seg_q_start,
-                                          const int* seg_q_len, const int* seg_ctx_len, void* out, int num_heads,
+                                          const int* seg_q_len, const int* seg_ctx_len, void* out, float* partial_o,
+                                          float* partial_ml, int num_heads,
                                           int num_kv_heads, int head_dim, int page_size, int max_pages, float scale,
                                           int window, hipStream_t stream) {
     if (head_dim % 32 != 0 || head_dim < 32 || head_dim > 256 || page_size % 4 != 0 || num_heads % num_kv_heads != 0)
         return -1;
-    if (max_pages > kMaxTablePages) return -1;       // the block table must fit the kernel's shared copy
     if (rows_per_item != 64 && rows_per_item != 128) return -1;
     if (num_items <= 0) return 0;
     const float scale_log2e = scale * 1.4426950408889634f;
 #define LAUNCH_RTW(HD, RTW)                                                                                         \
     paged_attention_prefill_kernel<HD, RTW><<<num_items, kPrefillThreads, 0, stream>>>(                             \
         static_cast<const bf16*>(qkv), static_cast<const bf16*>(cache), block_tables, items, seg_q_start, seg_q_len, \
-        seg_ctx_len, static_cast<bf16*>(out), num_heads, num_kv_heads, page_size, max_pages, scale_log2e, window)
+        seg_ctx_len, static_cast<bf16*>(out), partial_o, partial_ml, num_heads, num_kv_heads, page_size, max_pages, \
+        scale_log2e, window)
 #define LAUNCH(HD)                            \
     if (rows_per_item == 64) LAUNCH_RTW(HD, 1); \
     else LAUNCH_RTW(HD, 2)

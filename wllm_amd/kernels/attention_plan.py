@@ -8,10 +8,15 @@ counted from key 0, so they depend on the key index only.  Longer segments are c
 workgroups of up to four tiles of 16 rows that each walk all their keys.
 
 A work item is 8 int32: segment, key/value head, first row, 1 (reserved), first key,
-end key, partial slot (-1: the workgroup writes the final result), unused.  A reduce item is
-4 int32: segment, key/value head, first partial slot, number of splits.  A prefill item (long
+end key, partial slot (-1: the workgroup writes the final result), unused.  A partial slot holds
+one tile of 16 rows.  A reduce item is 8 int32: segment, key/value head, first partial slot, number
+of splits, first row of the tile, slots between two splits, 2 unused.  A prefill item (long
 segments, 64 or 128 rows each, for the kernel that stages keys and values through shared memory) is
-4 int32: segment, key/value head, first row, unused.
+8 int32: segment, key/value head, first row, first key, end key, partial slot (-1: final), 2
+unused.  The keys of a block of rows are split over several prefill items when the step has too
+few blocks to fill the compute units (a portion of a prompt late in a long context) or when they
+span more pages than the kernel's shared copy of the block table holds; the pieces of a block are
+equal and begin at multiples of 32 keys.
 """
 from __future__ import annotations
 
@@ -24,18 +29,23 @@ import torch
 KEY_CHUNK = 128
 ROWS_PER_TILE = 16
 ITEM_INTS = 8
+PREFILL_TABLE_PAGES = 1024      # pages one prefill item may span (the kernel's shared block table)
+PREFILL_TARGET_ITEMS = 1024     # prefill items wanted in a step: about four for each compute unit
+PREFILL_MIN_CHUNK = 256         # keys; smaller pieces cost more in partial results than they gain
+PREFILL_WIDE_SPAN = 131072      # keys walked by all blocks of 128 rows together from which on a workgroup
+                                # takes 128 rows (more reuse of staged keys) instead of 64 (more workgroups)
 
 
 @dataclass
 class AttentionPlan:
     items: torch.Tensor                 # int32 [num_items, 8] on the device
-    reduce_items: Optional[torch.Tensor]  # int32 [num_reduce, 4] or None
+    reduce_items: Optional[torch.Tensor]  # int32 [num_reduce, 8] or None
     num_items: int
     num_reduce: int
     num_partial_slots: int
     partial_o: Optional[torch.Tensor] = None    # float32 [slots * 16 * head_dim]
     partial_ml: Optional[torch.Tensor] = None   # float32 [slots * 16 * 2]
-    prefill_items: Optional[torch.Tensor] = None  # int32 [num_prefill, 4]
+    prefill_items: Optional[torch.Tensor] = None  # int32 [num_prefill, 8]
     num_prefill: int = 0
     prefill_rows: int = 64
 
@@ -49,11 +59,11 @@ class StaticAttentionPlan(AttentionPlan):
     def __init__(self, segments: int, group: int, num_kv_heads: int, window: int, fixed_splits: int,
                  max_slots: int, head_dim: int, device):
         n_i, n_r = segments * num_kv_heads * fixed_splits, segments * num_kv_heads
-        self._host = torch.empty(n_i * ITEM_INTS + n_r * 4, dtype=torch.int32, pin_memory=True)
+        self._host = torch.empty((n_i + n_r) * ITEM_INTS, dtype=torch.int32, pin_memory=True)
         self._dev = torch.empty_like(self._host, device=device)
         self._args = (group, num_kv_heads, window, fixed_splits)
         self.max_slots = max_slots
-        super().__init__(self._dev[:n_i * ITEM_INTS].view(n_i, ITEM_INTS), self._dev[n_i * ITEM_INTS:].view(n_r, 4),
+        super().__init__(self._dev[:n_i * ITEM_INTS].view(n_i, ITEM_INTS), self._dev[n_i * ITEM_INTS:].view(n_r, ITEM_INTS),
                          n_i, n_r, max_slots,
                          torch.empty(max(1, max_slots) * ROWS_PER_TILE * head_dim, dtype=torch.float32, device=device),
                          torch.empty(max(1, max_slots) * ROWS_PER_TILE * 2, dtype=torch.float32, device=device))
@@ -72,8 +82,9 @@ class StaticAttentionPlan(AttentionPlan):
 
 
 def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_heads: int, window: int,
-                     fixed_splits: int = 0):
-    """Returns (items [n, 8], reduce_items [m, 4], partial slots, prefill items [p, 4]) as int32 arrays.
+                     fixed_splits: int = 0, page_size: int = 16):
+    """Returns (items [n, 8], reduce_items [m, 8], partial slots, prefill items [p, 8], rows per
+    prefill item) as int32 arrays.
 
     `fixed_splits` > 0 gives every short segment exactly that many items per key/value head
     (items beyond the segment's keys are padding that the kernel skips), so that the number
@@ -123,27 +134,79 @@ def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_
         items.append(it[keep].reshape(-1, ITEM_INTS))
         split_seg = ~single
         if split_seg.any():
-            rs = np.zeros((S, num_kv_heads, 4), dtype=np.int32)
+            rs = np.zeros((S, num_kv_heads, ITEM_INTS), dtype=np.int32)
             rs[..., 0] = idx[:, None]
             rs[..., 1] = kv[None, :]
             rs[..., 2] = seg_base[:, None] + kv[None, :] * n_split_seg[:, None]
             rs[..., 3] = ns[:, None]
-            reduces.append(rs[split_seg].reshape(-1, 4))
+            rs[..., 4] = 0
+            rs[..., 5] = 1
+            reduces.append(rs[split_seg].reshape(-1, ITEM_INTS))
         slots = int((n_split_seg * num_kv_heads).sum())
-    # ---- long segments: workgroups of 64 or 128 rows that walk all their keys ----
+    # ---- long segments: workgroups of 64 or 128 rows of one key/value head ----
     prefill = []
-    long_rows = rows[~short]
-    # 128 rows a workgroup when that still gives every compute unit two workgroups, else 64
-    prefill_rows = 128 if int((-(-long_rows // 128)).sum()) * num_kv_heads >= 512 else 64
-    for s in np.nonzero(~short)[0]:
-        blocks = -(-int(rows[s]) // prefill_rows)
-        it = np.zeros((blocks, num_kv_heads, 4), dtype=np.int32)
-        it[..., 0] = s
-        it[..., 1] = kv[None, :]
-        it[..., 2] = (np.arange(blocks, dtype=np.int32) * prefill_rows)[:, None]
-        # the last rows see the most keys: start them first
-        prefill.append(it[::-1].reshape(-1, 4))
-    prefill = np.concatenate(prefill) if prefill else np.zeros((0, 4), np.int32)
+    long_idx = np.nonzero(~short)[0]
+    prefill_rows = 64
+    if long_idx.size:
+        for prefill_rows in (128, 64):
+            blocks = []              # (segment, first rows, lowest key, end key) per long segment
+            span_total = 0
+            for s in long_idx:
+                n_blocks = -(-int(rows[s]) // prefill_rows)
+                rb = np.arange(n_blocks, dtype=np.int64) * prefill_rows
+                first_pos = int(ctx_len[s] - q_len[s])
+                hi = first_pos + np.minimum(rows[s] - 1, rb + prefill_rows - 1) // group + 1
+                lo = np.maximum(0, first_pos + rb // group - window + 1) if window > 0 else np.zeros_like(rb)
+                blocks.append((int(s), rb, lo, hi))
+                span_total += int((hi - lo).sum()) * num_kv_heads
+            if span_total >= PREFILL_WIDE_SPAN:
+                break
+        tiles = prefill_rows // ROWS_PER_TILE
+        # a piece that starts inside a page touches up to two pages more than its keys fill
+        max_chunk = max(KEY_CHUNK, (PREFILL_TABLE_PAGES - 2) * page_size // KEY_CHUNK * KEY_CHUNK)
+        chunk = -(-span_total // (PREFILL_TARGET_ITEMS * KEY_CHUNK)) * KEY_CHUNK
+        chunk = min(max(chunk, PREFILL_MIN_CHUNK), max_chunk)
+        for s, rb, lo, hi in blocks:
+            # a block's keys are cut into pieces of about `chunk` keys, equal within the block,
+            # whose boundaries are multiples of 32 counted from the block's first group of 32
+            lo32 = lo // 32 * 32
+            span = hi - lo32
+            ns = np.maximum(np.maximum(1, (span + chunk // 2) // chunk), -(-span // max_chunk))   # items per block
+            piece = -(-span // (ns * 32)) * 32
+            ns = -(-span // piece)
+            n_items = int(ns.sum())
+            block_of = np.repeat(np.arange(rb.size), ns)
+            j = np.arange(n_items) - np.repeat(np.cumsum(ns) - ns, ns)
+            split = ns > 1
+            # slots of a split block: [split][tile], blocks one after the other, per key/value head
+            block_slots = np.where(split, ns * tiles, 0)
+            block_base = np.cumsum(block_slots) - block_slots
+            per_head = int(block_slots.sum())
+            it = np.zeros((num_kv_heads, n_items, ITEM_INTS), dtype=np.int32)
+            it[..., 0] = s
+            it[..., 1] = kv[:, None]
+            it[..., 2] = rb[block_of][None, :]
+            it[..., 3] = (lo32[block_of] + j * piece[block_of])[None, :]
+            it[..., 4] = (lo32[block_of] + (j + 1) * piece[block_of])[None, :]
+            slot = slots + kv[:, None] * per_head + (block_base[block_of] + j * tiles)[None, :]
+            it[..., 5] = np.where(split[block_of][None, :], slot, -1)
+            # the last rows see the most keys: start them first
+            prefill.append(it[:, ::-1].reshape(-1, ITEM_INTS))
+            sb = np.nonzero(split)[0]
+            if sb.size:
+                t = np.arange(tiles, dtype=np.int64)
+                first_row = rb[sb][:, None] + t[None, :] * ROWS_PER_TILE           # [blocks, tiles]
+                live = first_row < rows[s]
+                rs = np.zeros((num_kv_heads, sb.size, tiles, ITEM_INTS), dtype=np.int32)
+                rs[..., 0] = s
+                rs[..., 1] = kv[:, None, None]
+                rs[..., 2] = slots + kv[:, None, None] * per_head + (block_base[sb][:, None] + t[None, :])[None]
+                rs[..., 3] = ns[sb][None, :, None]
+                rs[..., 4] = first_row[None]
+                rs[..., 5] = tiles
+                reduces.append(rs[:, live].reshape(-1, ITEM_INTS))
+            slots += per_head * num_kv_heads
+    prefill = np.concatenate(prefill) if prefill else np.zeros((0, ITEM_INTS), np.int32)
     items = np.concatenate(items) if items else np.zeros((0, ITEM_INTS), np.int32)
-    reduces = np.concatenate(reduces) if reduces else np.zeros((0, 4), np.int32)
+    reduces = np.concatenate(reduces) if reduces else np.zeros((0, ITEM_INTS), np.int32)
     return items, reduces, slots, prefill, prefill_rows

@@ -35,7 +35,8 @@ _SIGNATURES = {
                                   c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
                                   c_int, c_void_p],
     "wllm_paged_attention_prefill": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
-                                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+                                     c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
+                                     c_void_p],
     "wllm_gemm_generic": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_argmax_rows": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "wllm_gemm_skinny": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
@@ -110,14 +111,14 @@ class HipBackend:
         if not self.mfma_attention_takes(dtype, head_dim, page_size):
             return None
         items, reduces, slots, prefill, prefill_rows = build_work_items(
-            host_q_len, host_ctx_len, num_heads // num_kv_heads, num_kv_heads, window, fixed_splits)
+            host_q_len, host_ctx_len, num_heads // num_kv_heads, num_kv_heads, window, fixed_splits, page_size)
         flat = np.concatenate([items.reshape(-1), reduces.reshape(-1), prefill.reshape(-1)])
         dev = torch.from_numpy(flat).to(device, non_blocking=True)
         n_i, n_r, n_p = items.shape[0], reduces.shape[0], prefill.shape[0]
         self._ensure_partials(slots, head_dim, device)
-        a, b = n_i * 8, n_i * 8 + n_r * 4
-        return AttentionPlan(dev[:a].view(n_i, 8), dev[a:b].view(n_r, 4) if n_r else None, n_i, n_r, slots,
-                             self._partial_o, self._partial_ml, dev[b:].view(n_p, 4) if n_p else None, n_p,
+        a, b = n_i * 8, (n_i + n_r) * 8
+        return AttentionPlan(dev[:a].view(n_i, 8), dev[a:b].view(n_r, 8) if n_r else None, n_i, n_r, slots,
+                             self._partial_o, self._partial_ml, dev[b:].view(n_p, 8) if n_p else None, n_p,
                              prefill_rows)
 
     def static_attention_plan(self, segments, num_heads, num_kv_heads, head_dim, page_size, window, dtype, device,
@@ -150,10 +151,11 @@ class HipBackend:
                 self._check(self.lib.wllm_paged_attention_prefill(
                     _ptr(qkv), _ptr(cache), _ptr(block_tables), _ptr(plan.prefill_items), plan.num_prefill,
                     plan.prefill_rows,
-                    _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out), num_heads, num_kv_heads,
+                    _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out), _ptr(plan.partial_o),
+                    _ptr(plan.partial_ml), num_heads, num_kv_heads,
                     head_dim, page_size, block_tables.shape[1], scale, window, self._stream()),
                     "paged_attention (prompt portions, matrix cores)")
-            if plan.num_items == 0:
+            if plan.num_items == 0 and plan.num_reduce == 0:
                 return
             self._check(self.lib.wllm_paged_attention_mfma(
                 _ptr(qkv), _ptr(cache), _ptr(block_tables), _ptr(plan.items), plan.num_items, _ptr(plan.reduce_items),
