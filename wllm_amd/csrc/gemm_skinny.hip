@@ -166,6 +166,8 @@ WLLM_API int wllm_gemm_skinny(const void* x, const void* w, void* out, int out_b
                               int K, int splits, int chunk, hipStream_t stream) {
     if (M < 1 || M > 64 || K % 32 != 0 || splits < 1 || K % splits != 0 || (K / splits) % 32 != 0 || chunk % 32 != 0)
         return -1;
+    // every result needs somewhere to go: a split product its partial sums, an unsplit one its output
+    if ((splits > 1 && partial == nullptr) || (splits == 1 && out == nullptr)) return -1;
     const int mt = (M + 15) / 16;
     const int k_per_split = K / splits;
     if (chunk > k_per_split) chunk = k_per_split;
