@@ -34,7 +34,8 @@ def build_model(shape: dict, dtype: str, seed: int):
     from wllm_amd.weights.random_init import RandomFetcher
     model = build(shape)
     tdt = {"bf16": torch.bfloat16, "fp32": torch.float32}[dtype]
-    model.load_from(RandomFetcher(model.expected_tensors(), seed, tdt, "cuda:0", std=0.02, norm_std=0.1))
+    model.load_from(RandomFetcher(model.expected_tensors(), seed, tdt, "cuda:0", std=0.02, norm_std=0.1,
+                                  tiled_copies=tdt == torch.bfloat16))
     return model
 
 
@@ -97,7 +98,7 @@ def measure_decode(model, batch: int, context: int, steps: int, warmup: int, blo
     runner = ModelRunner.create(model, num_pages=pages, page_size=block_size, max_requests=batch)
     if hip_graphs and hasattr(runner, "enable_graphs"):
         runner.enable_graphs()
-    sched = Scheduler(runner, max_prefill_tokens_per_step=chunk, compute_logprobs=False)
+    sched = Scheduler(runner, max_prefill_tokens_per_step=chunk, compute_logprobs=False, lookahead=True)
     g = torch.Generator().manual_seed(2)
     vocab = model.plan.embedding.vocab_size
     for i in range(batch):
@@ -141,7 +142,7 @@ def run_stress(model, args) -> dict:
     runner = ModelRunner.create(model, num_pages=pages, page_size=args.block_size, max_requests=n)
     if not args.no_graphs:
         runner.enable_graphs()
-    sched = Scheduler(runner, max_prefill_tokens_per_step=512, seed=args.seed)
+    sched = Scheduler(runner, max_prefill_tokens_per_step=512, seed=args.seed, lookahead=True)
     for i in range(n):
         ids = rng.integers(0, vocab, size=int(prompts[i])).tolist()
         sched.add_request(Request(i, ids, int(outputs[i]), sampling_params=SamplingParams(temperature=0.7, seed=1000 + i)))

@@ -27,6 +27,12 @@ class EmulatedKernels:
         self._count("embed_lookup")
         out.copy_((table[ids.long()].to(self.acc) * scale).to(out.dtype))
 
+    def feed_tokens(self, ids, dst, src, source):
+        self._count("feed_tokens")
+        for d, s in zip(dst.tolist(), src.tolist()):
+            if 0 <= d < ids.shape[0] and 0 <= s < source.shape[0]:
+                ids[d] = source[s]
+
     def rms_norm(self, x, weight, eps, offset, out, delta, rows):
         self._count("rms_norm")
         if delta is not None and delta.dim() == 3:
@@ -125,8 +131,26 @@ class EmulatedKernels:
     def linear_splits(self, rows, out_features, in_features, dtype):
         return self.splits
 
-    def linear(self, x, weight, out):
+    def tile_weight(self, weight, tiles):
+        """[n, k] -> [band][step][g][i][8]: lane 16g + i of a wavefront holds w[16 band + i][32 step + 8g .. +8]."""
+        n, k = weight.shape
+        padded = torch.zeros(-(-n // 16) * 16, k, dtype=weight.dtype, device=weight.device)
+        padded[:n] = weight
+        tiles.copy_(padded.view(-1, 16, k // 32, 4, 8).permute(0, 2, 3, 1, 4).reshape(-1))
+
+    def _same_numbers(self, weight, tiles, halves):
+        """A tile-major copy must hold the weight's numbers: the emulation computes from the weight."""
+        if tiles is None:
+            return
+        n, k = weight.shape[0] // halves, weight.shape[1]
+        size = -(-n // 16) * 16 * k
+        for h in range(halves):
+            back = tiles[h * size:(h + 1) * size].view(-1, k // 32, 4, 16, 8).permute(0, 3, 1, 2, 4).reshape(-1, k)[:n]
+            assert torch.equal(back, weight[h * n:(h + 1) * n]), "the tile-major copy differs from the weight"
+
+    def linear(self, x, weight, out, tiles=None):
         self._count("linear")
+        self._same_numbers(weight, tiles, 1)
         if out.dim() == 3:
             k = x.shape[1]
             edges = [round(i * k / out.shape[0]) for i in range(out.shape[0] + 1)]
@@ -136,8 +160,9 @@ class EmulatedKernels:
             return
         out.copy_((x.to(self.acc) @ weight.to(self.acc).T).to(out.dtype))
 
-    def gated_linear(self, x, weight, out, activation, scratch):
+    def gated_linear(self, x, weight, out, activation, scratch, tiles=None):
         self._count("gated_linear")
+        self._same_numbers(weight, tiles, 2)
         gu = (x.to(self.acc) @ weight.to(self.acc).T)
         self.gated_activation(gu, out, activation)
 

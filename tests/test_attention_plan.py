@@ -21,6 +21,10 @@ def covered(q_len, ctx_len, group, nkv, window, page_size):
         seg, kvh, row0, _, kb, ke, slot, _ = (int(v) for v in it)
         rows = q_len[seg] * group
         assert rows <= 16 and row0 == 0
+        # the kernel gives each of its four wavefronts one block of 32 keys of an aligned group of 128
+        assert kb < ke and kb // 128 == (ke - 1) // 128, (kb, ke)
+        first_pos = ctx_len[seg] - q_len[seg]
+        assert kb >= (max(0, first_pos - window + 1) if window > 0 else 0) and ke <= ctx_len[seg]
         if slot >= 0:
             hold(slot, ("short", n))
         for r in range(rows):

@@ -179,6 +179,46 @@ def test_captured_graphs_give_what_eager_steps_give(model_folders, dtype):
         assert torch.allclose(torch.tensor(a.logprobs), torch.tensor(b.logprobs), atol=1e-5 if dtype == "float32" else 2e-2)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("graphs", [False, True])
+def test_looking_ahead_gives_the_same_tokens_on_the_gpu(model_folders, dtype, graphs):
+    """Steps started before the step before them was read (token ids taken from the device, in
+    eager steps and in replayed graphs) against the same requests run step by step: mixed greedy
+    and seeded sampling, prompt portions beside decoded tokens, requests that stop on a token."""
+    folder = model_folders["M"]
+    model = load_model(folder, dtype, "cuda")
+    prompts = [random_ids(90 + i, n, 1000) for i, n in enumerate([9, 33, 17, 70, 5, 41, 12])]
+    news = [30, 12, 25, 8, 40, 18, 22]
+    params = [SamplingParams(temperature=0.7, top_p=0.9, seed=40 + i) if i % 2 else SamplingParams() for i in range(7)]
+
+    def run(lookahead, stops):
+        runner = ModelRunner.create(model, num_pages=40, page_size=16, max_requests=4)
+        if graphs:
+            runner.enable_graphs(buckets=(1, 2, 4))
+        s = Scheduler(runner, max_prefill_tokens_per_step=16, lookahead=lookahead)
+        reqs = [Request(i, p, n, sampling_params=sp, **stops.get(i, {}))
+                for i, (p, n, sp) in enumerate(zip(prompts, news, params))]
+        for r in reqs:
+            s.add_request(r)
+        s.run_to_completion()
+        runner.cache.check()
+        assert not runner.cache.requests
+        return reqs, runner
+
+    free, _ = run(False, {})
+    # stop three of them in the middle of what they generate
+    stops = {0: dict(eos_token_id=free[0].output_token_ids[11]), 3: dict(stop_token_ids=frozenset([free[3].output_token_ids[2]])),
+             4: dict(eos_token_id=free[4].output_token_ids[20])}
+    stepwise, _ = run(False, stops)
+    ahead, runner = run(True, stops)
+    if graphs:
+        assert runner.graph_steps > 20
+    assert sum(r.finish_reason == "stop" for r in ahead) == 3
+    for a, b in zip(stepwise, ahead):
+        assert a.output_token_ids == b.output_token_ids and a.finish_reason == b.finish_reason
+        assert torch.allclose(torch.tensor(a.logprobs), torch.tensor(b.logprobs), atol=1e-5 if dtype == "float32" else 2e-2)
+
+
 def test_command_line_generates_what_the_entry_point_generates(model_folders, tmp_path):
     folder = model_folders["A"]
     cfg, w = plain_model(folder)

@@ -298,54 +298,73 @@ def test_paged_attention_finds_one_far_key(dtype):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("m,n,k", [(1, 100, 64), (7, 777, 250), (65, 130, 96), (128, 64, 2048), (3, 2560, 2048),
                                    (8, 2048, 16384), (17, 777, 96), (33, 1000, 128), (64, 4099, 2048), (49, 32768, 256),
-                                   (200, 777, 64), (2, 16, 32), (16, 20, 1056)])
+                                   (200, 777, 64), (2, 16, 32), (16, 20, 1056), (16, 2048, 8192), (12, 100, 4128),
+                                   (9, 3072, 24576), (11, 16500, 320)])
 def test_linear(dtype, m, n, k):
     torch.manual_seed(4)
     for out_dtype in {dtype, torch.float32}:
-        def make():
-            x = torch.randn(m, k, device=DEV).to(dtype)
-            w = (torch.randn(n, k, device=DEV) / math.sqrt(k)).to(dtype)
-            return [x, w, torch.zeros(m, n, device=DEV, dtype=out_dtype)], {}
-        torch.manual_seed(4)
-        g, r = both("linear", make, dtype)
-        close(g[2], r[2], out_dtype, f"product to {out_dtype}")
+        for tiled in (False, True):         # from the weight row by row, and from its tile-major copy
+            def make():
+                x = torch.randn(m, k, device=DEV).to(dtype)
+                w = (torch.randn(n, k, device=DEV) / math.sqrt(k)).to(dtype)
+                return [x, w, torch.zeros(m, n, device=DEV, dtype=out_dtype)], {"tiles": ops.tile_weight(w) if tiled else None}
+            torch.manual_seed(4)
+            g, r = both("linear", make, dtype)
+            close(g[2], r[2], out_dtype, f"product to {out_dtype}, tiled {tiled}")
 
 
-@pytest.mark.parametrize("m,n,k", [(8, 2048, 16384), (5, 2560, 2048), (64, 1000, 1024), (1, 777, 512)])
+def test_tile_weight_is_the_documented_permutation():
+    torch.manual_seed(12)
+    for n, k, halves in ((40, 96, 1), (16, 32, 1), (2 * 23, 64, 2), (777, 2048, 1)):
+        w = torch.randn(n, k, device=DEV).to(torch.bfloat16)
+        got = ops.tile_weight(w, halves)
+        with ops.use_backend(EmulatedKernels(precise=True)):
+            ref = ops.tile_weight(w, halves)
+        assert torch.equal(got, ref)
+    assert ops.tile_weight(torch.randn(8, 40, device=DEV).to(torch.bfloat16)) is None      # 40 keys: no tiles
+    assert ops.tile_weight(torch.randn(8, 64, device=DEV)) is None                         # float32: no tiles
+
+
+@pytest.mark.parametrize("m,n,k", [(8, 2048, 16384), (5, 2560, 2048), (64, 1000, 1024), (1, 777, 512), (16, 1000, 8192),
+                                   (3, 3072, 24576), (40, 2048, 16384)])
 def test_linear_leaves_partial_sums_to_the_caller(m, n, k):
     torch.manual_seed(8)
     x = torch.randn(m, k, device=DEV).to(torch.bfloat16)
     w = (torch.randn(n, k, device=DEV) / math.sqrt(k)).to(torch.bfloat16)
     s = ops.linear_splits(m, n, k, torch.bfloat16)
-    whole = torch.zeros(m, n, device=DEV)
-    ops.linear(x, w, whole)
-    if s == 1:
-        with pytest.raises(ops.KernelShapeError):
-            ops.linear(x, w, torch.zeros(2, m, n, device=DEV))
-        return
-    stack = torch.full((s, m, n), 7.0, device=DEV)
-    ops.linear(x, w, stack)
-    total = stack[0].clone()
-    for p in range(1, s):
-        total += stack[p]
-    assert torch.equal(total, whole), "the partial sums add up, in order, to what the kernel gives unsplit"
-    close(whole, x.double() @ w.double().T, torch.float32, "product")
+    for tiles in (None, ops.tile_weight(w)):
+        whole = torch.zeros(m, n, device=DEV)
+        ops.linear(x, w, whole, tiles)
+        if s == 1:
+            with pytest.raises(ops.KernelShapeError):
+                ops.linear(x, w, torch.zeros(2, m, n, device=DEV), tiles)
+            continue
+        stack = torch.full((s, m, n), 7.0, device=DEV)
+        ops.linear(x, w, stack, tiles)
+        total = stack[0].clone()
+        for p in range(1, s):
+            total += stack[p]
+        assert torch.equal(total, whole), "the partial sums add up, in order, to what the kernel gives unsplit"
+        close(whole, x.double() @ w.double().T, torch.float32, "product")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("act", ["gelu_tanh", "silu"])
-@pytest.mark.parametrize("m,inter,k", [(8, 16384, 2048), (3, 250, 96), (64, 777, 128), (100, 384, 96), (17, 112, 80)])
+@pytest.mark.parametrize("m,inter,k", [(8, 16384, 2048), (3, 250, 96), (64, 777, 128), (100, 384, 96), (17, 112, 80),
+                                       (16, 1000, 4128), (1, 250, 96), (13, 2000, 3072), (16, 20, 32)])
 def test_gated_linear(dtype, act, m, inter, k):
     torch.manual_seed(9)
 
-    def make():
-        x = torch.randn(m, k, device=DEV).to(dtype)
-        w = (torch.randn(2 * inter, k, device=DEV) / math.sqrt(k)).to(dtype)
-        return [x, w, torch.zeros(m, inter, device=DEV, dtype=dtype), act, torch.zeros(m, 2 * inter, device=DEV, dtype=dtype)], {}
+    for tiled in (False, True):
+        def make():
+            x = torch.randn(m, k, device=DEV).to(dtype)
+            w = (torch.randn(2 * inter, k, device=DEV) / math.sqrt(k)).to(dtype)
+            return ([x, w, torch.zeros(m, inter, device=DEV, dtype=dtype), act, torch.zeros(m, 2 * inter, device=DEV, dtype=dtype)],
+                    {"tiles": ops.tile_weight(w, 2) if tiled else None})
 
-    torch.manual_seed(9)
-    g, r = both("gated_linear", make, dtype)
-    close(g[2], r[2], dtype)
+        torch.manual_seed(9)
+        g, r = both("gated_linear", make, dtype)
+        close(g[2], r[2], dtype, f"tiled {tiled}")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -386,3 +405,12 @@ def test_shape_errors_are_raised_on_the_host():
         ops.linear(x, torch.zeros(10, 32, device=DEV), torch.zeros(4, 10, device=DEV))
     with pytest.raises(ops.KernelShapeError):
         ops.linear(x.to(torch.bfloat16), torch.zeros(10, 64, device=DEV), torch.zeros(4, 10, device=DEV))
+
+
+def test_feed_tokens_writes_only_the_named_places():
+    ids = torch.arange(10, dtype=torch.int32, device=DEV)
+    dst = torch.tensor([3, -1, 7, 99, 5], dtype=torch.int32, device=DEV)
+    src = torch.tensor([0, 1, 2, 0, 44], dtype=torch.int32, device=DEV)       # 99 and 44 are out of range: skipped
+    source = torch.tensor([100, 200, 300], dtype=torch.int32, device=DEV)
+    ops.feed_tokens(ids, dst, src, source)
+    assert ids.tolist() == [0, 1, 2, 100, 4, 5, 6, 300, 8, 9]

@@ -262,3 +262,100 @@ def test_every_admitted_request_finishes_and_no_page_is_lost(tiny):
             assert steps < 2000
         assert all(r.is_finished() and len(r.output_token_ids) == r.max_new_tokens for r in reqs)
         assert s.cache.num_free_pages(0) == 24 and not s.cache.requests
+
+
+def _workload(seed, count=9):
+    """Requests of mixed lengths; a third stop on a token that greedy decoding will produce."""
+    g = torch.Generator().manual_seed(seed)
+    reqs = []
+    for i in range(count):
+        n = int(torch.randint(1, 40, (1,), generator=g))
+        mx = int(torch.randint(1, 16, (1,), generator=g))
+        kind = i % 3
+        sp = SamplingParams(temperature=0.9, top_k=20, seed=7 + i) if kind == 1 else SamplingParams()
+        reqs.append(dict(request_id=i, prompt_token_ids=random_ids(seed * 100 + i, n, 512), max_new_tokens=mx,
+                         sampling_params=sp))
+    return reqs
+
+
+@pytest.mark.parametrize("admission,pages", [("pledged", 40), ("prompt_only", 16)])
+def test_looking_ahead_gives_every_request_the_same_tokens(tiny, admission, pages):
+    """A step started before the step before it was read: the tokens come from the device, stops on
+    an end token are seen one step late and the extra token is dropped."""
+    model, _, _ = tiny
+    specs = _workload(3)
+    results = {}
+    for lookahead in (False, True):
+        # first without stop tokens, to learn what is generated; then stop in the middle of that
+        plain_run = make(model, num_pages=pages, page_size=4, max_requests=4, max_prefill_tokens_per_step=10,
+                         admission=admission, lookahead=lookahead)
+        first = [Request(**spec) for spec in specs]
+        for r in first:
+            plain_run.add_request(r)
+        plain_run.run_to_completion()
+        s = make(model, num_pages=pages, page_size=4, max_requests=4, max_prefill_tokens_per_step=10,
+                 admission=admission, lookahead=lookahead)
+        reqs = []
+        for spec, done in zip(specs, first):
+            out = done.output_token_ids
+            extra = {}
+            if spec["request_id"] % 3 == 0 and len(out) >= 3:
+                extra = dict(eos_token_id=out[len(out) // 2])
+            elif spec["request_id"] % 3 == 2 and len(out) >= 2:
+                extra = dict(stop_token_ids=frozenset([out[-2]]))
+            reqs.append(Request(**spec, **extra))
+            s.add_request(reqs[-1])
+        steps = 0
+        while s.has_unfinished_requests():
+            s.step()
+            s.cache.check()
+            steps += 1
+            assert steps < 3000
+        assert all(r.is_finished() for r in reqs)
+        assert s.cache.num_free_pages(0) == pages and not s.cache.requests, "every page came back"
+        for r in reqs:
+            assert len(r.output_token_ids) == len(r.logprobs) <= r.max_new_tokens
+            if r.finish_reason == "stop":
+                assert r.ends_with(r.output_token_ids[-1]) and not any(r.ends_with(t) for t in r.output_token_ids[:-1])
+        results[lookahead] = ([r.output_token_ids for r in reqs], [r.finish_reason for r in reqs],
+                              [r.output_token_ids for r in first], s.stats["preemptions"])
+    assert results[True][:3] == results[False][:3]
+    assert any(reason == "stop" for reason in results[True][1]), "the workload has requests that stop early"
+    if admission == "prompt_only":
+        assert results[True][3] > 0, "the small pool forces preemptions"
+
+
+def test_looking_ahead_starts_the_next_step_before_the_tokens_are_read(tiny):
+    model, cfg, w = tiny
+    prompt = prompts_of([9])[0]
+    s = make(model, lookahead=True)
+    fed = []
+    real_step = s.runner.step
+    def spy(entries, feed_tokens=None):
+        fed.append([e.feed_row for e in entries])
+        return real_step(entries, feed_tokens)
+    s.runner.step = spy
+    r = Request("r", prompt, 5)
+    s.add_request(r)
+    got = s.step()
+    # the prompt's step and the first decode step have both been started; only the first was read
+    assert len(fed) == 2 and fed[1] == [0] and got == [r]
+    assert len(r.output_token_ids) == 2 and r.logprobs[1] is None, "the second token is a placeholder still"
+    s.run_to_completion()
+    assert r.output_token_ids == gemma_plain.generate_greedy(cfg, w, prompt, 5)
+    assert [rows for rows in fed[1:]] == [[0]] * 4, "four decode steps, each fed from the device"
+
+
+def test_a_repetition_penalty_is_never_run_ahead(tiny):
+    model, _, _ = tiny
+    prompt = prompts_of([12])[0]
+    outs = []
+    for lookahead in (False, True):
+        s = make(model, lookahead=lookahead)
+        r = Request("p", prompt, 8, sampling_params=SamplingParams(repetition_penalty=1.3))
+        s.add_request(r)
+        while s.has_unfinished_requests():
+            s.step()
+            assert s._started is None, "a penalised request waits for its tokens"
+        outs.append(r.output_token_ids)
+    assert outs[0] == outs[1]

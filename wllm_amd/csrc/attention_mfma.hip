@@ -10,11 +10,14 @@
 // src/wllm/kernels/csrc/paged_attention.cu:44-45,185).
 //
 // Work items.  The host cuts every (segment, key/value head) into work items, one workgroup of 4
-// wavefronts each: the segment's one tile of 16 rows and a chunk of keys.  The four wavefronts
-// split the chunk's blocks of 32 keys and are merged through shared memory.  A segment with more
-// keys than a chunk is split over workgroups; those write partial results (running maximum, sum,
-// unnormalised accumulator) that `attention_reduce_kernel` combines.  Chunk boundaries depend
-// on the key index only, never on the batch.
+// wavefronts each: the segment's one tile of 16 rows and a chunk of keys that lies within one
+// aligned group of 128 keys, cut to what the rows can need.  Each wavefront takes one of the
+// chunk's four blocks of 32 keys; its loads of keys and values wait for the item and the block
+// table only (the request's lengths and the queries are read while they are in flight), and the
+// four are merged through shared memory.  A segment with more keys than a chunk is split over
+// workgroups; those write partial results (maximum, sum, unnormalised accumulator) that
+// `attention_reduce_kernel` combines.  Chunk boundaries depend on the key index only, never on
+// the batch.
 //
 // Matrix products (v_mfma_f32_16x16x32_bf16, 64 lanes: i = lane % 16, g = lane / 16):
 //   scores^T[key, row] = K[key, :] . Q[row, :]     A = K: lane (i, g) holds K[key_i][32c + 8g ..+8]
@@ -45,7 +48,7 @@ union Pack16 {
 __device__ __forceinline__ uint16_t bf16_bits(float f) { return from_float<bf16>(f).bits; }
 
 template <int HD, bool V16>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, 2)
 paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict__ cache,
                             const int* __restrict__ block_tables, const int* __restrict__ items,
                             const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
@@ -67,29 +70,85 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
     const int key_splits = 4 / row_tiles;           // wavefronts that share a row tile
     const int rt = wave % row_tiles, ks = wave / row_tiles;
 
+    // ---- The walk over the keys depends on the item alone: the host cut the item's keys to what
+    //      its rows can need (from the lowest window start of the first row to the last row's
+    //      position).  The loads of the first block of keys and values are issued before anything
+    //      else is read, so they wait for the item and the block table only; the request's
+    //      lengths and the queries arrive while they are in flight. ----
     const int group = num_heads / num_kv_heads;
+    const int width = (num_heads + 2 * num_kv_heads) * HD;
+    const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * HD;
+    const size_t k_off = static_cast<size_t>(kvh) * page_size * HD;
+    const size_t v_off = (static_cast<size_t>(num_kv_heads) + kvh) * page_size * HD;
+    const int* table = block_tables + static_cast<size_t>(seg) * max_pages;
+    const int blk_first = key_begin / kKeysPerBlock;
+    const int blk_end = (key_end + kKeysPerBlock - 1) / kKeysPerBlock;
+    Pack16 ka_[2][DC], va_[DT];
+    // All loads of a block are issued before the first product needs one, so a block costs one
+    // trip to memory.  Keys beyond the request are masked later; their table entry is clamped to
+    // the table's width (entries beyond a request's pages name a valid page), not to the length.
+    auto issue = [&](int blk) {
+        const int kbase = blk * kKeysPerBlock;
+        const bf16* krow[2];
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2) {
+            // which key the A row i of the score product is; see the header for why
+            const int kk = kbase + (V16 ? 8 * (i / 4) + 4 * t2 + (i % 4) : 16 * t2 + i);
+            const int page = table[min(kk / page_size, max_pages - 1)];
+            krow[t2] = cache + static_cast<size_t>(page) * page_elems + k_off +
+                       static_cast<size_t>(kk % page_size) * HD + 8 * g;
+        }
+        int vpage0, vslot0, vpage1 = 0, vslot1 = 0;
+        if (V16) {
+            const int kk = kbase + 8 * g;
+            vpage0 = table[min(kk / page_size, max_pages - 1)];
+            vslot0 = kk % page_size;
+        } else {
+            const int ka = kbase + 4 * g, kb = kbase + 16 + 4 * g;
+            vpage0 = table[min(ka / page_size, max_pages - 1)];
+            vslot0 = ka % page_size;
+            vpage1 = table[min(kb / page_size, max_pages - 1)];
+            vslot1 = kb % page_size;
+        }
+        const bf16* vbase0 = cache + static_cast<size_t>(vpage0) * page_elems + v_off + vslot0;
+        const bf16* vbase1 = cache + static_cast<size_t>(vpage1) * page_elems + v_off + vslot1;
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+            for (int c = 0; c < DC; ++c) ka_[t2][c].u = *reinterpret_cast<const uint4*>(krow[t2] + c * 32);
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+            const size_t drow = static_cast<size_t>(t * 16 + i) * page_size;
+            if (V16) {
+                va_[t].u = *reinterpret_cast<const uint4*>(vbase0 + drow);
+            } else {
+                va_[t].half[0] = *reinterpret_cast<const uint2*>(vbase0 + drow);
+                va_[t].half[1] = *reinterpret_cast<const uint2*>(vbase1 + drow);
+            }
+        }
+    };
+    // An item's keys lie within one aligned group of 128 (the host's chunk), so each of the four
+    // wavefronts has at most one block of 32 keys and nothing is carried from block to block.
+    const int blk = blk_first + ks;
+    const bool has_block = blk < blk_end && blk < blk_first + key_splits;
+    if (has_block) issue(blk);
+
     const int q_start = seg_q_start[seg], q_len = seg_q_len[seg], ctx = seg_ctx_len[seg];
     const int total_rows = q_len * group;
     const int first_pos = ctx - q_len;
     const int seg_lo = window > 0 ? max(0, first_pos - window + 1) : 0;   // keys below may be given back
-    const int r0 = row_begin + rt * kRowsPerTile;
-    const bool tile_active = r0 < total_rows;
-    const int row = r0 + i;
+    const int row = row_begin + i;
     const bool row_valid = row < total_rows;
     const int tok = row_valid ? row / group : 0;
     const int head = kvh * group + (row_valid ? row % group : 0);
     const int pos = first_pos + tok;
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
 
-    const int width = (num_heads + 2 * num_kv_heads) * HD;
-    const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * HD;
-    const size_t k_off = static_cast<size_t>(kvh) * page_size * HD;
-    const size_t v_off = (static_cast<size_t>(num_kv_heads) + kvh) * page_size * HD;
-    const int* table = block_tables + static_cast<size_t>(seg) * max_pages;
-
-    // the queries of this lane's row
-    bf16x8_t qreg[DC];
-    {
+    float4_t acc[DT];
+    float m_run = -INFINITY, l_run = 0.f;
+    if (has_block) {
+        // the queries of this lane's row
+        bf16x8_t qreg[DC];
         const bf16* qrow = qkv + static_cast<size_t>(q_start + tok) * width + static_cast<size_t>(head) * HD;
 #pragma unroll
         for (int c = 0; c < DC; ++c) {
@@ -97,124 +156,64 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
             p.u = row_valid ? *reinterpret_cast<const uint4*>(qrow + c * 32 + 8 * g) : make_uint4(0, 0, 0, 0);
             qreg[c] = p.v;
         }
-    }
-
-    float4_t acc[DT];
+        const int kbase = blk * kKeysPerBlock;
+        const bool edge = kbase < seg_lo || kbase + kKeysPerBlock > ctx;
+        // ---- scores of two tiles of 16 keys ----
+        float4_t s[2];
 #pragma unroll
-    for (int t = 0; t < DT; ++t) acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
-    float m_run = -INFINITY, l_run = 0.f;
-
-    if (tile_active) {
-        // keys this tile can need: from the lowest window start to the highest position of its rows
-        const int last_row = min(total_rows - 1, r0 + kRowsPerTile - 1);
-        const int tile_hi = min(key_end, first_pos + last_row / group + 1);
-        const int tile_lo = max(key_begin, window > 0 ? max(0, first_pos + r0 / group - window + 1) : 0);
-        const int blk_first = tile_lo / kKeysPerBlock;
-        const int blk_end = (tile_hi + kKeysPerBlock - 1) / kKeysPerBlock;
-        for (int blk = blk_first + ks; blk < blk_end; blk += key_splits) {
-            const int kbase = blk * kKeysPerBlock;
-            const bool edge = kbase < seg_lo || kbase + kKeysPerBlock > ctx;
-            // ---- addresses of the keys and values of this block; all loads are issued before
-            //      the first product needs one, so the block costs one trip to memory ----
-            const bf16* krow[2];
+        for (int t2 = 0; t2 < 2; ++t2) {
+            float4_t sc = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2) {
-                // which key the A row i of the score product is; see the header for why
-                int kk = kbase + (V16 ? 8 * (i / 4) + 4 * t2 + (i % 4) : 16 * t2 + i);
-                kk = min(kk, ctx - 1);
-                const int page = table[kk / page_size];
-                krow[t2] = cache + static_cast<size_t>(page) * page_elems + k_off +
-                           static_cast<size_t>(kk % page_size) * HD + 8 * g;
-            }
-            int vpage0, vslot0, vpage1 = 0, vslot1 = 0;
-            if (V16) {
-                const int kk = min(kbase + 8 * g, ctx - 1) & ~7;
-                vpage0 = table[kk / page_size];
-                vslot0 = kk % page_size;
-            } else {
-                const int ka = min(kbase + 4 * g, ctx - 1) & ~3, kb = min(kbase + 16 + 4 * g, ctx - 1) & ~3;
-                vpage0 = table[ka / page_size];
-                vslot0 = ka % page_size;
-                vpage1 = table[kb / page_size];
-                vslot1 = kb % page_size;
-            }
-            const bf16* vbase0 = cache + static_cast<size_t>(vpage0) * page_elems + v_off + vslot0;
-            const bf16* vbase1 = cache + static_cast<size_t>(vpage1) * page_elems + v_off + vslot1;
-            Pack16 ka_[2][DC], va_[DT];
-#pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2)
-#pragma unroll
-                for (int c = 0; c < DC; ++c) ka_[t2][c].u = *reinterpret_cast<const uint4*>(krow[t2] + c * 32);
-#pragma unroll
-            for (int t = 0; t < DT; ++t) {
-                const size_t drow = static_cast<size_t>(t * 16 + i) * page_size;
-                if (V16) {
-                    va_[t].u = *reinterpret_cast<const uint4*>(vbase0 + drow);
-                } else {
-                    va_[t].half[0] = *reinterpret_cast<const uint2*>(vbase0 + drow);
-                    va_[t].half[1] = *reinterpret_cast<const uint2*>(vbase1 + drow);
-                }
-            }
-            // ---- scores of two tiles of 16 keys ----
-            float4_t s[2];
-#pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2) {
-                float4_t sc = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int c = 0; c < DC; ++c)
-                    sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka_[t2][c].v, qreg[c], sc, 0, 0, 0);
-                s[t2] = sc;
-            }
-            // ---- mask, running maximum, probabilities ----
-            float sv[8];
-            bool ok[8];
-            float tile_max = -INFINITY;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int t2 = e / 4, v = e % 4;
-                const int key = kbase + (V16 ? 8 * g + 4 * t2 + v : 16 * t2 + 4 * g + v);
-                ok[e] = row_valid && key <= pos && key >= lo && key >= key_begin && key < key_end;
-                sv[e] = s[t2][v];
-                if (ok[e]) tile_max = fmaxf(tile_max, sv[e]);
-            }
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
-            const float m_new = fmaxf(m_run, tile_max);
-            const float m_use = m_new == -INFINITY ? 0.f : m_new;
-            const float alpha = exp2f((m_run - m_use) * scale_log2e);    // 0 while nothing was seen
-            Pack16 pv;
-            float psum = 0.f;
-            const float mc = m_use * scale_log2e;
-            float pe[8];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                pe[e] = ok[e] ? exp2f(fmaf(sv[e], scale_log2e, -mc)) : 0.f;
-                psum += pe[e];
-            }
-            pv.u = make_uint4(pack2_bf16(pe[0], pe[1]), pack2_bf16(pe[2], pe[3]), pack2_bf16(pe[4], pe[5]),
-                              pack2_bf16(pe[6], pe[7]));
-            l_run = l_run * alpha + psum;      // per lane; the four lanes of a row are added at the end
-            m_run = m_new;
-            // ---- out^T += V^T . P^T ----
-#pragma unroll
-            for (int t = 0; t < DT; ++t) {
-                Pack16 a = va_[t];
-                if (edge) {
-                    // keys outside the request (stale slots, pages given back) may hold anything,
-                    // NaN included; 0 * NaN would poison the sum, so they are cleared
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const int key = kbase + (V16 ? 8 * g + e : (e < 4 ? 4 * g + e : 16 + 4 * g + e - 4));
-                        if (key >= ctx || key < seg_lo) a.s[e] = 0;
-                    }
-                }
-                acc[t] *= alpha;
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pv.v, acc[t], 0, 0, 0);
-            }
+            for (int c = 0; c < DC; ++c)
+                sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka_[t2][c].v, qreg[c], sc, 0, 0, 0);
+            s[t2] = sc;
         }
+        // ---- mask, maximum, probabilities ----
+        float sv[8];
+        bool ok[8];
+        float tile_max = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int t2 = e / 4, v = e % 4;
+            const int key = kbase + (V16 ? 8 * g + 4 * t2 + v : 16 * t2 + 4 * g + v);
+            ok[e] = row_valid && key <= pos && key >= lo && key >= key_begin && key < key_end;
+            sv[e] = s[t2][v];
+            if (ok[e]) tile_max = fmaxf(tile_max, sv[e]);
+        }
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
+        m_run = tile_max;
+        const float mc = (tile_max == -INFINITY ? 0.f : tile_max) * scale_log2e;
+        Pack16 pv;
+        float pe[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            pe[e] = ok[e] ? exp2f(fmaf(sv[e], scale_log2e, -mc)) : 0.f;
+            l_run += pe[e];
+        }
+        pv.u = make_uint4(pack2_bf16(pe[0], pe[1]), pack2_bf16(pe[2], pe[3]), pack2_bf16(pe[4], pe[5]),
+                          pack2_bf16(pe[6], pe[7]));
         // the row's sum over its four lanes
         l_run += __shfl_xor(l_run, 16, kWave);
         l_run += __shfl_xor(l_run, 32, kWave);
+        // ---- out^T = V^T . P^T ----
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+            Pack16 a = va_[t];
+            if (edge) {
+                // keys outside the request (stale slots, pages given back) may hold anything,
+                // NaN included; 0 * NaN would poison the sum, so they are cleared
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int key = kbase + (V16 ? 8 * g + e : (e < 4 ? 4 * g + e : 16 + 4 * g + e - 4));
+                    if (key >= ctx || key < seg_lo) a.s[e] = 0;
+                }
+            }
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pv.v, float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < DT; ++t) acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
     }
 
     // ---- merge the wavefronts that split the keys of one row tile ----

@@ -29,6 +29,24 @@ WLLM_API int wllm_embed_lookup(const int* ids, const void* table, int is_bf16, f
                    : embed_lookup_launch<float>(ids, table, scale, out, n, hidden, vocab, stream);
 }
 
+// ---- token ids that come from the device: ids[dst[j]] = source[src[j]] for every j with dst[j] >= 0.
+// A step that is started before the step before it has been read takes the tokens that step sampled
+// straight from its output, without a trip through the host.
+__global__ void feed_tokens_kernel(int* __restrict__ ids, const int* __restrict__ dst, const int* __restrict__ src,
+                                   const int* __restrict__ source, int count, int num_ids, int num_source) {
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= count) return;
+    const int d = dst[j], s = src[j];
+    if (d >= 0 && d < num_ids && s >= 0 && s < num_source) ids[d] = source[s];
+}
+
+WLLM_API int wllm_feed_tokens(int* ids, const int* dst, const int* src, const int* source, int count, int num_ids,
+                              int num_source, hipStream_t stream) {
+    if (count <= 0) return 0;
+    feed_tokens_kernel<<<(count + 255) / 256, 256, 0, stream>>>(ids, dst, src, source, count, num_ids, num_source);
+    return launch_status();
+}
+
 // ---- RMS norm: out = v * rsqrt(mean(v^2) + eps) * (offset + w), v = x (+ delta) ------------
 // One workgroup per output row.  Without `rows` the sum x + delta is written back to x.  `delta`
 // may be a stack of `splits` partial sums (a product split over K), `split_stride` elements apart;

@@ -21,6 +21,36 @@ union Frag {
     bf16x8_t v;
 };
 
+// ---- the tile-major copy of a weight that the few-row kernels stream --------------------------
+// dst holds, for each band of 16 rows (the last one padded with zero rows) and each step of 32
+// keys, the tile's 1 KiB: lane l = 16g + i holds w[16 * band + i][32 * step + 8g .. +8].  A
+// wavefront's load of a tile is then one contiguous KiB and its walk along K one contiguous run,
+// which the memory system serves faster than 16 pieces of 64 bytes a row apart.
+__global__ void tile_weight_kernel(const bf16* __restrict__ src, bf16* __restrict__ dst, int N, int K, long long pieces) {
+    const long long p = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (p >= pieces) return;
+    const int lane = static_cast<int>(p % 64);
+    const long long tile = p / 64;
+    const int steps = K / 32;
+    const int step = static_cast<int>(tile % steps);
+    const long long band = tile / steps;
+    const long long row = band * 16 + lane % 16;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (row < N) v = *reinterpret_cast<const uint4*>(src + row * K + step * 32 + 8 * (lane / 16));
+    *reinterpret_cast<uint4*>(dst + p * 8) = v;
+}
+
+// dst must hold ceil(N / 16) * 16 * K elements.  Returns 0, a HIP error code, or -1 for sizes it does not take.
+WLLM_API int wllm_tile_weight(const void* src, void* dst, int N, int K, hipStream_t stream) {
+    if (N < 1 || K < 32 || K % 32 != 0) return -1;
+    const long long pieces = static_cast<long long>((N + 15) / 16) * (K / 32) * 64;
+    const long long blocks = (pieces + 255) / 256;
+    if (blocks > 0x7fffffffLL) return -1;
+    tile_weight_kernel<<<static_cast<unsigned>(blocks), 256, 0, stream>>>(static_cast<const bf16*>(src), static_cast<bf16*>(dst), N, K,
+                                                                        pieces);
+    return launch_status();
+}
+
 template <typename TO> __device__ __forceinline__ void store4(TO* p, float4_t v);
 template <> __device__ __forceinline__ void store4<float>(float* p, float4_t v) { *reinterpret_cast<float4_t*>(p) = v; }
 template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float4_t v) {
@@ -32,7 +62,10 @@ template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float4_t v) {
 
 // NT: tiles of 16 weight rows per wavefront.  With many rows of x (MT > 1) every fragment of x read
 // from shared memory then feeds NT products, and a workgroup stages x once for 64*NT weight rows.
-template <int MT, int NT, typename TO>
+// TILED: w is stored tile by tile (see `wllm_tile_weight`): a tile of 16 rows and 32 keys as the 16
+// bytes of each of the 64 lanes in lane order, the tiles of a band of 16 rows one after the other along
+// K, so a wavefront streams one contiguous run.
+template <int MT, int NT, typename TO, bool TILED>
 __global__ void __launch_bounds__(256)
 gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* __restrict__ out,
                    float* __restrict__ partial, int M, int N, int K, int k_per_split, int chunk) {
@@ -42,10 +75,17 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* _
     const int n0 = (blockIdx.x * 4 + wave) * 16 * NT;
     const int k_begin = blockIdx.y * k_per_split, k_end = min(K, k_begin + k_per_split);
     const int stride = chunk / 8 + 1;             // in uint4; the odd stride spreads rows over the banks
+    constexpr int kStep = TILED ? 512 : 32;       // elements from one step of 32 keys to the next
     const bf16* wp[NT];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-        wp[nt] = w + static_cast<size_t>(min(n0 + nt * 16 + i, N - 1)) * K + k_begin + 8 * g;
+    for (int nt = 0; nt < NT; ++nt) {
+        if (TILED) {
+            const int band = min(n0 / 16 + nt, (N + 15) / 16 - 1);
+            wp[nt] = w + (static_cast<size_t>(band) * (K / 32) + k_begin / 32) * 512 + lane * 8;
+        } else {
+            wp[nt] = w + static_cast<size_t>(min(n0 + nt * 16 + i, N - 1)) * K + k_begin + 8 * g;
+        }
+    }
     float4_t acc[NT][MT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
@@ -63,7 +103,7 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* _
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
             for (int u = 0; u < kBatch; ++u)
-                dst[nt][u].u = (live && step0 + u < steps) ? *reinterpret_cast<const uint4*>(wp[nt] + (step0 + u) * 32)
+                dst[nt][u].u = (live && step0 + u < steps) ? *reinterpret_cast<const uint4*>(wp[nt] + (step0 + u) * kStep)
                                                            : make_uint4(0, 0, 0, 0);
     };
     fetch(cur, 0);
@@ -162,8 +202,8 @@ __global__ void split_sum_kernel(const float* __restrict__ partial, TO* __restri
 // Returns 0, a HIP error code, or -1 for sizes this kernel does not take.
 // `partial` must hold splits * M * N floats when splits > 1; with `out` null the partial sums
 // are the result and nothing adds them.
-WLLM_API int wllm_gemm_skinny(const void* x, const void* w, void* out, int out_bf16, float* partial, int M, int N,
-                              int K, int splits, int chunk, hipStream_t stream) {
+WLLM_API int wllm_gemm_skinny(const void* x, const void* w, int tiled, void* out, int out_bf16, float* partial, int M,
+                              int N, int K, int splits, int chunk, hipStream_t stream) {
     if (M < 1 || M > 64 || K % 32 != 0 || splits < 1 || K % splits != 0 || (K / splits) % 32 != 0 || chunk % 32 != 0)
         return -1;
     // every result needs somewhere to go: a split product its partial sums, an unsplit one its output
@@ -181,9 +221,12 @@ WLLM_API int wllm_gemm_skinny(const void* x, const void* w, void* out, int out_b
         else if (tiles / 2 * splits >= 1024) nt = 2;
     }
     const dim3 grid((N + 64 * nt - 1) / (64 * nt), splits);
-#define LAUNCH(MT, NT, TO)                                                                                   \
-    gemm_skinny_kernel<MT, NT, TO><<<grid, 256, smem, stream>>>(static_cast<const bf16*>(x), static_cast<const bf16*>(w), \
-                                                                static_cast<TO*>(out), partial, M, N, K, k_per_split, chunk)
+#define LAUNCH_T(MT, NT, TO, T)                                                                                  \
+    gemm_skinny_kernel<MT, NT, TO, T><<<grid, 256, smem, stream>>>(static_cast<const bf16*>(x), static_cast<const bf16*>(w), \
+                                                                   static_cast<TO*>(out), partial, M, N, K, k_per_split, chunk)
+#define LAUNCH(MT, NT, TO)                  \
+    if (tiled) LAUNCH_T(MT, NT, TO, true);  \
+    else LAUNCH_T(MT, NT, TO, false)
 #define BY_NT(MT, TO)                    \
     if (nt == 4) LAUNCH(MT, 4, TO);      \
     else if (nt == 2) LAUNCH(MT, 2, TO); \
@@ -199,6 +242,7 @@ WLLM_API int wllm_gemm_skinny(const void* x, const void* w, void* out, int out_b
 #undef BY_MT
 #undef BY_NT
 #undef LAUNCH
+#undef LAUNCH_T
     int err = launch_status();
     if (err) return err;
     if (splits > 1 && out != nullptr) {
@@ -224,7 +268,7 @@ __device__ __forceinline__ float act_silu(float z) { return z / (1.f + expf(-z))
 // A workgroup is 8 wavefronts: 4 tiles of 16 gate rows (with their up rows) times 2 halves of the
 // K axis, so that two wavefronts per SIMD keep loads in flight; the halves are added through shared
 // memory in a fixed order before the activation.
-template <int MT, int ACT>
+template <int MT, int ACT, bool TILED>
 __global__ void __launch_bounds__(512)
 gemm_skinny_gated_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, bf16* __restrict__ out, int M,
                          int inter, int K, int chunk) {
@@ -237,9 +281,14 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
     const int half_k = K / 2;                     // a multiple of 32
     const int k_begin = half * half_k;
     uint4* xh = xs + half * (MT * 16 * stride);
+    // TILED: the gate rows' bands of 16 rows first, then the up rows' bands
+    constexpr int kStep = TILED ? 512 : 32;
     const int nrow = min(n0 + i, inter - 1);
-    const bf16* gp = w + static_cast<size_t>(nrow) * K + k_begin + 8 * g;
-    const bf16* up = w + static_cast<size_t>(inter + nrow) * K + k_begin + 8 * g;
+    const int bands = (inter + 15) / 16, band = min(n0 / 16, bands - 1);
+    const bf16* gp = TILED ? w + (static_cast<size_t>(band) * (K / 32) + k_begin / 32) * 512 + lane * 8
+                           : w + static_cast<size_t>(nrow) * K + k_begin + 8 * g;
+    const bf16* up = TILED ? w + (static_cast<size_t>(bands + band) * (K / 32) + k_begin / 32) * 512 + lane * 8
+                           : w + static_cast<size_t>(inter + nrow) * K + k_begin + 8 * g;
     float4_t accg[MT], accu[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
@@ -254,8 +303,8 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
 #pragma unroll
         for (int u = 0; u < kBatch; ++u) {
             const bool ok = live && step0 + u < steps;
-            dg[u].u = ok ? *reinterpret_cast<const uint4*>(gp + (step0 + u) * 32) : make_uint4(0, 0, 0, 0);
-            du[u].u = ok ? *reinterpret_cast<const uint4*>(up + (step0 + u) * 32) : make_uint4(0, 0, 0, 0);
+            dg[u].u = ok ? *reinterpret_cast<const uint4*>(gp + (step0 + u) * kStep) : make_uint4(0, 0, 0, 0);
+            du[u].u = ok ? *reinterpret_cast<const uint4*>(up + (step0 + u) * kStep) : make_uint4(0, 0, 0, 0);
         }
     };
     fetch(curg, curu, 0);
@@ -346,8 +395,8 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
     }
 }
 
-WLLM_API int wllm_gemm_skinny_gated(const void* x, const void* w, void* out, int M, int inter, int K, int activation,
-                                    int chunk, hipStream_t stream) {
+WLLM_API int wllm_gemm_skinny_gated(const void* x, const void* w, int tiled, void* out, int M, int inter, int K,
+                                    int activation, int chunk, hipStream_t stream) {
     if (M < 1 || M > 64 || K % 64 != 0 || chunk % 32 != 0 || activation < 0 || activation > 1) return -1;
     const int mt = (M + 15) / 16;
     if (chunk > K / 2) chunk = K / 2;
@@ -356,9 +405,12 @@ WLLM_API int wllm_gemm_skinny_gated(const void* x, const void* w, void* out, int
     if (red > smem) smem = red;
     if (smem > 65536 || mt * 16 * (chunk / 8) > 1024) return -1;     // 4 pieces of x per thread at most
     const dim3 grid((inter + 63) / 64);
-#define LAUNCH(MT, A)                                                                                              \
-    gemm_skinny_gated_kernel<MT, A><<<grid, 512, smem, stream>>>(static_cast<const bf16*>(x), static_cast<const bf16*>(w), \
-                                                                 static_cast<bf16*>(out), M, inter, K, chunk)
+#define LAUNCH_T(MT, A, T)                                                                                            \
+    gemm_skinny_gated_kernel<MT, A, T><<<grid, 512, smem, stream>>>(static_cast<const bf16*>(x), static_cast<const bf16*>(w), \
+                                                                    static_cast<bf16*>(out), M, inter, K, chunk)
+#define LAUNCH(MT, A)                  \
+    if (tiled) LAUNCH_T(MT, A, true);  \
+    else LAUNCH_T(MT, A, false)
 #define BY_MT(A)                     \
     switch (mt) {                    \
         case 1: LAUNCH(1, A); break; \
@@ -369,5 +421,6 @@ WLLM_API int wllm_gemm_skinny_gated(const void* x, const void* w, void* out, int
     if (activation == 0) { BY_MT(0) } else { BY_MT(1) }
 #undef BY_MT
 #undef LAUNCH
+#undef LAUNCH_T
     return launch_status();
 }

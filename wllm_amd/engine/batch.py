@@ -22,6 +22,10 @@ class StepEntry:
     request: object
     tokens: list
     want: list = field(default_factory=list)
+    # The last of `tokens` is not known on the host yet: it is row `feed_row` of the tensor of
+    # sampled tokens that the step is given (`ModelRunner.step(..., feed_tokens=...)`), read on the
+    # device.  The value in `tokens` is then a placeholder.
+    feed_row: Optional[int] = None
 
 
 @dataclass

@@ -35,7 +35,8 @@ class DecodeGraph:
         self.table_width = -(-max_context // cache.page_size)
         b = bucket
         # layout of the packed buffer: eight arrays of b, then per group slots [b] and tables [b, width]
-        sizes = [b] * 8 + [b] * self.num_groups + [b * self.table_width] * self.num_groups
+        # and two arrays of b that say which token ids come from the device (`feed_row`)
+        sizes = [b] * 8 + [b] * self.num_groups + [b * self.table_width] * self.num_groups + [b] * 2
         self._offsets = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
         total = int(self._offsets[-1])
         self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
@@ -43,6 +44,7 @@ class DecodeGraph:
         self.np = self.host.numpy()
         v = [self.dev[self._offsets[i]:self._offsets[i + 1]] for i in range(len(sizes))]
         g = self.num_groups
+        self._feed_dst, self._feed_src = v[8 + 2 * g], v[9 + 2 * g]
         self.workspace = Workspace(self.device)
         self.ctx = StepContext(
             n=b, num_segments=b, dtype=model.dtype, device=self.device, workspace=self.workspace, cache=cache,
@@ -94,6 +96,12 @@ class DecodeGraph:
                 slots[i] = reserved[i][gi][0]
                 t = cache.block_table(e.request, gi)
                 table[i, :len(t)] = np.maximum(np.asarray(t, dtype=np.int32), 0)
+        feed_dst, feed_src = self._field(8 + 2 * g), self._field(9 + 2 * g)
+        feed_dst[:] = -1
+        feed_src[:] = 0
+        for i, e in enumerate(entries):
+            if e.feed_row is not None:
+                feed_dst[i], feed_src[i] = i, e.feed_row
         self.ctx.host_ctx_len = cl.copy()
         self.ctx.host_state_slots = st.copy()
         self.ctx.requests = [e.request for e in entries] + [None] * (b - n)
@@ -104,8 +112,11 @@ class DecodeGraph:
         self._copied.record()
         self._in_flight = True
 
-    def run(self, entries: list, reserved: list) -> torch.Tensor:
+    def run(self, entries: list, reserved: list, feed_tokens=None) -> torch.Tensor:
         self.fill(entries, reserved)
+        if feed_tokens is not None:
+            # outside the captured graph: the tensor of sampled tokens is not the graph's own
+            ops.feed_tokens(self.ctx.token_ids, self._feed_dst, self._feed_src, feed_tokens)
         if self.graph is None:
             # once eagerly: scratch tensors and plans come into being, lazy library state settles
             self.runner.model.forward(self.ctx)

@@ -67,9 +67,20 @@ class Request:
         """sequence.py:53-59."""
         self.output_token_ids.append(int(token))
         self.logprobs.append(logprob)
-        if self.eos_token_id is not None and token == self.eos_token_id:
-            self.status, self.finish_reason = RequestStatus.FINISHED, "stop"
-        elif token in self.stop_token_ids:
+        if self.ends_with(token):
             self.status, self.finish_reason = RequestStatus.FINISHED, "stop"
         elif len(self.output_token_ids) >= self.max_new_tokens:
             self.status, self.finish_reason = RequestStatus.FINISHED, "length"
+
+    def ends_with(self, token: int) -> bool:
+        """Whether sampling this token ends the request whatever its length."""
+        return (self.eos_token_id is not None and token == self.eos_token_id) or token in self.stop_token_ids
+
+    def append_placeholder(self) -> int:
+        """Room for a token that has been sampled on the device and not been read yet; returns its
+        index among the outputs.  Only the length rule can be applied before the value is known."""
+        self.output_token_ids.append(0)
+        self.logprobs.append(None)
+        if len(self.output_token_ids) >= self.max_new_tokens:
+            self.status, self.finish_reason = RequestStatus.FINISHED, "length"
+        return len(self.output_token_ids) - 1

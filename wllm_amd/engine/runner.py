@@ -10,12 +10,15 @@ tool and the benchmark all call it.
 """
 from __future__ import annotations
 
+from typing import Optional
+
 import numpy as np
 import torch
 
 from wllm_amd.cache.manager import CacheManager
 from wllm_amd.cache.pages import OutOfPages
 from wllm_amd.engine.batch import StepContext, StepEntry, Workspace, pack_int32
+from wllm_amd.kernels import ops
 
 
 class StepError(ValueError):
@@ -74,17 +77,26 @@ class ModelRunner:
     def close(self, request) -> None:
         self.cache.close(request)
 
-    def step(self, entries: list) -> torch.Tensor:
+    def step(self, entries: list, feed_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Returns float32 logits [wanted, vocab] in the order of the entries and of
-        each entry's `want`.  The tensor is a view of a buffer the next step reuses."""
+        each entry's `want`.  The tensor is a view of a buffer the next step reuses.
+        `feed_tokens` (int32, on the device) holds the tokens of entries with a `feed_row`: the
+        output of a sampling that the host has not read yet."""
+        if any(e.feed_row is not None for e in entries):
+            if feed_tokens is None:
+                raise StepError("an entry names a feed_row but the step was given no feed_tokens")
+        else:
+            feed_tokens = None
         graph = self._graph_for(entries) if entries else None
         if graph is not None:
             self._validate(entries)
             reserved = self._reserve(entries)
-            logits = graph.run(entries, reserved)
+            logits = graph.run(entries, reserved, feed_tokens)
             self.graph_steps += 1
         else:
             ctx = self.prepare(entries)
+            if feed_tokens is not None:
+                ops.feed_tokens(ctx.token_ids, ctx.feed_dst, ctx.feed_src, feed_tokens)
             logits = self.model.forward(ctx)
         self.commit(entries)
         return logits
@@ -119,6 +131,8 @@ class ModelRunner:
             if cache.context_len(e.request) + len(e.tokens) > max_pos:
                 raise StepError(f"request {e.request!r} would reach {cache.context_len(e.request) + len(e.tokens)} "
                                 f"tokens; the model allows {max_pos}")
+            if e.feed_row is not None and e.feed_row < 0:
+                raise StepError(f"request {e.request!r}: feed_row {e.feed_row} is negative")
             for w in e.want:
                 if not 0 <= w < len(e.tokens):
                     raise StepError(f"request {e.request!r}: wanted place {w} is not among its {len(e.tokens)} tokens")
@@ -166,8 +180,11 @@ class ModelRunner:
                 # a page given back (-1) lies outside every window that is still read
                 bt[i, :len(t)] = np.maximum(np.asarray(t, dtype=np.int32), 0)
             group_tables.append(bt)
+        fed = [i for i, e in enumerate(entries) if e.feed_row is not None]
+        feed_dst = np.array([q_start[i] + q_len[i] - 1 for i in fed], dtype=np.int32)
+        feed_src = np.array([entries[i].feed_row for i in fed], dtype=np.int32)
         arrays = [token_ids, positions, token_segment, q_start, q_len, ctx_len, state_slots, logit_rows]
-        arrays += group_slots + group_tables
+        arrays += group_slots + group_tables + [feed_dst, feed_src]
         dev = pack_int32(arrays, self.device)
         ctx = StepContext(
             n=n, num_segments=s, dtype=self.model.dtype, device=self.device, workspace=self.workspace,
@@ -177,4 +194,5 @@ class ModelRunner:
             group_slots=dev[8:8 + num_groups], group_block_tables=dev[8 + num_groups:8 + 2 * num_groups],
             host_q_start=q_start, host_q_len=q_len, host_ctx_len=ctx_len, host_state_slots=state_slots,
             requests=[e.request for e in entries])
+        ctx.feed_dst, ctx.feed_src = dev[8 + 2 * num_groups], dev[9 + 2 * num_groups]
         return ctx

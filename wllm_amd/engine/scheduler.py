@@ -27,9 +27,18 @@ without it.  The preempted request keeps the tokens it generated and recomputes 
 and outputs when it is admitted again (the reference drops the outputs,
 scheduler.py:303), so that a seeded request gives the same tokens with or without a
 preemption.
+
+Looking ahead.  With `lookahead=True` a step is started before the tokens of the step before it
+have been read: the sampled tokens stay on the device, the next step takes them from there
+(`StepEntry.feed_row`), and the host reads them while that step runs, so the GPU does not wait
+for the host between steps.  Whether a request ended on its end-of-sequence or a stop token is
+then known one step late: the request has been given one more token, which is dropped, and its
+pages go back one step later.  What each request generates is the same.  A request whose
+sampling needs the tokens it generated (a repetition penalty) is never run ahead.
 """
 from __future__ import annotations
 
+from dataclasses import dataclass, field
 from typing import Optional
 
 from wllm_amd.cache.pages import OutOfPages
@@ -42,9 +51,18 @@ class RequestRefused(ValueError):
     """A request that can never run: too long for the model or for the page pool."""
 
 
+@dataclass
+class _StartedStep:
+    """A step whose sampling has been enqueued and not been read."""
+    sampled: list                       # the requests that sample in it, in the order of its logits rows
+    places: list                        # for each, the index among its outputs that the token will fill
+    pending: object                     # the sampler's handle: tokens on the device, on their way to the host
+    dropped: set = field(default_factory=set)     # rows whose request ended before this step's token counted
+
+
 class Scheduler:
     def __init__(self, runner, max_prefill_tokens_per_step: Optional[int] = None, admission: str = "pledged",
-                 seed: int = 0, compute_logprobs: bool = True):
+                 seed: int = 0, compute_logprobs: bool = True, lookahead: bool = False):
         if admission not in ("pledged", "prompt_only"):
             raise ValueError(f"admission {admission!r}: expected 'pledged' or 'prompt_only'")
         if max_prefill_tokens_per_step is not None and max_prefill_tokens_per_step <= 0:
@@ -55,6 +73,8 @@ class Scheduler:
         self.admission = admission
         self.compute_logprobs = compute_logprobs
         self.sampler = Sampler(runner.device, seed)
+        self.lookahead = lookahead
+        self._started: Optional[_StartedStep] = None      # the step that has been started and not been read
         self.waiting: list = []
         self.running: list = []           # PREFILLING and RUNNING, in the order of admission
         self._arrivals = 0
@@ -83,10 +103,15 @@ class Scheduler:
         self.waiting.append(request)
 
     def has_unfinished_requests(self) -> bool:
-        return bool(self.waiting or self.running)
+        return bool(self.waiting or self.running or self._started is not None)
 
     def cancel(self, request_id) -> None:
         """Running: give back its pages; waiting: drop it; unknown: nothing (scheduler.py:158-176)."""
+        if self._started is not None:
+            for row, r in enumerate(self._started.sampled):
+                if r.request_id == request_id:
+                    self._started.dropped.add(row)
+                    del r.output_token_ids[self._started.places[row]:], r.logprobs[self._started.places[row]:]
         for i, r in enumerate(self.running):
             if r.request_id == request_id:
                 self.cache.close(request_id)
@@ -170,16 +195,40 @@ class Scheduler:
 
     def step(self) -> list:
         """One batch.  Returns the requests that got a token."""
+        if self._started is None:
+            self._started = self._start(None)
+            if self._started is None:
+                return []
+        current = self._started
+        self._started = self._start(current) if self.lookahead and self._may_run_ahead(current) else None
+        return self._finish(current)
+
+    @staticmethod
+    def _may_run_ahead(step: _StartedStep) -> bool:
+        """Not past a request whose next sampling needs the token that has not been read."""
+        return all(r.sampling_params.repetition_penalty == 1.0 for r in step.sampled)
+
+    def _start(self, before: Optional[_StartedStep]) -> Optional[_StartedStep]:
+        """Plans a step, runs it and enqueues its sampling; nothing is read.  `before` is the step
+        that has been started and not been read: its tokens are taken from the device."""
+        unread = {}
+        if before is not None:
+            unread = {id(r): row for row, r in enumerate(before.sampled) if row not in before.dropped}
         plan = self._plan()
         logits = None
         while plan:
             entries = []
             for r, take in plan:
                 completes = r.num_computed + take == r.num_tokens
+                # the last output of a request sampled in `before` is a placeholder on the host
+                feed = unread.get(id(r)) if completes and r.output_token_ids else None
                 entries.append(StepEntry(r.request_id, r.tokens(r.num_computed, r.num_computed + take),
-                                         [take - 1] if completes else []))
+                                         [take - 1] if completes else [], feed_row=feed))
             try:
-                logits = self.runner.step(entries)
+                if any(e.feed_row is not None for e in entries):
+                    logits = self.runner.step(entries, before.pending.tokens)
+                else:
+                    logits = self.runner.step(entries)
                 break
             except OutOfPages:
                 victim = self.running[-1]
@@ -188,7 +237,7 @@ class Scheduler:
                 self._preempt(victim)
                 plan = [(r, take) for r, take in plan if r is not victim]
         if not plan:
-            return []
+            return None
         self.stats["steps"] += 1
         held = sum(g.pool.num_pages - g.pool.num_free for g in self.cache.groups)
         self.stats["peak_pages"] = max(self.stats["peak_pages"], held)
@@ -201,18 +250,52 @@ class Scheduler:
             r.num_computed += take
             if r.num_computed == r.num_tokens:
                 sampled.append(r)
+        started = _StartedStep(sampled, [], None)
         if sampled:
-            tokens, logprobs = self.sampler.sample(
+            started.pending = self.sampler.start(
                 logits, [r.sampling_params for r in sampled], [r.seed for r in sampled],
                 [len(r.output_token_ids) for r in sampled], [r.output_token_ids for r in sampled],
                 want_logprobs=self.compute_logprobs)
-            for i, r in enumerate(sampled):
+            for r in sampled:
                 r.status = RequestStatus.RUNNING
-                r.append_token(tokens[i], logprobs[i] if logprobs is not None else None)
+                started.places.append(r.append_placeholder())       # may end the request by its length
         for r in [r for r in self.running if r.is_finished()]:
             self.cache.close(r.request_id)
         self.running = [r for r in self.running if not r.is_finished()]
-        return sampled
+        return started
+
+    def _finish(self, step: _StartedStep) -> list:
+        """Reads a started step's tokens and applies the rules that need their values."""
+        if not step.sampled:
+            return []
+        tokens, logprobs = self.sampler.finish(step.pending)
+        got = []
+        for row, r in enumerate(step.sampled):
+            if row in step.dropped:
+                continue
+            place = step.places[row]
+            r.output_token_ids[place] = int(tokens[row])
+            r.logprobs[place] = logprobs[row] if logprobs is not None else None
+            got.append(r)
+            if r.ends_with(tokens[row]):
+                # sequence.py:53-59: the stop rules come before the length rule
+                already_over = r.is_finished()
+                r.status, r.finish_reason = RequestStatus.FINISHED, "stop"
+                if already_over:
+                    continue
+                # the request may have been run ahead: that token does not count
+                ahead = self._started
+                if ahead is not None:
+                    for row2, r2 in enumerate(ahead.sampled):
+                        if r2 is r:
+                            ahead.dropped.add(row2)
+                del r.output_token_ids[place + 1:], r.logprobs[place + 1:]
+                if r in self.running:
+                    self.running.remove(r)
+                    self.cache.close(r.request_id)
+                elif r in self.waiting:         # preempted after it was sampled
+                    self.waiting.remove(r)
+        return got
 
     def run_to_completion(self, max_steps: int = 1_000_000) -> list:
         finished = []

@@ -22,12 +22,14 @@ def _ptr(t):
 
 
 _SIGNATURES = {
+    "wllm_feed_tokens": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "wllm_embed_lookup": [c_void_p, c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
     "wllm_rms_norm": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                       c_float, c_float, c_void_p],
     "wllm_rope_cache_write": [c_void_p, c_int, c_void_p, c_int, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p,
                               c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
-    "wllm_gemm_skinny_gated": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "wllm_gemm_skinny_gated": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "wllm_tile_weight": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "wllm_gated_activation": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_paged_attention_generic": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
@@ -39,9 +41,8 @@ _SIGNATURES = {
                                      c_void_p],
     "wllm_gemm_generic": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_argmax_rows": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
-    "wllm_gemm_skinny": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
-    "wllm_gemm_rows16": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
-    "wllm_gemm_rows16_gated": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "wllm_gemm_skinny": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                         c_void_p],
     "wllm_sample_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
 }
 
@@ -82,6 +83,11 @@ class HipBackend:
         self._check(self.lib.wllm_embed_lookup(_ptr(ids), _ptr(table), int(table.dtype == torch.bfloat16), scale,
                                                _ptr(out), ids.shape[0], table.shape[1], table.shape[0],
                                                self._stream()), "embed_lookup")
+
+    def feed_tokens(self, ids, dst, src, source):
+        self._on_gpu(ids, dst, src, source)
+        self._check(self.lib.wllm_feed_tokens(_ptr(ids), _ptr(dst), _ptr(src), _ptr(source), dst.shape[0], ids.shape[0],
+                                              source.shape[0], self._stream()), "feed_tokens")
 
     def rms_norm(self, x, weight, eps, offset, out, delta, rows):
         self._on_gpu(x, weight, out, delta, rows)
@@ -206,32 +212,38 @@ class HipBackend:
             return self.skinny_split(out_features, in_features)
         return 1
 
-    def _skinny(self, x, weight, out) -> None:
+    def tile_weight(self, weight, tiles) -> None:
+        self._on_gpu(weight, tiles)
+        self._check(self.lib.wllm_tile_weight(_ptr(weight), _ptr(tiles), weight.shape[0], weight.shape[1], self._stream()),
+                    "tile_weight")
+
+    def _skinny(self, x, weight, out, tiles=None) -> None:
         m, k = x.shape
         n = weight.shape[0]
         splits = self.skinny_split(n, k)
         chunk = self.SKINNY_CHUNK[-(-m // 16)]
+        w, tiled = (tiles, 1) if tiles is not None else (weight, 0)
         if out.dim() == 3:      # the caller adds the partial sums later
-            self._check(self.lib.wllm_gemm_skinny(_ptr(x), _ptr(weight), c_void_p(0), 0, _ptr(out), m, n, k, splits,
+            self._check(self.lib.wllm_gemm_skinny(_ptr(x), _ptr(w), tiled, c_void_p(0), 0, _ptr(out), m, n, k, splits,
                                                   chunk, self._stream()), "linear (few rows, partial sums)")
             return
         partial = self._gemm_partial(splits * m * n, x.device) if splits > 1 else None
-        self._check(self.lib.wllm_gemm_skinny(_ptr(x), _ptr(weight), _ptr(out), int(out.dtype == torch.bfloat16),
+        self._check(self.lib.wllm_gemm_skinny(_ptr(x), _ptr(w), tiled, _ptr(out), int(out.dtype == torch.bfloat16),
                                               _ptr(partial), m, n, k, splits, chunk, self._stream()),
                     "linear (few rows, matrix cores)")
 
-    def linear(self, x, weight, out):
-        self._on_gpu(x, weight, out)
+    def linear(self, x, weight, out, tiles=None):
+        self._on_gpu(x, weight, out, tiles)
         m, k = x.shape
         if x.dtype == torch.bfloat16:
             if self.skinny_takes(x.dtype, m, k):
-                self._skinny(x, weight, out)
+                self._skinny(x, weight, out, tiles)
                 return
             if k % 32 == 0 and out.dtype == torch.float32:
                 # float32 results from bfloat16 operands (logits at many rows): the few-row kernel
                 # in blocks of 64 rows
                 for r in range(0, m, 64):
-                    self._skinny(x[r:r + 64], weight, out[r:r + 64])
+                    self._skinny(x[r:r + 64], weight, out[r:r + 64], tiles)
                 return
             if out.dtype == torch.bfloat16 and m > 64:
                 # many rows: the library's matrix-core product (float32 accumulation)
@@ -241,12 +253,13 @@ class HipBackend:
             _ptr(x), _ptr(weight), int(x.dtype == torch.bfloat16), _ptr(out), int(out.dtype == torch.bfloat16),
             x.shape[0], weight.shape[0], x.shape[1], self._stream()), "linear")
 
-    def gated_linear(self, x, weight, out, activation, scratch):
-        self._on_gpu(x, weight, out, scratch)
+    def gated_linear(self, x, weight, out, activation, scratch, tiles=None):
+        self._on_gpu(x, weight, out, scratch, tiles)
         m, k = x.shape
+        w, tiled = (tiles, 1) if tiles is not None else (weight, 0)
         if self.skinny_takes(x.dtype, m, k) and k % 64 == 0:
             self._check(self.lib.wllm_gemm_skinny_gated(
-                _ptr(x), _ptr(weight), _ptr(out), m, out.shape[1], k, 0 if activation == "gelu_tanh" else 1,
+                _ptr(x), _ptr(w), tiled, _ptr(out), m, out.shape[1], k, 0 if activation == "gelu_tanh" else 1,
                 self.SKINNY_CHUNK[-(-m // 16)] // 2, self._stream()), "gated_linear (few rows, matrix cores)")
             return
         self.linear(x, weight, scratch)

@@ -71,6 +71,18 @@ def embed_lookup(ids: torch.Tensor, table: torch.Tensor, scale: float, out: torc
         backend().embed_lookup(ids, table, float(scale), out)
 
 
+def feed_tokens(ids: torch.Tensor, dst: torch.Tensor, src: torch.Tensor, source: torch.Tensor) -> None:
+    """ids[dst[j]] = source[src[j]] for every j with dst[j] >= 0 (entries out of range are skipped).
+    All int32 and one axis; dst and src of equal length.  It feeds a step the tokens that the step
+    before it sampled on the device."""
+    for t, name in ((ids, "ids"), (dst, "dst"), (src, "src"), (source, "source")):
+        _dense(t, name, torch.int32)
+        _need(t.dim() == 1, f"{name}: expected one axis")
+    _need(dst.shape == src.shape, "dst and src: expected equal lengths")
+    if dst.shape[0]:
+        backend().feed_tokens(ids, dst, src, source)
+
+
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, offset: float, out: torch.Tensor,
              delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None) -> None:
     """out = x * rsqrt(mean(x^2) + eps) * (offset + weight), all in float32, cast to out's dtype.
@@ -201,15 +213,50 @@ def linear_splits(rows: int, out_features: int, in_features: int, dtype: torch.d
     return int(backend().linear_splits(rows, out_features, in_features, dtype))
 
 
-def linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> None:
+def tiled_size(rows: int, in_features: int) -> int:
+    """Elements of the tile-major copy of a [rows, in_features] weight (`tile_weight`)."""
+    return -(-rows // 16) * 16 * in_features
+
+
+def tile_weight(weight: torch.Tensor, halves: int = 1) -> Optional[torch.Tensor]:
+    """The tile-major copy of a bfloat16 weight [n, k] that the few-row product kernels stream:
+    for each band of 16 rows (the last padded with zero rows) and each step of 32 keys, a tile of
+    1 KiB in which lane l = 16g + i of a wavefront finds w[16 * band + i][32 * step + 8g .. +8].
+    With halves = 2 (a stacked gate and up matrix) each half is tiled by itself, the gate's bands
+    first.  Returns a flat tensor, or None for weights the few-row kernels do not take (float32,
+    k not a multiple of 32)."""
+    _dense(weight, "weight", _ACT)
+    _need(weight.dim() == 2 and halves in (1, 2) and weight.shape[0] % halves == 0, "weight: expected [out, in]")
+    n, k = weight.shape[0] // halves, weight.shape[1]
+    if weight.dtype != torch.bfloat16 or k % 32 != 0 or n == 0:
+        return None
+    size = tiled_size(n, k)
+    tiles = torch.empty(halves * size, dtype=weight.dtype, device=weight.device)
+    for h in range(halves):
+        backend().tile_weight(weight[h * n:(h + 1) * n], tiles[h * size:(h + 1) * size])
+    return tiles
+
+
+def _check_tiles(tiles, weight, halves: int) -> None:
+    if tiles is None:
+        return
+    n, k = weight.shape[0] // halves, weight.shape[1]
+    _dense(tiles, "tiles", weight.dtype, (halves * tiled_size(n, k),))
+    _need(weight.dtype == torch.bfloat16 and k % 32 == 0, "tiles: only bfloat16 weights with in_features % 32 == 0 have them")
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, tiles: Optional[torch.Tensor] = None) -> None:
     """out = x @ weight^T.  x T [m, k]; weight T [n, k]; out T or float32 [m, n], or float32
     [S, m, n] with S = linear_splits(m, n, k, T): then the S slices are partial sums whose sum in
-    order is the product.  Products of bfloat16 accumulate in float32; float32 stays float32."""
+    order is the product.  Products of bfloat16 accumulate in float32; float32 stays float32.
+    `tiles` is `tile_weight(weight)`, the same numbers in the order the few-row kernels read
+    fastest; with it they read that copy instead."""
     _dense(x, "x", _ACT)
     _need(x.dim() == 2, "x: expected [rows, in]")
     _dense(weight, "weight", x.dtype)
     _need(weight.dim() == 2 and weight.shape[1] == x.shape[1],
           f"weight: shape {tuple(weight.shape)}, expected [out, {x.shape[1]}]")
+    _check_tiles(tiles, weight, 1)
     if out.dim() == 3:
         s = linear_splits(x.shape[0], weight.shape[0], x.shape[1], x.dtype)
         _dense(out, "out", torch.float32, (s, x.shape[0], weight.shape[0]))
@@ -217,7 +264,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> None:
     else:
         _dense(out, "out", (x.dtype, torch.float32), (x.shape[0], weight.shape[0]))
     if x.shape[0]:
-        backend().linear(x, weight, out)
+        backend().linear(x, weight, out, tiles)
 
 
 ACTIVATIONS = ("gelu_tanh", "silu")
@@ -234,9 +281,10 @@ def gated_activation(gate_up: torch.Tensor, out: torch.Tensor, activation: str) 
 
 
 def gated_linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, activation: str,
-                 scratch: torch.Tensor) -> None:
+                 scratch: torch.Tensor, tiles: Optional[torch.Tensor] = None) -> None:
     """out = act(x @ Wg^T) * (x @ Wu^T) with weight = [Wg; Wu] stacked, T [2I, k]; x T [m, k];
-    out T [m, I]; scratch T [m, 2I] may be used for the unfused product."""
+    out T [m, I]; scratch T [m, 2I] may be used for the unfused product.  `tiles` is
+    `tile_weight(weight, halves=2)`."""
     _need(activation in ACTIVATIONS, f"activation {activation!r}: expected one of {ACTIVATIONS}")
     _dense(x, "x", _ACT)
     _need(x.dim() == 2, "x: expected [rows, in]")
@@ -246,8 +294,9 @@ def gated_linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, activ
     inter = weight.shape[0] // 2
     _dense(out, "out", x.dtype, (x.shape[0], inter))
     _dense(scratch, "scratch", x.dtype, (x.shape[0], 2 * inter))
+    _check_tiles(tiles, weight, 2)
     if x.shape[0]:
-        backend().gated_linear(x, weight, out, activation, scratch)
+        backend().gated_linear(x, weight, out, activation, scratch, tiles)
 
 
 def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> None:

@@ -17,7 +17,7 @@ import torch
 
 from wllm_amd.cache.manager import CacheNeed
 from wllm_amd.kernels import ops
-from wllm_amd.parts.common import project
+from wllm_amd.parts.common import load_matrix, project
 from wllm_amd.parts.registry import build_position, register_mixer
 from wllm_amd.parts.specs import AttentionSpec
 from wllm_amd.weights.checkpoint import ExpectedTensor
@@ -60,8 +60,8 @@ class PagedAttention:
     def load(self, fetch) -> None:
         s = self.spec
         w = torch.cat([fetch.matrix(s.q_weight), fetch.matrix(s.k_weight), fetch.matrix(s.v_weight)], dim=0)
-        self.w_qkv = fetch.to_device(w)
-        self.w_o = fetch.to_device(fetch.matrix(s.o_weight))
+        self.w_qkv, self.t_qkv = load_matrix(fetch, w)        # the matrix and its tile-major copy
+        self.w_o, self.t_o = load_matrix(fetch, fetch.matrix(s.o_weight))
         if s.q_bias is not None or s.k_bias is not None or s.v_bias is not None:
             q, kv = s.num_heads * s.head_dim, s.num_kv_heads * s.head_dim
             parts = [fetch.vector(name) if name is not None else torch.zeros(width)
@@ -80,7 +80,7 @@ class PagedAttention:
         n = h.shape[0]
         qkv = ctx.buffer("qkv", (n, self.qkv_width), h.dtype)
         # where the product kernel splits its sums, the rotation kernel adds them as it reads
-        projected = project(ctx, "qkv", h, self.w_qkv, qkv)
+        projected = project(ctx, "qkv", h, self.w_qkv, qkv, tiles=self.t_qkv)
         parts = projected if projected.dim() == 3 else None
         pages = ctx.pages(entry)
         ops.rope_and_cache_write(
@@ -97,4 +97,4 @@ class PagedAttention:
             plan=ctx.attention_plan(num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim,
                                     page_size=pages.page_size, window=s.window or 0))
         # the next norm adds the contribution to the residual stream, partial sums and all
-        return project(ctx, "mixer_out", attn, self.w_o)
+        return project(ctx, "mixer_out", attn, self.w_o, tiles=self.t_o)

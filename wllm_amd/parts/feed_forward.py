@@ -7,7 +7,7 @@ from __future__ import annotations
 import torch
 
 from wllm_amd.kernels import ops
-from wllm_amd.parts.common import project
+from wllm_amd.parts.common import load_matrix, project
 from wllm_amd.parts.registry import register_feed_forward
 from wllm_amd.parts.specs import GatedMLPSpec
 from wllm_amd.weights.checkpoint import ExpectedTensor
@@ -19,8 +19,8 @@ class GatedMLP:
         if spec.activation not in ops.ACTIVATIONS:
             raise ValueError(f"activation {spec.activation!r} is not implemented; known: {ops.ACTIVATIONS}")
         self.spec = spec
-        self.w_gate_up = None
-        self.w_down = None
+        self.w_gate_up = self.t_gate_up = None      # the matrix and its tile-major copy
+        self.w_down = self.t_down = None
 
     def expected_tensors(self) -> dict:
         s = self.spec
@@ -32,13 +32,14 @@ class GatedMLP:
 
     def load(self, fetch) -> None:
         s = self.spec
-        self.w_gate_up = fetch.to_device(torch.cat([fetch.matrix(s.gate_weight), fetch.matrix(s.up_weight)], dim=0))
-        self.w_down = fetch.to_device(fetch.matrix(s.down_weight))
+        self.w_gate_up, self.t_gate_up = load_matrix(
+            fetch, torch.cat([fetch.matrix(s.gate_weight), fetch.matrix(s.up_weight)], dim=0), halves=2)
+        self.w_down, self.t_down = load_matrix(fetch, fetch.matrix(s.down_weight))
 
     def forward(self, ctx, h: torch.Tensor) -> torch.Tensor:
         s = self.spec
         n = h.shape[0]
         gate_up = ctx.buffer("gate_up", (n, 2 * s.intermediate_size), h.dtype)
         act = ctx.buffer("ffn_act", (n, s.intermediate_size), h.dtype)
-        ops.gated_linear(h, self.w_gate_up, act, s.activation, gate_up)
-        return project(ctx, "ffn_out", act, self.w_down)
+        ops.gated_linear(h, self.w_gate_up, act, s.activation, gate_up, self.t_gate_up)
+        return project(ctx, "ffn_out", act, self.w_down, tiles=self.t_down)

@@ -36,13 +36,21 @@ class Sampler:
         """logits float32 [m, V] (overwritten where a repetition penalty applies).
         Returns (tokens, logprobs) as Python lists; logprobs is None if they are not
         wanted and every row is greedy and unpenalised."""
+        return self.finish(self.start(logits, params, seeds, counters, generated, want_logprobs))
+
+    def start(self, logits: torch.Tensor, params: Sequence[SamplingParams], seeds: Sequence[int],
+              counters: Sequence[int], generated: Optional[Sequence[Sequence[int]]] = None,
+              want_logprobs: bool = True) -> "PendingSample":
+        """Enqueues the sampling and the copy of its results to the host and returns without
+        waiting.  `PendingSample.tokens` stays on the device: a step started before the results are
+        read takes its token ids from there."""
         m = logits.shape[0]
         assert len(params) == m and len(seeds) == m and len(counters) == m
         tokens = torch.empty(m, dtype=torch.int32, device=logits.device)
         plain_greedy = all(p.greedy and p.repetition_penalty == 1.0 for p in params)
         if plain_greedy and not want_logprobs:
             ops.argmax_rows(logits, tokens)
-            return tokens.tolist(), None
+            return PendingSample(tokens, None)
         table = np.array([[p.temperature, p.top_k, p.top_p, p.min_p, p.repetition_penalty] for p in params],
                          dtype=np.float32)
         keys = np.array([[s, c] for s, c in zip(seeds, counters)], dtype=np.int64)
@@ -59,4 +67,36 @@ class Sampler:
         logprobs = torch.empty(m, dtype=torch.float32, device=logits.device)
         ops.sample_rows(logits, torch.from_numpy(table).to(logits.device), torch.from_numpy(keys).to(logits.device),
                         pen_ids, pen_off, tokens, logprobs)
-        return tokens.tolist(), logprobs.tolist()
+        return PendingSample(tokens, logprobs)
+
+    @staticmethod
+    def finish(pending: "PendingSample"):
+        """Waits for a started sampling (and for nothing enqueued after it) and returns
+        (tokens, logprobs) as Python lists."""
+        return pending.read()
+
+
+class PendingSample:
+    """A sampling whose results are on their way to the host."""
+
+    def __init__(self, tokens: torch.Tensor, logprobs: Optional[torch.Tensor]):
+        self.tokens = tokens                # int32 [m] on the device
+        self.logprobs = logprobs
+        self._host_tokens = self._host_logprobs = self._event = None
+        if tokens.is_cuda:
+            # into pinned memory, with an event after the copies: reading them later does not wait
+            # for work that was enqueued after this sampling
+            self._host_tokens = torch.empty(tokens.shape, dtype=tokens.dtype, pin_memory=True)
+            self._host_tokens.copy_(tokens, non_blocking=True)
+            if logprobs is not None:
+                self._host_logprobs = torch.empty(logprobs.shape, dtype=logprobs.dtype, pin_memory=True)
+                self._host_logprobs.copy_(logprobs, non_blocking=True)
+            self._event = torch.cuda.Event()
+            self._event.record()
+
+    def read(self):
+        if self._event is None:
+            return self.tokens.tolist(), (self.logprobs.tolist() if self.logprobs is not None else None)
+        self._event.synchronize()
+        return (self._host_tokens.tolist(),
+                self._host_logprobs.tolist() if self._host_logprobs is not None else None)

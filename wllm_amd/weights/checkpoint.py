@@ -135,10 +135,12 @@ class TensorFetcher:
     32 bits stays so).  Integer tables are kept as int32.
     """
 
-    def __init__(self, checkpoint: Checkpoint, dtype: torch.dtype, device):
+    def __init__(self, checkpoint: Checkpoint, dtype: torch.dtype, device, tiled_copies: bool = False):
         self.checkpoint = checkpoint
         self.dtype = dtype
         self.device = device
+        # whether parts keep a second, tile-major copy of each matrix for the few-row product kernels
+        self.tiled_copies = tiled_copies
 
     def has(self, name: str) -> bool:
         return name in self.checkpoint

@@ -59,8 +59,9 @@ class RandomFetcher:
     generator (so not the same numbers as a written folder of that seed)."""
 
     def __init__(self, expected: dict, seed: int, dtype: torch.dtype, device, std: float = 0.02,
-                 norm_std: float = 0.1):
+                 norm_std: float = 0.1, tiled_copies: bool = False):
         self.expected, self.dtype, self.device = expected, dtype, torch.device(device)
+        self.tiled_copies = tiled_copies
         self.std, self.norm_std = std, norm_std
         self._gen = torch.Generator(device=self.device)
         self._seed = seed
