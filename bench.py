@@ -247,7 +247,7 @@ def main() -> int:
             "num_key_value_heads": c.num_key_value_heads, "head_dim": c.head_dim, "vocab_size": c.vocab_size,
             "tied_embeddings": c.tie_word_embeddings, "rope_theta": c.rope_theta, "rms_norm_eps": c.rms_norm_eps,
             "max_position_embeddings": c.max_position_embeddings, "kv_block_size": args.block_size,
-            "sampling": "greedy", "hip_graphs": graphs,
+            "sampling": "greedy", "hip_graphs": graphs, "lookahead": True,
         },
         "prefill": {"value": round(args.prefill_tokens / t_prefill, 1), "tokens": args.prefill_tokens,
                     "ms": round(1000.0 * t_prefill, 3),
