@@ -294,15 +294,34 @@ attention_reduce_kernel(const int* __restrict__ reduce_items, const float* __res
     if (row0 + r >= seg_q_len[seg] * group) return;
     const float* ml = partial_ml + (static_cast<size_t>(first) * kRowsPerTile + r) * 2;
     const float* po = partial_o + (static_cast<size_t>(first) * kRowsPerTile + r) * HD + d;
-    float m = -INFINITY;
-    for (int s = 0; s < splits; ++s) m = fmaxf(m, ml[s * stride * 2]);
-    float num = 0.f, den = 0.f;
-#pragma unroll 4
-    for (int s = 0; s < splits; ++s) {
-        const float ms = ml[s * stride * 2];
-        const float f = ms == -INFINITY ? 0.f : exp2f((ms - m) * scale_log2e);
-        num = fmaf(po[s * stride * HD], f, num);
-        den = fmaf(ml[s * stride * 2 + 1], f, den);
+    // One pass in groups of eight splits: all loads of a group are issued together, and the sums are
+    // rescaled when a group raises the maximum, so the kernel makes one trip to memory per group.
+    float m = -INFINITY, num = 0.f, den = 0.f;
+    for (int s0 = 0; s0 < splits; s0 += 8) {
+        float ms[8], ls[8], ps[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const bool ok = s0 + u < splits;
+            const size_t at = static_cast<size_t>(ok ? s0 + u : s0) * stride;
+            ms[u] = ml[at * 2];
+            ls[u] = ml[at * 2 + 1];
+            ps[u] = po[at * HD];
+            if (!ok) ms[u] = -INFINITY;
+        }
+        float m_new = m;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) m_new = fmaxf(m_new, ms[u]);
+        if (m_new == -INFINITY) continue;       // nothing seen yet
+        const float keep = m == -INFINITY ? 0.f : exp2f((m - m_new) * scale_log2e);
+        num *= keep;
+        den *= keep;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const float f = ms[u] == -INFINITY ? 0.f : exp2f((ms[u] - m_new) * scale_log2e);
+            num = fmaf(ps[u], f, num);
+            den = fmaf(ls[u], f, den);
+        }
+        m = m_new;
     }
     const int row = row0 + r;
     const int tok = row / group, head = kvh * group + row % group;

@@ -220,6 +220,12 @@ WLLM_API int wllm_gemm_skinny(const void* x, const void* w, int tiled, void* out
         if (tiles / 4 * splits >= 1024) nt = 4;
         else if (tiles / 2 * splits >= 1024) nt = 2;
     }
+    // a wavefront reads its weights in batches of 16 / nt steps of 32 keys, and a batch must not be
+    // longer than a chunk of x (else steps would be read twice)
+    if (chunk < k_per_split) {
+        while (nt < 4 && (16 / nt) * 32 > chunk) nt *= 2;
+        if ((16 / nt) * 32 > chunk) return -1;
+    }
     const dim3 grid((N + 64 * nt - 1) / (64 * nt), splits);
 #define LAUNCH_T(MT, NT, TO, T)                                                                                  \
     gemm_skinny_kernel<MT, NT, TO, T><<<grid, 256, smem, stream>>>(static_cast<const bf16*>(x), static_cast<const bf16*>(w), \
@@ -233,7 +239,7 @@ WLLM_API int wllm_gemm_skinny(const void* x, const void* w, int tiled, void* out
     else LAUNCH(MT, 1, TO)
 #define BY_MT(TO)                         \
     switch (mt) {                         \
-        case 1: LAUNCH(1, 1, TO); break;  \
+        case 1: BY_NT(1, TO); break;      \
         case 2: BY_NT(2, TO); break;      \
         case 3: BY_NT(3, TO); break;      \
         default: BY_NT(4, TO); break;     \
@@ -311,7 +317,7 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
     int step = 0;
     const int tid_half = threadIdx.x % 256;
     // x is staged chunk by chunk (per half of K); the next chunk's loads are in flight during the products
-    constexpr int kXRegs = 4;                     // MT*16*chunk/8 <= 1024 pieces for 256 threads
+    constexpr int kXRegs = MT >= 3 ? 8 : 4;       // MT*16*chunk/8 <= 256 * kXRegs pieces for 256 threads
     uint4 xreg[kXRegs];
     auto fetch_x = [&](int kc) {
         const int vecs = min(chunk, half_k - kc) / 8;
@@ -403,11 +409,22 @@ WLLM_API int wllm_gemm_skinny_gated(const void* x, const void* w, int tiled, voi
     size_t smem = static_cast<size_t>(2) * mt * 16 * (chunk / 8 + 1) * sizeof(uint4);
     const size_t red = static_cast<size_t>(4) * kWave * mt * 8 * sizeof(float);
     if (red > smem) smem = red;
-    if (smem > 65536 || mt * 16 * (chunk / 8) > 1024) return -1;     // 4 pieces of x per thread at most
+    // 4 pieces of x per thread (8 from 33 rows on); a batch of 8 steps must not be longer than a chunk
+    if (smem > 160 * 1024 - 4096 || mt * 16 * (chunk / 8) > (mt >= 3 ? 2048 : 1024) || (chunk < 256 && chunk < K / 2))
+        return -1;
     const dim3 grid((inter + 63) / 64);
 #define LAUNCH_T(MT, A, T)                                                                                            \
-    gemm_skinny_gated_kernel<MT, A, T><<<grid, 512, smem, stream>>>(static_cast<const bf16*>(x), static_cast<const bf16*>(w), \
-                                                                    static_cast<bf16*>(out), M, inter, K, chunk)
+    do {                                                                                                              \
+        static bool roomy = false;     /* more than 64 KiB of shared memory must be asked for once */                \
+        if (smem > 65536 && !roomy) {                                                                                 \
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_gated_kernel<MT, A, T>),               \
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 4096) != hipSuccess)    \
+                return launch_status();                                                                               \
+            roomy = true;                                                                                             \
+        }                                                                                                             \
+        gemm_skinny_gated_kernel<MT, A, T><<<grid, 512, smem, stream>>>(                                             \
+            static_cast<const bf16*>(x), static_cast<const bf16*>(w), static_cast<bf16*>(out), M, inter, K, chunk);   \
+    } while (0)
 #define LAUNCH(MT, A)                  \
     if (tiled) LAUNCH_T(MT, A, true);  \
     else LAUNCH_T(MT, A, false)

@@ -202,6 +202,7 @@ class HipBackend:
         return self._gemm_partials
 
     SKINNY_CHUNK = {1: 1024, 2: 512, 3: 256, 4: 256}     # K elements of x staged at a time, by row tiles
+    GATED_CHUNK = {1: 512, 2: 256, 3: 256, 4: 256}       # the same per half of K in the gated product
 
     @staticmethod
     def skinny_takes(dtype, rows: int, in_features: int) -> bool:
@@ -260,7 +261,7 @@ class HipBackend:
         if self.skinny_takes(x.dtype, m, k) and k % 64 == 0:
             self._check(self.lib.wllm_gemm_skinny_gated(
                 _ptr(x), _ptr(w), tiled, _ptr(out), m, out.shape[1], k, 0 if activation == "gelu_tanh" else 1,
-                self.SKINNY_CHUNK[-(-m // 16)] // 2, self._stream()), "gated_linear (few rows, matrix cores)")
+                self.GATED_CHUNK[-(-m // 16)], self._stream()), "gated_linear (few rows, matrix cores)")
             return
         self.linear(x, weight, scratch)
         self.gated_activation(scratch, out, activation)
