@@ -92,21 +92,20 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* _
 #pragma unroll
         for (int t = 0; t < MT; ++t) acc[nt][t] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    // The weight stream is read in batches of kBatch 16-byte loads per lane and tile; the next batch
-    // is in flight while the products of this one are made, the first before x is staged at all.
+    // The weight stream: kBatch 16-byte loads per lane and tile are in flight, the first before x is
+    // staged at all; a register is refilled with the step kBatch further on as soon as its products
+    // have been issued.
     constexpr int kBatch = 16 / NT;
     const bool live = n0 < N;
     const int steps = (k_end - k_begin) / 32;
-    Frag cur[NT][kBatch], nxt[NT][kBatch];
-    auto fetch = [&](Frag (&dst)[NT][kBatch], int step0) {
+    Frag cur[NT][kBatch];
+    auto load_step = [&](int u, int at) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u)
-                dst[nt][u].u = (live && step0 + u < steps) ? *reinterpret_cast<const uint4*>(wp[nt] + (step0 + u) * kStep)
-                                                           : make_uint4(0, 0, 0, 0);
+            cur[nt][u].u = (live && at < steps) ? *reinterpret_cast<const uint4*>(wp[nt] + at * kStep) : make_uint4(0, 0, 0, 0);
     };
-    fetch(cur, 0);
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) load_step(u, u);
     // x is staged chunk by chunk; the loads of the next chunk are in flight during the products
     constexpr int kXRegs = 8;                     // 16-byte pieces of a chunk per thread (MT*16*chunk/8 <= 2048)
     uint4 xreg[kXRegs];
@@ -123,7 +122,7 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* _
     fetch_x(k_begin);
     int step = 0;
     for (int kc = k_begin; kc < k_end; kc += chunk) {
-        const int len = min(chunk, k_end - kc);   // a multiple of 32
+        const int len = min(chunk, k_end - kc);   // a multiple of 32 * kBatch, except the last
         const int vecs = len / 8;
         __syncthreads();
 #pragma unroll
@@ -134,8 +133,6 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* _
         __syncthreads();
         if (kc + chunk < k_end) fetch_x(kc + chunk);
         for (int k = 0; k < len; k += 32 * kBatch) {
-            const int used = min(kBatch, (len - k) / 32);      // steps of this batch that lie in the chunk
-            fetch(nxt, step + used);
 #pragma unroll
             for (int u = 0; u < kBatch; ++u) {
                 if (k + 32 * u < len) {
@@ -147,13 +144,10 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* _
 #pragma unroll
                         for (int t = 0; t < MT; ++t)
                             acc[nt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[nt][u].v, b[t].v, acc[nt][t], 0, 0, 0);
+                    load_step(u, step + u + kBatch);
                 }
             }
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                for (int u = 0; u < kBatch; ++u) cur[nt][u] = nxt[nt][u];
-            step += used;
+            step += kBatch;
         }
     }
     if (!live) return;
@@ -220,11 +214,11 @@ WLLM_API int wllm_gemm_skinny(const void* x, const void* w, int tiled, void* out
         if (tiles / 4 * splits >= 1024) nt = 4;
         else if (tiles / 2 * splits >= 1024) nt = 2;
     }
-    // a wavefront reads its weights in batches of 16 / nt steps of 32 keys, and a batch must not be
-    // longer than a chunk of x (else steps would be read twice)
+    // a wavefront reads its weights in batches of 16 / nt steps of 32 keys; a chunk of x that is not the
+    // last must be whole batches
     if (chunk < k_per_split) {
-        while (nt < 4 && (16 / nt) * 32 > chunk) nt *= 2;
-        if ((16 / nt) * 32 > chunk) return -1;
+        while (nt < 4 && chunk % ((16 / nt) * 32) != 0) nt *= 2;
+        if (chunk % ((16 / nt) * 32) != 0) return -1;     // a register's step is fixed by its place in the batch
     }
     const dim3 grid((N + 64 * nt - 1) / (64 * nt), splits);
 #define LAUNCH_T(MT, NT, TO, T)                                                                                  \
@@ -271,18 +265,19 @@ __device__ __forceinline__ float act_gelu_tanh(float z) {
 }
 __device__ __forceinline__ float act_silu(float z) { return z / (1.f + expf(-z)); }
 
-// A workgroup is 8 wavefronts: 4 tiles of 16 gate rows (with their up rows) times 2 halves of the
-// K axis, so that two wavefronts per SIMD keep loads in flight; the halves are added through shared
-// memory in a fixed order before the activation.
-template <int MT, int ACT, bool TILED>
-__global__ void __launch_bounds__(512)
+// A workgroup is TPW tiles of 16 gate rows (with their up rows) times 2 halves of the K axis; the
+// halves are added through shared memory in a fixed order before the activation.  With few rows of
+// x (MT <= 2) the kernel needs few registers, a workgroup is 2 tiles (4 wavefronts), and four
+// workgroups share a compute unit: 16 wavefronts with 16 loads each in flight.
+template <int MT, int ACT, bool TILED, int TPW>
+__global__ void __launch_bounds__(TPW * 128, MT == 1 ? 4 : (MT == 2 ? 3 : 2))
 gemm_skinny_gated_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, bf16* __restrict__ out, int M,
                          int inter, int K, int chunk) {
     extern __shared__ uint4 xs[];                 // two halves of [MT*16][chunk/8 + 1]
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const int i = lane % 16, g = lane / 16;
-    const int tile = wave % 4, half = wave / 4;
-    const int n0 = (blockIdx.x * 4 + tile) * 16;
+    const int tile = wave % TPW, half = wave / TPW;
+    const int n0 = (blockIdx.x * TPW + tile) * 16;
     const int stride = chunk / 8 + 1;
     const int half_k = K / 2;                     // a multiple of 32
     const int k_begin = half * half_k;
@@ -301,29 +296,31 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
         accg[t] = float4_t{0.f, 0.f, 0.f, 0.f};
         accu[t] = float4_t{0.f, 0.f, 0.f, 0.f};
     }
+    // The weight stream: kBatch 16-byte loads per lane and stream are in flight; a register is
+    // refilled with the step kBatch further on as soon as its product has been issued, so the loads
+    // in flight take 16 registers a stream and not twice that, and two workgroups fit a compute unit.
     constexpr int kBatch = 8;       // per stream; two streams
     const bool live = n0 < inter;
     const int steps = half_k / 32;
-    Frag curg[kBatch], curu[kBatch], nxtg[kBatch], nxtu[kBatch];
-    auto fetch = [&](Frag* dg, Frag* du, int step0) {
-#pragma unroll
-        for (int u = 0; u < kBatch; ++u) {
-            const bool ok = live && step0 + u < steps;
-            dg[u].u = ok ? *reinterpret_cast<const uint4*>(gp + (step0 + u) * kStep) : make_uint4(0, 0, 0, 0);
-            du[u].u = ok ? *reinterpret_cast<const uint4*>(up + (step0 + u) * kStep) : make_uint4(0, 0, 0, 0);
-        }
+    Frag curg[kBatch], curu[kBatch];
+    auto load_step = [&](int u, int at) {
+        const bool ok = live && at < steps;
+        curg[u].u = ok ? *reinterpret_cast<const uint4*>(gp + at * kStep) : make_uint4(0, 0, 0, 0);
+        curu[u].u = ok ? *reinterpret_cast<const uint4*>(up + at * kStep) : make_uint4(0, 0, 0, 0);
     };
-    fetch(curg, curu, 0);
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) load_step(u, u);
     int step = 0;
-    const int tid_half = threadIdx.x % 256;
+    constexpr int kHalfThreads = TPW * 64;        // the threads that stage one half's x
+    const int tid_half = threadIdx.x % kHalfThreads;
     // x is staged chunk by chunk (per half of K); the next chunk's loads are in flight during the products
-    constexpr int kXRegs = MT >= 3 ? 8 : 4;       // MT*16*chunk/8 <= 256 * kXRegs pieces for 256 threads
+    constexpr int kXRegs = MT == 1 ? 4 : 8;       // MT*16*chunk/8 <= kHalfThreads * kXRegs pieces
     uint4 xreg[kXRegs];
     auto fetch_x = [&](int kc) {
         const int vecs = min(chunk, half_k - kc) / 8;
 #pragma unroll
         for (int u = 0; u < kXRegs; ++u) {
-            const int idx = tid_half + u * 256;
+            const int idx = tid_half + u * kHalfThreads;
             const int m = idx / vecs, c = idx % vecs;
             xreg[u] = (idx < MT * 16 * vecs && m < M)
                           ? *reinterpret_cast<const uint4*>(x + static_cast<size_t>(m) * K + k_begin + kc + c * 8)
@@ -332,19 +329,17 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
     };
     fetch_x(0);
     for (int kc = 0; kc < half_k; kc += chunk) {
-        const int len = min(chunk, half_k - kc);
+        const int len = min(chunk, half_k - kc);      // a multiple of 32 * kBatch, except the last
         const int vecs = len / 8;
         __syncthreads();
 #pragma unroll
         for (int u = 0; u < kXRegs; ++u) {
-            const int idx = tid_half + u * 256;
+            const int idx = tid_half + u * kHalfThreads;
             if (idx < MT * 16 * vecs) xh[(idx / vecs) * stride + idx % vecs] = xreg[u];
         }
         __syncthreads();
         if (kc + chunk < half_k) fetch_x(kc + chunk);
         for (int k = 0; k < len; k += 32 * kBatch) {
-            const int used = min(kBatch, (len - k) / 32);
-            fetch(nxtg, nxtu, step + used);
 #pragma unroll
             for (int u = 0; u < kBatch; ++u) {
                 if (k + 32 * u < len) {
@@ -355,14 +350,10 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
                         accg[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(curg[u].v, b.v, accg[t], 0, 0, 0);
                         accu[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(curu[u].v, b.v, accu[t], 0, 0, 0);
                     }
+                    load_step(u, step + u + kBatch);
                 }
             }
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u) {
-                curg[u] = nxtg[u];
-                curu[u] = nxtu[u];
-            }
-            step += used;
+            step += kBatch;
         }
     }
     // the second half hands its sums to the first through shared memory
@@ -406,28 +397,31 @@ WLLM_API int wllm_gemm_skinny_gated(const void* x, const void* w, int tiled, voi
     if (M < 1 || M > 64 || K % 64 != 0 || chunk % 32 != 0 || activation < 0 || activation > 1) return -1;
     const int mt = (M + 15) / 16;
     if (chunk > K / 2) chunk = K / 2;
+    const int tpw = mt <= 2 ? 2 : 4;                 // tiles of 16 gate rows per workgroup
     size_t smem = static_cast<size_t>(2) * mt * 16 * (chunk / 8 + 1) * sizeof(uint4);
-    const size_t red = static_cast<size_t>(4) * kWave * mt * 8 * sizeof(float);
+    const size_t red = static_cast<size_t>(tpw) * kWave * mt * 8 * sizeof(float);
     if (red > smem) smem = red;
-    // 4 pieces of x per thread (8 from 33 rows on); a batch of 8 steps must not be longer than a chunk
-    if (smem > 160 * 1024 - 4096 || mt * 16 * (chunk / 8) > (mt >= 3 ? 2048 : 1024) || (chunk < 256 && chunk < K / 2))
+    // the pieces of x a thread stages (4 up to 16 rows, else 8); a chunk that is not the last must be
+    // whole batches of 8 steps, because a register's step is fixed by its place
+    const int x_regs = mt == 1 ? 4 : 8;
+    if (smem > 160 * 1024 - 4096 || mt * 16 * (chunk / 8) > tpw * 64 * x_regs || (chunk % 256 != 0 && chunk < K / 2))
         return -1;
-    const dim3 grid((inter + 63) / 64);
-#define LAUNCH_T(MT, A, T)                                                                                            \
+    const dim3 grid((inter + 16 * tpw - 1) / (16 * tpw));
+#define LAUNCH_T(MT, A, T, TPW)                                                                                       \
     do {                                                                                                              \
         static bool roomy = false;     /* more than 64 KiB of shared memory must be asked for once */                \
         if (smem > 65536 && !roomy) {                                                                                 \
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_gated_kernel<MT, A, T>),               \
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_gated_kernel<MT, A, T, TPW>),          \
                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 4096) != hipSuccess)    \
                 return launch_status();                                                                               \
             roomy = true;                                                                                             \
         }                                                                                                             \
-        gemm_skinny_gated_kernel<MT, A, T><<<grid, 512, smem, stream>>>(                                             \
+        gemm_skinny_gated_kernel<MT, A, T, TPW><<<grid, TPW * 128, smem, stream>>>(                                  \
             static_cast<const bf16*>(x), static_cast<const bf16*>(w), static_cast<bf16*>(out), M, inter, K, chunk);   \
     } while (0)
-#define LAUNCH(MT, A)                  \
-    if (tiled) LAUNCH_T(MT, A, true);  \
-    else LAUNCH_T(MT, A, false)
+#define LAUNCH(MT, A)                                        \
+    if (tiled) LAUNCH_T(MT, A, true, (MT <= 2 ? 2 : 4));      \
+    else LAUNCH_T(MT, A, false, (MT <= 2 ? 2 : 4))
 #define BY_MT(A)                     \
     switch (mt) {                    \
         case 1: LAUNCH(1, A); break; \

@@ -202,7 +202,7 @@ class HipBackend:
         return self._gemm_partials
 
     SKINNY_CHUNK = {1: 1024, 2: 512, 3: 256, 4: 256}     # K elements of x staged at a time, by row tiles
-    GATED_CHUNK = {1: 512, 2: 256, 3: 256, 4: 256}       # the same per half of K in the gated product
+    GATED_CHUNK = {1: 256, 2: 256, 3: 256, 4: 256}       # the same per half of K in the gated product
 
     @staticmethod
     def skinny_takes(dtype, rows: int, in_features: int) -> bool:
