@@ -302,11 +302,10 @@ attention_reduce_kernel(const int* __restrict__ reduce_items, const float* __res
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const bool ok = s0 + u < splits;
-            const size_t at = static_cast<size_t>(ok ? s0 + u : s0) * stride;
-            ms[u] = ml[at * 2];
-            ls[u] = ml[at * 2 + 1];
-            ps[u] = po[at * HD];
-            if (!ok) ms[u] = -INFINITY;
+            const size_t at = static_cast<size_t>(s0 + u) * stride;
+            ms[u] = ok ? ml[at * 2] : -INFINITY;
+            ls[u] = ok ? ml[at * 2 + 1] : 0.f;
+            ps[u] = ok ? po[at * HD] : 0.f;
         }
         float m_new = m;
 #pragma unroll

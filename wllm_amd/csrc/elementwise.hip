@@ -167,23 +167,30 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, const float* __restrict__
     }
     // rotated pairs of query and key heads
     const int rot_heads = num_heads + num_kv_heads;
-    for (int idx = threadIdx.x; idx < rot_heads * half; idx += blockDim.x) {
-        const int head = idx / half, j = idx % half;
-        const int ia = head * head_dim + j, ib = ia + half;
-        float a = value(ia), b = value(ib);
-        if (bias) {
-            a += bias[ia];
-            b += bias[ib];
-        }
+    // a thread keeps one pair index j and walks the heads, so the sine and cosine of its angle are
+    // computed once; threads beyond `half` start at further heads
+    const int lanes_j = max(1, min(static_cast<int>(blockDim.x), half));
+    const int head_step = max(1, static_cast<int>(blockDim.x) / lanes_j);
+    for (int j = threadIdx.x % lanes_j; j < half; j += lanes_j) {
+        const int head_first = threadIdx.x / lanes_j;
+        if (head_first >= head_step) break;          // threads that do not fit a whole group of heads idle
         float s, c;
         sincosf(pos * inv_freq[j], &s, &c);
-        const T ra = from_float<T>(a * c - b * s), rb = from_float<T>(b * c + a * s);
-        row[ia] = ra;
-        row[ib] = rb;
-        if (kpage && head >= num_heads) {
-            T* dst = kpage + (static_cast<size_t>(head - num_heads) * page_size + off) * head_dim;
-            dst[j] = ra;
-            dst[j + half] = rb;
+        for (int head = head_first; head < rot_heads; head += head_step) {
+            const int ia = head * head_dim + j, ib = ia + half;
+            float a = value(ia), b = value(ib);
+            if (bias) {
+                a += bias[ia];
+                b += bias[ib];
+            }
+            const T ra = from_float<T>(a * c - b * s), rb = from_float<T>(b * c + a * s);
+            row[ia] = ra;
+            row[ib] = rb;
+            if (kpage && head >= num_heads) {
+                T* dst = kpage + (static_cast<size_t>(head - num_heads) * page_size + off) * head_dim;
+                dst[j] = ra;
+                dst[j + half] = rb;
+            }
         }
     }
     // the part of query and key heads that is not rotated
