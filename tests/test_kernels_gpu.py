@@ -226,6 +226,8 @@ MFMA_SHAPES = ATTENTION_SHAPES + [
     (8, 2, 64, 16, [(1, 1000), (40, 500)], 300),                                   # window over several key chunks
     (10, 5, 160, 32, [(1, 90), (33, 33)], 0),
     (3, 1, 224, 16, [(1, 400), (6, 6), (7, 20)], 0),                               # group of 3: rows straddle tokens
+    (4, 2, 64, 12, [(1, 300), (2, 77), (1, 5), (1, 128), (1, 129)], 0),            # pages that do not divide 128 keys
+    (8, 2, 64, 20, [(1, 500), (3, 90), (1, 260)], 70),                             # the same with a window
 ]
 
 

@@ -301,11 +301,13 @@ attention_reduce_kernel(const int* __restrict__ reduce_items, const float* __res
         float ms[8], ls[8], ps[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
+            // a split beyond the last reads the last one again (the same addresses) and does not count
             const bool ok = s0 + u < splits;
-            const size_t at = static_cast<size_t>(s0 + u) * stride;
-            ms[u] = ok ? ml[at * 2] : -INFINITY;
-            ls[u] = ok ? ml[at * 2 + 1] : 0.f;
-            ps[u] = ok ? po[at * HD] : 0.f;
+            const size_t at = static_cast<size_t>(ok ? s0 + u : splits - 1) * stride;
+            const float m_at = ml[at * 2];
+            ms[u] = ok ? m_at : -INFINITY;
+            ls[u] = ml[at * 2 + 1];
+            ps[u] = po[at * HD];
         }
         float m_new = m;
 #pragma unroll
