@@ -55,6 +55,22 @@ class EmulatedKernels:
         y = v * torch.rsqrt(var + eps) * (offset + weight.to(self.acc))
         out.copy_(y.to(out.dtype))
 
+    fused_qkv = True        # whether the emulation offers the fused projection and rotation
+
+    def qkv_rope_takes(self, rows, dtype, in_features, head_dim, rotary_dim):
+        return self.fused_qkv and rotary_dim == head_dim and rows <= 16
+
+    def qkv_rope(self, x, weight, tiles, qkv, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads,
+                 head_dim, page_size):
+        self._count("qkv_rope")
+        self._same_numbers(weight, tiles, 1)
+        # the kernel rotates the float32 sums, not their rounding to the activation dtype: hand them
+        # on as a stack of one partial sum
+        pre = (x.to(self.acc) @ weight.to(self.acc).T).to(torch.float32)[None]
+        self.rope_and_cache_write(qkv, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads, head_dim,
+                                  head_dim if inv_freq is not None else 0, page_size, parts=pre)
+        self.calls["rope_and_cache_write"] -= 1
+
     def rope_and_cache_write(self, qkv, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads,
                              head_dim, rotary_dim, page_size, parts=None):
         self._count("rope_and_cache_write")

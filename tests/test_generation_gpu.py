@@ -191,11 +191,17 @@ def test_looking_ahead_gives_the_same_tokens_on_the_gpu(model_folders, dtype, gr
     news = [30, 12, 25, 8, 40, 18, 22]
     params = [SamplingParams(temperature=0.7, top_p=0.9, seed=40 + i) if i % 2 else SamplingParams() for i in range(7)]
 
+    # Looking ahead changes which requests share a step (a request that stops is in one step more).
+    # In bfloat16 the kernels for at most 16 rows and for more round differently, so the portions
+    # are kept small enough that every step of both runs has at most 16 rows and takes the same
+    # kernels; float32 has no such boundary.
+    budget = 16 if dtype == "float32" else 8
+
     def run(lookahead, stops):
         runner = ModelRunner.create(model, num_pages=40, page_size=16, max_requests=4)
         if graphs:
             runner.enable_graphs(buckets=(1, 2, 4))
-        s = Scheduler(runner, max_prefill_tokens_per_step=16, lookahead=lookahead)
+        s = Scheduler(runner, max_prefill_tokens_per_step=budget, lookahead=lookahead)
         reqs = [Request(i, p, n, sampling_params=sp, **stops.get(i, {}))
                 for i, (p, n, sp) in enumerate(zip(prompts, news, params))]
         for r in reqs:

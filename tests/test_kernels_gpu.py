@@ -416,3 +416,35 @@ def test_feed_tokens_writes_only_the_named_places():
     source = torch.tensor([100, 200, 300], dtype=torch.int32, device=DEV)
     ops.feed_tokens(ids, dst, src, source)
     assert ids.tolist() == [0, 1, 2, 100, 4, 5, 6, 300, 8, 9]
+
+
+@pytest.mark.parametrize("tiled", [False, True])
+@pytest.mark.parametrize("m,k,nh,nkv,d,ps,with_bias,with_cache", [
+    (8, 2048, 8, 1, 256, 16, False, True), (16, 96, 3, 1, 32, 4, True, True), (1, 320, 4, 2, 64, 8, False, True),
+    (5, 4128, 2, 2, 96, 12, True, True), (3, 64, 5, 5, 128, 16, False, False)])
+def test_qkv_projection_rotation_and_cache_write_in_one_kernel(tiled, m, k, nh, nkv, d, ps, with_bias, with_cache):
+    dtype = torch.bfloat16
+    assert ops.qkv_rope_takes(m, dtype, k, d, d)
+    assert not ops.qkv_rope_takes(17, dtype, k, d, d) and not ops.qkv_rope_takes(m, torch.float32, k, d, d)
+    assert not ops.qkv_rope_takes(m, dtype, k, d, d // 2), "heads rotated in part take the two kernels"
+    width = (nh + 2 * nkv) * d
+
+    def make():
+        g = torch.Generator(device="cpu").manual_seed(21)
+        x = torch.randn(m, k, generator=g).to(dtype).to(DEV)
+        w = (torch.randn(width, k, generator=g) / math.sqrt(k)).to(dtype).to(DEV)
+        bias = (torch.randn(width, generator=g) * 0.3).to(DEV) if with_bias else None
+        positions = torch.randint(0, 3000, (m,), generator=g, dtype=torch.int32).to(DEV)
+        inv_freq = (1.0 / (10000.0 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).to(DEV)
+        pages = m + 3
+        slots = (torch.randperm(pages * ps, generator=g)[:m]).to(torch.int32).to(DEV) if with_cache else None
+        cache = torch.zeros(pages, 2, nkv, ps * d, dtype=dtype, device=DEV) if with_cache else None
+        qkv = torch.zeros(m, width, dtype=dtype, device=DEV)
+        return [x, w, qkv, bias, positions, inv_freq, slots, cache], dict(
+            num_heads=nh, num_kv_heads=nkv, head_dim=d, page_size=ps, tiles=ops.tile_weight(w) if tiled else None)
+
+    g_, r_ = both("qkv_rope", make, dtype)
+    close(g_[2], r_[2], dtype, "rotated queries, keys and values")
+    if with_cache:
+        close(g_[7], r_[7], dtype, "pages")
+        assert (g_[7] != 0).sum() == (r_[7] != 0).sum(), "only the tokens' slots are written"

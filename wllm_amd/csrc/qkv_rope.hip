@@ -1,0 +1,159 @@
+// The query/key/value projection of a decode step, its bias, the rotation of queries and keys and
+// the write of keys and values into their pages, in one kernel: for at most 16 tokens, bfloat16,
+// heads whose size is a multiple of 32 and that are rotated whole.
+//
+// out[m, :] = x[m, :] . w^T as in `gemm_skinny.hip` (weights as the A operand of
+// v_mfma_f32_16x16x32_bf16, read row by row or from the tile-major copy).  A workgroup owns two
+// bands of 16 columns of one head that the rotation pairs: columns 16p .. 16p+15 and the same
+// HD/2 further on.  Its eight wavefronts split the K axis, issue all their loads before the first
+// product (a register is refilled as soon as its product is issued), and add their sums through
+// shared memory in the order of the pieces.  The first wavefront then holds, per lane, four
+// columns of both bands for one token: element j of the head and its partner j + HD/2, so the
+// pair is turned in registers by position * inv_freq[j] (angle, sine, cosine in float32), written
+// to the row of queries, keys and values, and keys go to the cache as [page_size, HD], values
+// transposed as [HD, page_size].  Heads of values take the same path without the rotation.
+#include "common.h"
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+union QFrag {
+    uint4 u;
+    bf16x8_t v;
+};
+
+constexpr int kQkvWaves = 8;
+constexpr int kQkvInFlight = 8;     // steps of 32 keys whose loads a wavefront keeps in flight, per band
+
+template <bool TILED>
+__global__ void __launch_bounds__(kQkvWaves * 64)
+qkv_rope_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const float* __restrict__ bias,
+                const int* __restrict__ positions, const float* __restrict__ inv_freq, const int* __restrict__ slots,
+                bf16* __restrict__ qkv, bf16* __restrict__ cache, int M, int K, int num_heads, int num_kv_heads, int HD,
+                int page_size, long long num_pages) {
+    __shared__ float4_t red[(kQkvWaves - 1) * kWave * 2];
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int i = lane % 16, g = lane / 16;
+    const int pairs = HD / 32;                          // pairs of bands in a head
+    const int head = blockIdx.x / pairs, p = blockIdx.x % pairs;
+    const int band_lo = head * (HD / 16) + p, band_hi = band_lo + pairs;
+    const int steps = K / 32;
+    const int per = (steps + kQkvWaves - 1) / kQkvWaves;
+    const int s0 = wave * per, s1 = min(steps, s0 + per);
+    constexpr int kStep = TILED ? 512 : 32;             // elements from one step of 32 keys to the next
+    const bf16* lo = TILED ? w + static_cast<size_t>(band_lo) * steps * 512 + lane * 8
+                           : w + (static_cast<size_t>(band_lo) * 16 + i) * K + 8 * g;
+    const bf16* hi = TILED ? w + static_cast<size_t>(band_hi) * steps * 512 + lane * 8
+                           : w + (static_cast<size_t>(band_hi) * 16 + i) * K + 8 * g;
+    const bf16* xp = x + static_cast<size_t>(min(i, M - 1)) * K + 8 * g;
+    const bool x_row = i < M;
+    const uint4 zero = make_uint4(0, 0, 0, 0);
+    constexpr int U = kQkvInFlight;
+    QFrag cl[U], ch[U], cx[U];
+    auto load_step = [&](int u, int at) {
+        const bool ok = at < s1;
+        cl[u].u = ok ? *reinterpret_cast<const uint4*>(lo + static_cast<size_t>(at) * kStep) : zero;
+        ch[u].u = ok ? *reinterpret_cast<const uint4*>(hi + static_cast<size_t>(at) * kStep) : zero;
+        cx[u].u = ok && x_row ? *reinterpret_cast<const uint4*>(xp + static_cast<size_t>(at) * 32) : zero;
+    };
+#pragma unroll
+    for (int u = 0; u < U; ++u) load_step(u, s0 + u);
+    float4_t acc_lo = float4_t{0.f, 0.f, 0.f, 0.f}, acc_hi = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int s = s0; s < s1; s += U) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            acc_lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cl[u].v, cx[u].v, acc_lo, 0, 0, 0);
+            acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ch[u].v, cx[u].v, acc_hi, 0, 0, 0);
+            load_step(u, s + U + u);
+        }
+    }
+    if (wave > 0) {
+        red[((wave - 1) * kWave + lane) * 2] = acc_lo;
+        red[((wave - 1) * kWave + lane) * 2 + 1] = acc_hi;
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int q = 0; q < kQkvWaves - 1; ++q) {
+        acc_lo += red[(q * kWave + lane) * 2];
+        acc_hi += red[(q * kWave + lane) * 2 + 1];
+    }
+    // lane (i, g): token m = i, elements j .. j + 3 of the head and their partners
+    const int m = i;
+    if (m >= M) return;
+    const int j0 = p * 16 + 4 * g, half = HD / 2;
+    const int width = (num_heads + 2 * num_kv_heads) * HD;
+    const int col = head * HD + j0;
+    if (bias) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            acc_lo[v] += bias[col + v];
+            acc_hi[v] += bias[col + half + v];
+        }
+    }
+    const bool rotated = head < num_heads + num_kv_heads;
+    if (rotated && inv_freq) {
+        const float pos = static_cast<float>(positions[m]);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            float s, c;
+            sincosf(pos * inv_freq[j0 + v], &s, &c);
+            const float a = acc_lo[v], b = acc_hi[v];
+            acc_lo[v] = a * c - b * s;
+            acc_hi[v] = b * c + a * s;
+        }
+    }
+    uint2 plo, phi;
+    plo.x = pack2_bf16(acc_lo[0], acc_lo[1]);
+    plo.y = pack2_bf16(acc_lo[2], acc_lo[3]);
+    phi.x = pack2_bf16(acc_hi[0], acc_hi[1]);
+    phi.y = pack2_bf16(acc_hi[2], acc_hi[3]);
+    bf16* row = qkv + static_cast<size_t>(m) * width + col;
+    *reinterpret_cast<uint2*>(row) = plo;
+    *reinterpret_cast<uint2*>(row + half) = phi;
+    if (!cache || head < num_heads) return;
+    const int slot = slots[m];
+    const long long page = slot / page_size;
+    const int off = slot % page_size;
+    if (slot < 0 || page >= num_pages) return;
+    const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * HD;
+    bf16* kpage = cache + page * page_elems;
+    if (head < num_heads + num_kv_heads) {
+        bf16* dst = kpage + (static_cast<size_t>(head - num_heads) * page_size + off) * HD + j0;
+        *reinterpret_cast<uint2*>(dst) = plo;
+        *reinterpret_cast<uint2*>(dst + half) = phi;
+    } else {
+        bf16* vpage = kpage + static_cast<size_t>(num_kv_heads) * page_size * HD;
+        const int vh = head - num_heads - num_kv_heads;
+        const uint16_t el[4] = {static_cast<uint16_t>(plo.x & 0xffff), static_cast<uint16_t>(plo.x >> 16),
+                                static_cast<uint16_t>(plo.y & 0xffff), static_cast<uint16_t>(plo.y >> 16)};
+        const uint16_t eh[4] = {static_cast<uint16_t>(phi.x & 0xffff), static_cast<uint16_t>(phi.x >> 16),
+                                static_cast<uint16_t>(phi.y & 0xffff), static_cast<uint16_t>(phi.y >> 16)};
+        uint16_t* vp = reinterpret_cast<uint16_t*>(vpage);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            vp[(static_cast<size_t>(vh) * HD + j0 + v) * page_size + off] = el[v];
+            vp[(static_cast<size_t>(vh) * HD + j0 + half + v) * page_size + off] = eh[v];
+        }
+    }
+}
+
+// Returns 0, a HIP error code, or -1 for sizes this kernel does not take (the caller then runs the
+// product and the rotation as two kernels).  `w` is the stacked [q; k; v] weight, row by row or
+// (`tiled`) its tile-major copy.  inv_freq has HD/2 entries or is null (no rotation).
+WLLM_API int wllm_qkv_rope(const void* x, const void* w, int tiled, const float* bias, const int* positions,
+                           const float* inv_freq, const int* slots, void* qkv, void* cache, long long num_pages, int M,
+                           int K, int num_heads, int num_kv_heads, int head_dim, int page_size, hipStream_t stream) {
+    if (M < 1 || M > 16 || K < 32 || K % 32 != 0 || head_dim < 32 || head_dim % 32 != 0 || num_heads < 1 || num_kv_heads < 1 ||
+        page_size < 1)
+        return -1;
+    const int grid = (num_heads + 2 * num_kv_heads) * (head_dim / 32);
+#define LAUNCH(T)                                                                                                      \
+    qkv_rope_kernel<T><<<grid, kQkvWaves * 64, 0, stream>>>(                                                           \
+        static_cast<const bf16*>(x), static_cast<const bf16*>(w), bias, positions, inv_freq, slots, static_cast<bf16*>(qkv), \
+        static_cast<bf16*>(cache), M, K, num_heads, num_kv_heads, head_dim, page_size, num_pages)
+    if (tiled) LAUNCH(true);
+    else LAUNCH(false);
+#undef LAUNCH
+    return launch_status();
+}

@@ -22,6 +22,8 @@ def _ptr(t):
 
 
 _SIGNATURES = {
+    "wllm_qkv_rope": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong,
+                      c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_feed_tokens": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "wllm_embed_lookup": [c_void_p, c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
     "wllm_rms_norm": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
@@ -108,6 +110,22 @@ class HipBackend:
             _ptr(inv_freq), _ptr(slots),
             _ptr(cache), cache.shape[0] if cache is not None else 0, qkv.shape[0], num_heads, num_kv_heads, head_dim,
             rotary_dim, page_size, self._stream()), "rope_and_cache_write")
+
+    @staticmethod
+    def qkv_rope_takes(rows: int, dtype, in_features: int, head_dim: int, rotary_dim: int) -> bool:
+        """The fused projection, rotation and cache write: bfloat16, at most 16 tokens, heads of a
+        multiple of 32 that are rotated whole."""
+        return (dtype == torch.bfloat16 and 1 <= rows <= 16 and in_features % 32 == 0 and head_dim % 32 == 0
+                and rotary_dim == head_dim)
+
+    def qkv_rope(self, x, weight, tiles, qkv, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads,
+                 head_dim, page_size):
+        self._on_gpu(x, weight, tiles, qkv, bias, positions, inv_freq, slots, cache)
+        w, tiled = (tiles, 1) if tiles is not None else (weight, 0)
+        self._check(self.lib.wllm_qkv_rope(
+            _ptr(x), _ptr(w), tiled, _ptr(bias), _ptr(positions), _ptr(inv_freq), _ptr(slots), _ptr(qkv), _ptr(cache),
+            cache.shape[0] if cache is not None else 0, x.shape[0], x.shape[1], num_heads, num_kv_heads, head_dim,
+            page_size, self._stream()), "qkv_rope")
 
     @staticmethod
     def mfma_attention_takes(dtype, head_dim: int, page_size: int) -> bool:

@@ -157,6 +157,49 @@ def rope_and_cache_write(qkv: torch.Tensor, bias: Optional[torch.Tensor], positi
                                        head_dim, rotary_dim, page_size, parts)
 
 
+def qkv_rope_takes(rows: int, dtype: torch.dtype, in_features: int, head_dim: int, rotary_dim: int) -> bool:
+    """Whether `qkv_rope` has a kernel for these sizes (else the caller runs `linear` and
+    `rope_and_cache_write`)."""
+    return bool(backend().qkv_rope_takes(rows, dtype, in_features, head_dim, rotary_dim))
+
+
+def qkv_rope(x: torch.Tensor, weight: torch.Tensor, qkv: torch.Tensor, bias: Optional[torch.Tensor],
+             positions: torch.Tensor, inv_freq: Optional[torch.Tensor], slots: Optional[torch.Tensor],
+             cache: Optional[torch.Tensor], *, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int,
+             tiles: Optional[torch.Tensor] = None) -> None:
+    """qkv = x @ weight^T, then everything `rope_and_cache_write` does, in one kernel: the
+    projection of a decode step never leaves the registers between the product and the rotation.
+    x T [n, k]; weight T [(num_heads + 2*num_kv_heads) * head_dim, k], the stacked query, key and
+    value matrices (`tiles`: its tile-major copy); the other operands as in `rope_and_cache_write`,
+    with inv_freq of head_dim/2 entries or None.  Only for sizes that `qkv_rope_takes`."""
+    width = (num_heads + 2 * num_kv_heads) * head_dim
+    _dense(x, "x", _ACT)
+    _need(x.dim() == 2, "x: expected [rows, in]")
+    n = x.shape[0]
+    _dense(weight, "weight", x.dtype, (width, x.shape[1]))
+    _check_tiles(tiles, weight, 1)
+    _dense(qkv, "qkv", x.dtype, (n, width))
+    rotary_dim = 0
+    if inv_freq is not None:
+        _dense(inv_freq, "inv_freq", torch.float32)
+        _need(inv_freq.dim() == 1, "inv_freq: expected one axis")
+        rotary_dim = 2 * inv_freq.shape[0]
+    _need(qkv_rope_takes(n, x.dtype, x.shape[1], head_dim, rotary_dim or head_dim),
+          "qkv_rope: no kernel for these sizes; run linear and rope_and_cache_write")
+    if bias is not None:
+        _dense(bias, "bias", torch.float32, (width,))
+    _dense(positions, "positions", torch.int32, (n,))
+    _need((slots is None) == (cache is None), "slots and cache go together")
+    if cache is not None:
+        _dense(slots, "slots", torch.int32, (n,))
+        _dense(cache, "cache", x.dtype)
+        _need(cache.dim() == 4 and tuple(cache.shape[1:]) == (2, num_kv_heads, page_size * head_dim),
+              f"cache: shape {tuple(cache.shape)}, expected [pages, 2, {num_kv_heads}, {page_size * head_dim}]")
+    if n:
+        backend().qkv_rope(x, weight, tiles, qkv, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads,
+                           head_dim, page_size)
+
+
 def paged_attention(qkv: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor,
                     token_segment: torch.Tensor, seg_q_start: torch.Tensor, seg_q_len: torch.Tensor,
                     seg_ctx_len: torch.Tensor, out: torch.Tensor, *, num_heads: int, num_kv_heads: int,

@@ -79,15 +79,22 @@ class PagedAttention:
         s = self.spec
         n = h.shape[0]
         qkv = ctx.buffer("qkv", (n, self.qkv_width), h.dtype)
-        # where the product kernel splits its sums, the rotation kernel adds them as it reads
-        projected = project(ctx, "qkv", h, self.w_qkv, qkv, tiles=self.t_qkv)
-        parts = projected if projected.dim() == 3 else None
         pages = ctx.pages(entry)
-        ops.rope_and_cache_write(
-            qkv, self.b_qkv, ctx.positions, self.position.inv_freq,
-            pages.slots if pages.writes else None, pages.storage if pages.writes else None,
-            num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim, page_size=pages.page_size,
-            parts=parts)
+        slots, storage = (pages.slots, pages.storage) if pages.writes else (None, None)
+        rotary_dim = 2 * self.position.inv_freq.shape[0] if self.position.inv_freq is not None else s.head_dim
+        if ops.qkv_rope_takes(n, h.dtype, h.shape[1], s.head_dim, rotary_dim):
+            # a decode step: projection, rotation and cache write in one kernel
+            ops.qkv_rope(h, self.w_qkv, qkv, self.b_qkv, ctx.positions, self.position.inv_freq, slots, storage,
+                         num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim,
+                         page_size=pages.page_size, tiles=self.t_qkv)
+        else:
+            # where the product kernel splits its sums, the rotation kernel adds them as it reads
+            projected = project(ctx, "qkv", h, self.w_qkv, qkv, tiles=self.t_qkv)
+            parts = projected if projected.dim() == 3 else None
+            ops.rope_and_cache_write(
+                qkv, self.b_qkv, ctx.positions, self.position.inv_freq, slots, storage,
+                num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim, page_size=pages.page_size,
+                parts=parts)
         attn = ctx.buffer("attn", (n, s.num_heads * s.head_dim), h.dtype)
         ops.paged_attention(
             qkv, pages.storage, pages.block_tables, ctx.token_segment, ctx.seg_q_start, ctx.seg_q_len,
