@@ -292,7 +292,9 @@ def test_looking_ahead_gives_every_request_the_same_tokens(tiny, admission, page
         first = [Request(**spec) for spec in specs]
         for r in first:
             plain_run.add_request(r)
-        plain_run.run_to_completion()
+        done = plain_run.run_to_completion()
+        assert sorted(r.request_id for r in done) == list(range(len(specs))), "each request is handed back once, complete"
+        assert all(r.is_complete() for r in done)
         s = make(model, num_pages=pages, page_size=4, max_requests=4, max_prefill_tokens_per_step=10,
                  admission=admission, lookahead=lookahead)
         reqs = []

@@ -40,6 +40,7 @@ class Request:
     num_preemptions: int = 0
     arrival_index: int = 0
     seed: int = 0
+    num_unread: int = 0             # outputs that were sampled on the device and have not been read yet
 
     @property
     def num_prompt_tokens(self) -> int:
@@ -63,6 +64,10 @@ class Request:
     def is_finished(self) -> bool:
         return self.status == RequestStatus.FINISHED
 
+    def is_complete(self) -> bool:
+        """Finished, and every output has its value."""
+        return self.status == RequestStatus.FINISHED and self.num_unread == 0
+
     def append_token(self, token: int, logprob: Optional[float]) -> None:
         """sequence.py:53-59."""
         self.output_token_ids.append(int(token))
@@ -81,6 +86,7 @@ class Request:
         index among the outputs.  Only the length rule can be applied before the value is known."""
         self.output_token_ids.append(0)
         self.logprobs.append(None)
+        self.num_unread += 1
         if len(self.output_token_ids) >= self.max_new_tokens:
             self.status, self.finish_reason = RequestStatus.FINISHED, "length"
         return len(self.output_token_ids) - 1

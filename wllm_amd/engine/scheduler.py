@@ -109,8 +109,9 @@ class Scheduler:
         """Running: give back its pages; waiting: drop it; unknown: nothing (scheduler.py:158-176)."""
         if self._started is not None:
             for row, r in enumerate(self._started.sampled):
-                if r.request_id == request_id:
+                if r.request_id == request_id and row not in self._started.dropped:
                     self._started.dropped.add(row)
+                    r.num_unread -= 1
                     del r.output_token_ids[self._started.places[row]:], r.logprobs[self._started.places[row]:]
         for i, r in enumerate(self.running):
             if r.request_id == request_id:
@@ -274,6 +275,7 @@ class Scheduler:
             if row in step.dropped:
                 continue
             place = step.places[row]
+            r.num_unread -= 1
             r.output_token_ids[place] = int(tokens[row])
             r.logprobs[place] = logprobs[row] if logprobs is not None else None
             got.append(r)
@@ -287,8 +289,9 @@ class Scheduler:
                 ahead = self._started
                 if ahead is not None:
                     for row2, r2 in enumerate(ahead.sampled):
-                        if r2 is r:
+                        if r2 is r and row2 not in ahead.dropped:
                             ahead.dropped.add(row2)
+                            r.num_unread -= 1
                 del r.output_token_ids[place + 1:], r.logprobs[place + 1:]
                 if r in self.running:
                     self.running.remove(r)
@@ -302,5 +305,5 @@ class Scheduler:
         for _ in range(max_steps):
             if not self.has_unfinished_requests():
                 break
-            finished.extend(r for r in self.step() if r.is_finished())
+            finished.extend(r for r in self.step() if r.is_complete())
         return finished
