@@ -48,6 +48,19 @@ qkv_rope_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const fl
     const bf16* xp = x + static_cast<size_t>(min(i, M - 1)) * K + 8 * g;
     const bool x_row = i < M;
     const uint4 zero = make_uint4(0, 0, 0, 0);
+    // what the first wavefront needs after the sums, asked for now so that it has arrived by then
+    const int j0 = p * 16 + 4 * g, half = HD / 2;
+    const bool rotated = head < num_heads + num_kv_heads && inv_freq != nullptr;
+    float pos = 0.f;
+    float4 freq = make_float4(0.f, 0.f, 0.f, 0.f);
+    int slot = -1;
+    if (wave == 0 && x_row) {
+        if (rotated) {
+            pos = static_cast<float>(positions[i]);
+            freq = *reinterpret_cast<const float4*>(inv_freq + j0);
+        }
+        if (cache && head >= num_heads) slot = slots[i];
+    }
     constexpr int U = kQkvInFlight;
     QFrag cl[U], ch[U], cx[U];
     auto load_step = [&](int u, int at) {
@@ -81,7 +94,6 @@ qkv_rope_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const fl
     // lane (i, g): token m = i, elements j .. j + 3 of the head and their partners
     const int m = i;
     if (m >= M) return;
-    const int j0 = p * 16 + 4 * g, half = HD / 2;
     const int width = (num_heads + 2 * num_kv_heads) * HD;
     const int col = head * HD + j0;
     if (bias) {
@@ -91,13 +103,12 @@ qkv_rope_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const fl
             acc_hi[v] += bias[col + half + v];
         }
     }
-    const bool rotated = head < num_heads + num_kv_heads;
-    if (rotated && inv_freq) {
-        const float pos = static_cast<float>(positions[m]);
+    if (rotated) {
+        const float fr[4] = {freq.x, freq.y, freq.z, freq.w};
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             float s, c;
-            sincosf(pos * inv_freq[j0 + v], &s, &c);
+            sincosf(pos * fr[v], &s, &c);
             const float a = acc_lo[v], b = acc_hi[v];
             acc_lo[v] = a * c - b * s;
             acc_hi[v] = b * c + a * s;
@@ -112,7 +123,6 @@ qkv_rope_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const fl
     *reinterpret_cast<uint2*>(row) = plo;
     *reinterpret_cast<uint2*>(row + half) = phi;
     if (!cache || head < num_heads) return;
-    const int slot = slots[m];
     const long long page = slot / page_size;
     const int off = slot % page_size;
     if (slot < 0 || page >= num_pages) return;
