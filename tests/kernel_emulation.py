@@ -56,6 +56,17 @@ class EmulatedKernels:
         out.copy_(y.to(out.dtype))
 
     fused_qkv = True        # whether the emulation offers the fused projection and rotation
+    fused_residual = True   # and the product that adds into the residual stream
+
+    def linear_residual_takes(self, rows, dtype, out_features, in_features):
+        return self.fused_residual and rows <= 16 and out_features % 16 == 0
+
+    def linear_residual(self, x, weight, tiles, residual, sumsq):
+        self._count("linear_residual")
+        self._same_numbers(weight, tiles, 1)
+        new = residual.to(self.acc) + x.to(self.acc) @ weight.to(self.acc).T
+        residual.copy_(new.to(torch.float32))
+        sumsq.copy_((residual.to(self.acc) ** 2).view(residual.shape[0], -1, 16).sum(-1).to(torch.float32))
 
     def qkv_rope_takes(self, rows, dtype, in_features, head_dim, rotary_dim):
         return self.fused_qkv and rotary_dim == head_dim and rows <= 16
@@ -175,6 +186,22 @@ class EmulatedKernels:
                 out[p].copy_((x[:, a:b].to(self.acc) @ weight[:, a:b].to(self.acc).T).to(out.dtype))
             return
         out.copy_((x.to(self.acc) @ weight.to(self.acc).T).to(out.dtype))
+
+    fused_norm = True       # and the gated product with the norm on load
+
+    def gated_linear_norm_takes(self, rows, dtype, in_features):
+        return self.fused_norm and rows <= 16
+
+    def gated_linear_norm(self, x, weight, out, activation, tiles=None):
+        self._count("gated_linear_norm")
+        self._same_numbers(weight, tiles, 2)
+        r = x.residual.to(self.acc)
+        # the mean square comes from the sums the producer left, not from the residual itself
+        inv = torch.rsqrt(x.sumsq.to(self.acc).sum(-1, keepdim=True) / r.shape[1] + x.eps)
+        h = (r * inv * (x.offset + x.weight.to(self.acc))).to(x.dtype)
+        gu = (h.to(self.acc) @ weight.to(self.acc).T)
+        self.gated_activation(gu, out, activation)
+        self.calls["gated_activation"] -= 1
 
     def gated_linear(self, x, weight, out, activation, scratch, tiles=None):
         self._count("gated_linear")

@@ -448,3 +448,56 @@ def test_qkv_projection_rotation_and_cache_write_in_one_kernel(tiled, m, k, nh, 
     if with_cache:
         close(g_[7], r_[7], dtype, "pages")
         assert (g_[7] != 0).sum() == (r_[7] != 0).sum(), "only the tokens' slots are written"
+
+
+@pytest.mark.parametrize("tiled", [False, True])
+@pytest.mark.parametrize("m,n,k", [(8, 2048, 2048), (8, 3072, 4096), (16, 96, 64), (1, 48, 4064), (5, 3072, 1056), (13, 16, 32)])
+def test_product_into_the_residual_stream_with_sums_of_squares(tiled, m, n, k):
+    dtype = torch.bfloat16
+    assert ops.linear_residual_takes(m, dtype, n, k)
+    assert not ops.linear_residual_takes(m, dtype, n, 16384), "a long K axis is left to the split product"
+    assert not ops.linear_residual_takes(17, dtype, n, k) and not ops.linear_residual_takes(m, dtype, n + 8, k)
+
+    def make():
+        g = torch.Generator(device="cpu").manual_seed(31)
+        x = torch.randn(m, k, generator=g).to(dtype).to(DEV)
+        w = (torch.randn(n, k, generator=g) / math.sqrt(k)).to(dtype).to(DEV)
+        residual = torch.randn(m, n, generator=g).to(DEV)
+        sumsq = torch.full((m, n // 16), -1.0, device=DEV)
+        return [x, w, residual, sumsq], {"tiles": ops.tile_weight(w) if tiled else None}
+
+    g_, r_ = both("linear_residual", make, dtype)
+    close(g_[2], r_[2], torch.float32, "residual")
+    assert torch.allclose(g_[3].double(), (g_[2].double() ** 2).view(m, -1, 16).sum(-1), rtol=1e-5), "sums of squares of what was written"
+
+
+@pytest.mark.parametrize("tiled", [False, True])
+@pytest.mark.parametrize("act", ["gelu_tanh", "silu"])
+@pytest.mark.parametrize("m,inter,k,offset", [(8, 16384, 2048, 1.0), (16, 250, 512, 0.0), (1, 777, 1024, 1.0), (11, 64, 3072, 1.0)])
+def test_gated_product_with_the_norm_on_load(tiled, act, m, inter, k, offset):
+    """The gated product reading the float32 residual stream and normalising it on the way, against
+    rms_norm followed by the gated product."""
+    dtype = torch.bfloat16
+    assert ops.gated_linear_norm_takes(m, dtype, k)
+    assert not ops.gated_linear_norm_takes(17, dtype, k) and not ops.gated_linear_norm_takes(m, dtype, k + 64)
+    g = torch.Generator(device="cpu").manual_seed(41)
+    residual = (torch.randn(m, k, generator=g) * 3).to(DEV)
+    norm_w = (torch.randn(k, generator=g) * 0.2).to(DEV)
+    w = (torch.randn(2 * inter, k, generator=g) / math.sqrt(k)).to(dtype).to(DEV)
+    # the producer's sums: here per band of 16 columns, as `linear_residual` leaves them
+    sumsq = (residual.double() ** 2).view(m, -1, 16).sum(-1).float()
+    x = ops.NormOnLoad(residual, sumsq, norm_w, 1e-6, offset, dtype)
+    tiles = ops.tile_weight(w, 2) if tiled else None
+    out = torch.zeros(m, inter, dtype=dtype, device=DEV)
+    ops.gated_linear(x, w, out, act, None, tiles)
+    torch.cuda.synchronize()
+    # the two kernels it replaces
+    h = torch.zeros(m, k, dtype=dtype, device=DEV)
+    ops.rms_norm(residual.clone(), norm_w, 1e-6, offset, h)
+    two = torch.zeros(m, inter, dtype=dtype, device=DEV)
+    ops.gated_linear(h, w, two, act, torch.zeros(m, 2 * inter, dtype=dtype, device=DEV), tiles)
+    close(out, two, dtype, "against norm then product on the GPU")
+    ref = torch.zeros(m, inter, dtype=dtype, device=DEV)
+    with ops.use_backend(EmulatedKernels(precise=True)):
+        ops.gated_linear(x, w, ref, act, None, tiles)
+    close(out, ref, dtype, "against the emulation")

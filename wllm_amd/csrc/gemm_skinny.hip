@@ -269,11 +269,28 @@ __device__ __forceinline__ float act_silu(float z) { return z / (1.f + expf(-z))
 // halves are added through shared memory in a fixed order before the activation.  With few rows of
 // x (MT <= 2) the kernel needs few registers, a workgroup is 2 tiles (4 wavefronts), and four
 // workgroups share a compute unit: 16 wavefronts with 16 loads each in flight.
-template <int MT, int ACT, bool TILED, int TPW>
-__global__ void __launch_bounds__(TPW * 128, MT == 1 ? 4 : (MT == 2 ? 3 : 2))
-gemm_skinny_gated_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, bf16* __restrict__ out, int M,
-                         int inter, int K, int chunk) {
+//
+// NORM (at most 16 rows, chunks of 256 keys): x is not given; the kernel reads the float32 residual
+// stream and applies the RMS norm as it stages a chunk: x = residual * rsqrt(mean square + eps) *
+// (offset + norm weight), rounded to bfloat16 as the norm kernel would round it.  A row's mean square
+// comes from `sumsq` ([M, sumsq_cols], whose row sums are the rows' sums of squares: see
+// `gemm_residual.hip`), so no kernel has to pass over the stream between the product that wrote it
+// and this one.  XR is the number of 16-byte pieces of x a thread stages per chunk (rows beyond M are
+// not staged: they only feed results that are not written).
+struct NormOnLoad {
+    const float* residual;      // [M, K]
+    const float* sumsq;         // [M, sumsq_cols]
+    const float* weight;        // [K]
+    int sumsq_cols;
+    float eps, offset;
+};
+
+template <int MT, int ACT, bool TILED, int TPW, bool NORM, int XR>
+__global__ void __launch_bounds__(TPW * 128, MT == 1 ? (NORM && XR > 2 ? 3 : 4) : (MT == 2 ? 3 : 2))
+gemm_skinny_gated_kernel(const bf16* __restrict__ x, NormOnLoad norm, const bf16* __restrict__ w, bf16* __restrict__ out,
+                         int M, int inter, int K, int chunk) {
     extern __shared__ uint4 xs[];                 // two halves of [MT*16][chunk/8 + 1]
+    __shared__ float inv_s[16];                   // NORM: a row's rsqrt(mean square + eps)
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const int i = lane % 16, g = lane / 16;
     const int tile = wave % TPW, half = wave / TPW;
@@ -313,13 +330,45 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
     int step = 0;
     constexpr int kHalfThreads = TPW * 64;        // the threads that stage one half's x
     const int tid_half = threadIdx.x % kHalfThreads;
+    if (NORM) {
+        // 16 threads a row add the row of `sumsq` in a fixed order
+        const int t = threadIdx.x;
+        if (t < 256) {
+            const int r = t / 16, part = t % 16;
+            float total = 0.f;
+            if (r < M)
+                for (int b = part; b < norm.sumsq_cols; b += 16) total += norm.sumsq[static_cast<size_t>(r) * norm.sumsq_cols + b];
+            total += __shfl_xor(total, 8, kWave);
+            total += __shfl_xor(total, 4, kWave);
+            total += __shfl_xor(total, 2, kWave);
+            total += __shfl_xor(total, 1, kWave);
+            if (part == 0) inv_s[r] = rsqrtf(total / static_cast<float>(K) + norm.eps);
+        }
+    }
     // x is staged chunk by chunk (per half of K); the next chunk's loads are in flight during the products
-    constexpr int kXRegs = MT == 1 ? 4 : 8;       // MT*16*chunk/8 <= kHalfThreads * kXRegs pieces
-    uint4 xreg[kXRegs];
+    constexpr int kXRegs = NORM ? XR : (MT == 1 ? 4 : 8);       // pieces of a chunk per thread
+    uint4 xreg[NORM ? 1 : kXRegs];
+    float4 xraw[NORM ? kXRegs : 1][2], wraw[2];
     auto fetch_x = [&](int kc) {
+        if (NORM) {
+            // chunks of 256 keys: a thread's pieces are rows tid_half / 32 + (kHalfThreads / 32) * u at the
+            // same 8 keys, so it needs 8 norm weights a chunk
+            const int c = tid_half % 32;
+            const float* wsrc = norm.weight + k_begin + kc + c * 8;
+            wraw[0] = *reinterpret_cast<const float4*>(wsrc);
+            wraw[1] = *reinterpret_cast<const float4*>(wsrc + 4);
+#pragma unroll
+            for (int u = 0; u < kXRegs; ++u) {
+                const int m = tid_half / 32 + (kHalfThreads / 32) * u;
+                const float* src = norm.residual + static_cast<size_t>(min(m, M - 1)) * K + k_begin + kc + c * 8;
+                xraw[u][0] = *reinterpret_cast<const float4*>(src);
+                xraw[u][1] = *reinterpret_cast<const float4*>(src + 4);
+            }
+            return;
+        }
         const int vecs = min(chunk, half_k - kc) / 8;
 #pragma unroll
-        for (int u = 0; u < kXRegs; ++u) {
+        for (int u = 0; u < (NORM ? 1 : kXRegs); ++u) {
             const int idx = tid_half + u * kHalfThreads;
             const int m = idx / vecs, c = idx % vecs;
             xreg[u] = (idx < MT * 16 * vecs && m < M)
@@ -327,16 +376,35 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
                           : make_uint4(0, 0, 0, 0);
         }
     };
-    fetch_x(0);
-    for (int kc = 0; kc < half_k; kc += chunk) {
-        const int len = min(chunk, half_k - kc);      // a multiple of 32 * kBatch, except the last
-        const int vecs = len / 8;
-        __syncthreads();
+    auto stage_x = [&](int vecs) {
+        if (NORM) {
+            const int c = tid_half % 32;
 #pragma unroll
-        for (int u = 0; u < kXRegs; ++u) {
+            for (int u = 0; u < kXRegs; ++u) {
+                const int m = tid_half / 32 + (kHalfThreads / 32) * u;
+                if (m >= 16) continue;
+                const float inv = inv_s[m];
+                const float4 a = xraw[u][0], b = xraw[u][1];
+                uint4 v;
+                v.x = pack2_bf16(a.x * inv * (norm.offset + wraw[0].x), a.y * inv * (norm.offset + wraw[0].y));
+                v.y = pack2_bf16(a.z * inv * (norm.offset + wraw[0].z), a.w * inv * (norm.offset + wraw[0].w));
+                v.z = pack2_bf16(b.x * inv * (norm.offset + wraw[1].x), b.y * inv * (norm.offset + wraw[1].y));
+                v.w = pack2_bf16(b.z * inv * (norm.offset + wraw[1].z), b.w * inv * (norm.offset + wraw[1].w));
+                xh[m * stride + c] = v;
+            }
+            return;
+        }
+#pragma unroll
+        for (int u = 0; u < (NORM ? 1 : kXRegs); ++u) {
             const int idx = tid_half + u * kHalfThreads;
             if (idx < MT * 16 * vecs) xh[(idx / vecs) * stride + idx % vecs] = xreg[u];
         }
+    };
+    fetch_x(0);
+    for (int kc = 0; kc < half_k; kc += chunk) {
+        const int len = min(chunk, half_k - kc);      // a multiple of 32 * kBatch, except the last
+        __syncthreads();
+        stage_x(len / 8);
         __syncthreads();
         if (kc + chunk < half_k) fetch_x(kc + chunk);
         for (int k = 0; k < len; k += 32 * kBatch) {
@@ -392,11 +460,13 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
     }
 }
 
-WLLM_API int wllm_gemm_skinny_gated(const void* x, const void* w, int tiled, void* out, int M, int inter, int K,
-                                    int activation, int chunk, hipStream_t stream) {
+static int gated_launch(const void* x, NormOnLoad norm, bool with_norm, const void* w, int tiled, void* out, int M,
+                        int inter, int K, int activation, int chunk, hipStream_t stream) {
     if (M < 1 || M > 64 || K % 64 != 0 || chunk % 32 != 0 || activation < 0 || activation > 1) return -1;
     const int mt = (M + 15) / 16;
     if (chunk > K / 2) chunk = K / 2;
+    // the norm on load: at most 16 rows, whole chunks of 256 keys
+    if (with_norm && (mt != 1 || chunk != 256 || (K / 2) % 256 != 0)) return -1;
     const int tpw = mt <= 2 ? 2 : 4;                 // tiles of 16 gate rows per workgroup
     size_t smem = static_cast<size_t>(2) * mt * 16 * (chunk / 8 + 1) * sizeof(uint4);
     const size_t red = static_cast<size_t>(tpw) * kWave * mt * 8 * sizeof(float);
@@ -407,21 +477,30 @@ WLLM_API int wllm_gemm_skinny_gated(const void* x, const void* w, int tiled, voi
     if (smem > 160 * 1024 - 4096 || mt * 16 * (chunk / 8) > tpw * 64 * x_regs || (chunk % 256 != 0 && chunk < K / 2))
         return -1;
     const dim3 grid((inter + 16 * tpw - 1) / (16 * tpw));
-#define LAUNCH_T(MT, A, T, TPW)                                                                                       \
+#define LAUNCH_K(MT, A, T, TPW, NORM, XR)                                                                            \
     do {                                                                                                              \
         static bool roomy = false;     /* more than 64 KiB of shared memory must be asked for once */                \
         if (smem > 65536 && !roomy) {                                                                                 \
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_gated_kernel<MT, A, T, TPW>),          \
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_gated_kernel<MT, A, T, TPW, NORM, XR>), \
                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 4096) != hipSuccess)    \
                 return launch_status();                                                                               \
             roomy = true;                                                                                             \
         }                                                                                                             \
-        gemm_skinny_gated_kernel<MT, A, T, TPW><<<grid, TPW * 128, smem, stream>>>(                                  \
-            static_cast<const bf16*>(x), static_cast<const bf16*>(w), static_cast<bf16*>(out), M, inter, K, chunk);   \
+        gemm_skinny_gated_kernel<MT, A, T, TPW, NORM, XR><<<grid, TPW * 128, smem, stream>>>(                        \
+            static_cast<const bf16*>(x), norm, static_cast<const bf16*>(w), static_cast<bf16*>(out), M, inter, K, chunk); \
     } while (0)
+#define LAUNCH_T(MT, A, T, TPW) LAUNCH_K(MT, A, T, TPW, false, 4)
 #define LAUNCH(MT, A)                                        \
     if (tiled) LAUNCH_T(MT, A, true, (MT <= 2 ? 2 : 4));      \
     else LAUNCH_T(MT, A, false, (MT <= 2 ? 2 : 4))
+#define LAUNCH_N(A)                                           \
+    if (tiled) {                                              \
+        if (M <= 8) LAUNCH_K(1, A, true, 2, true, 2);         \
+        else LAUNCH_K(1, A, true, 2, true, 4);                \
+    } else {                                                  \
+        if (M <= 8) LAUNCH_K(1, A, false, 2, true, 2);        \
+        else LAUNCH_K(1, A, false, 2, true, 4);               \
+    }
 #define BY_MT(A)                     \
     switch (mt) {                    \
         case 1: LAUNCH(1, A); break; \
@@ -429,9 +508,32 @@ WLLM_API int wllm_gemm_skinny_gated(const void* x, const void* w, int tiled, voi
         case 3: LAUNCH(3, A); break; \
         default: LAUNCH(4, A); break; \
     }
-    if (activation == 0) { BY_MT(0) } else { BY_MT(1) }
+    if (with_norm) {
+        if (activation == 0) { LAUNCH_N(0) } else { LAUNCH_N(1) }
+    } else {
+        if (activation == 0) { BY_MT(0) } else { BY_MT(1) }
+    }
 #undef BY_MT
+#undef LAUNCH_N
 #undef LAUNCH
 #undef LAUNCH_T
+#undef LAUNCH_K
     return launch_status();
+}
+
+WLLM_API int wllm_gemm_skinny_gated(const void* x, const void* w, int tiled, void* out, int M, int inter, int K,
+                                    int activation, int chunk, hipStream_t stream) {
+    return gated_launch(x, NormOnLoad{nullptr, nullptr, nullptr, 0, 0.f, 0.f}, false, w, tiled, out, M, inter, K, activation,
+                        chunk, stream);
+}
+
+// The same product with the RMS norm of the residual stream folded into the load of x: at most 16
+// rows, K a multiple of 512.  sumsq float32 [M, sumsq_cols]: a row's entries add up to the sum of
+// squares of the row of `residual`.  Returns -1 for sizes it does not take.
+WLLM_API int wllm_gemm_skinny_gated_norm(const float* residual, const float* sumsq, int sumsq_cols, const float* norm_weight,
+                                         float eps, float offset, const void* w, int tiled, void* out, int M, int inter,
+                                         int K, int activation, hipStream_t stream) {
+    if (M > 16 || sumsq_cols < 1) return -1;
+    return gated_launch(nullptr, NormOnLoad{residual, sumsq, norm_weight, sumsq_cols, eps, offset}, true, w, tiled, out, M,
+                        inter, K, activation, 256, stream);
 }

@@ -47,7 +47,6 @@ qkv_rope_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const fl
                            : w + (static_cast<size_t>(band_hi) * 16 + i) * K + 8 * g;
     const bf16* xp = x + static_cast<size_t>(min(i, M - 1)) * K + 8 * g;
     const bool x_row = i < M;
-    const uint4 zero = make_uint4(0, 0, 0, 0);
     // what the first wavefront needs after the sums, asked for now so that it has arrived by then
     const int j0 = p * 16 + 4 * g, half = HD / 2;
     const bool rotated = head < num_heads + num_kv_heads && inv_freq != nullptr;
@@ -65,9 +64,9 @@ qkv_rope_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const fl
     QFrag cl[U], ch[U], cx[U];
     auto load_step = [&](int u, int at) {
         const bool ok = at < s1;
-        cl[u].u = ok ? *reinterpret_cast<const uint4*>(lo + static_cast<size_t>(at) * kStep) : zero;
-        ch[u].u = ok ? *reinterpret_cast<const uint4*>(hi + static_cast<size_t>(at) * kStep) : zero;
-        cx[u].u = ok && x_row ? *reinterpret_cast<const uint4*>(xp + static_cast<size_t>(at) * 32) : zero;
+        cl[u].u = ok ? *reinterpret_cast<const uint4*>(lo + static_cast<size_t>(at) * kStep) : make_uint4(0, 0, 0, 0);
+        ch[u].u = ok ? *reinterpret_cast<const uint4*>(hi + static_cast<size_t>(at) * kStep) : make_uint4(0, 0, 0, 0);
+        cx[u].u = ok && x_row ? *reinterpret_cast<const uint4*>(xp + static_cast<size_t>(at) * 32) : make_uint4(0, 0, 0, 0);
     };
 #pragma unroll
     for (int u = 0; u < U; ++u) load_step(u, s0 + u);

@@ -22,6 +22,7 @@ def _ptr(t):
 
 
 _SIGNATURES = {
+    "wllm_gemm_residual": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "wllm_qkv_rope": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong,
                       c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_feed_tokens": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
@@ -31,6 +32,8 @@ _SIGNATURES = {
     "wllm_rope_cache_write": [c_void_p, c_int, c_void_p, c_int, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p,
                               c_void_p, c_longlong, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_gemm_skinny_gated": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "wllm_gemm_skinny_gated_norm": [c_void_p, c_void_p, c_int, c_void_p, c_float, c_float, c_void_p, c_int, c_void_p, c_int,
+                                    c_int, c_int, c_int, c_void_p],
     "wllm_tile_weight": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "wllm_gated_activation": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_paged_attention_generic": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -110,6 +113,20 @@ class HipBackend:
             _ptr(inv_freq), _ptr(slots),
             _ptr(cache), cache.shape[0] if cache is not None else 0, qkv.shape[0], num_heads, num_kv_heads, head_dim,
             rotary_dim, page_size, self._stream()), "rope_and_cache_write")
+
+    @staticmethod
+    def linear_residual_takes(rows: int, dtype, out_features: int, in_features: int) -> bool:
+        """The product that adds into the residual stream: bfloat16, at most 16 rows, whole bands of
+        16 columns.  Its workgroups are the bands; with a long K axis there are too few of them for the
+        weight to stream from all compute units, and the split product with its norm kernel is faster."""
+        return (dtype == torch.bfloat16 and 1 <= rows <= 16 and out_features % 16 == 0 and in_features % 32 == 0
+                and in_features <= 4096)
+
+    def linear_residual(self, x, weight, tiles, residual, sumsq):
+        self._on_gpu(x, weight, tiles, residual, sumsq)
+        w, tiled = (tiles, 1) if tiles is not None else (weight, 0)
+        self._check(self.lib.wllm_gemm_residual(_ptr(x), _ptr(w), tiled, _ptr(residual), _ptr(sumsq), x.shape[0],
+                                                weight.shape[0], x.shape[1], self._stream()), "linear_residual")
 
     @staticmethod
     def qkv_rope_takes(rows: int, dtype, in_features: int, head_dim: int, rotary_dim: int) -> bool:
@@ -283,6 +300,20 @@ class HipBackend:
             return
         self.linear(x, weight, scratch)
         self.gated_activation(scratch, out, activation)
+
+    @staticmethod
+    def gated_linear_norm_takes(rows: int, dtype, in_features: int) -> bool:
+        """The gated product with the norm folded into its load of x: bfloat16, at most 16 rows,
+        input size a multiple of 512 (whole chunks of 256 keys per half of the K axis)."""
+        return dtype == torch.bfloat16 and 1 <= rows <= 16 and in_features % 512 == 0
+
+    def gated_linear_norm(self, x, weight, out, activation, tiles=None):
+        self._on_gpu(x.residual, x.sumsq, x.weight, weight, out, tiles)
+        w, tiled = (tiles, 1) if tiles is not None else (weight, 0)
+        self._check(self.lib.wllm_gemm_skinny_gated_norm(
+            _ptr(x.residual), _ptr(x.sumsq), x.sumsq.shape[1], _ptr(x.weight), x.eps, x.offset, _ptr(w), tiled,
+            _ptr(out), x.shape[0], out.shape[1], x.shape[1], 0 if activation == "gelu_tanh" else 1, self._stream()),
+            "gated_linear (norm on load)")
 
     def gated_activation(self, gate_up, out, activation):
         self._on_gpu(gate_up, out)

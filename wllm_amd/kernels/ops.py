@@ -157,6 +157,32 @@ def rope_and_cache_write(qkv: torch.Tensor, bias: Optional[torch.Tensor], positi
                                        head_dim, rotary_dim, page_size, parts)
 
 
+def linear_residual_takes(rows: int, dtype: torch.dtype, out_features: int, in_features: int) -> bool:
+    """Whether `linear_residual` has a kernel for these sizes."""
+    return bool(backend().linear_residual_takes(rows, dtype, out_features, in_features))
+
+
+def linear_residual(x: torch.Tensor, weight: torch.Tensor, residual: torch.Tensor, sumsq: torch.Tensor,
+                    tiles: Optional[torch.Tensor] = None) -> None:
+    """residual += x @ weight^T in float32, and sumsq[m, b] = the sum of squares of the new
+    residual[m, 16b : 16b + 16].  x T [m, k]; weight T [n, k] (`tiles`: its tile-major copy);
+    residual float32 [m, n]; sumsq float32 [m, n / 16].  A row's mean square is then the sum of
+    its row of `sumsq` over n: what a norm needs, without a pass over the residual.  Only for sizes
+    that `linear_residual_takes`."""
+    _dense(x, "x", _ACT)
+    _need(x.dim() == 2, "x: expected [rows, in]")
+    m, k = x.shape
+    _dense(weight, "weight", x.dtype)
+    _need(weight.dim() == 2 and weight.shape[1] == k, f"weight: shape {tuple(weight.shape)}, expected [out, {k}]")
+    n = weight.shape[0]
+    _check_tiles(tiles, weight, 1)
+    _need(linear_residual_takes(m, x.dtype, n, k), "linear_residual: no kernel for these sizes")
+    _dense(residual, "residual", torch.float32, (m, n))
+    _dense(sumsq, "sumsq", torch.float32, (m, n // 16))
+    if m:
+        backend().linear_residual(x, weight, tiles, residual, sumsq)
+
+
 def qkv_rope_takes(rows: int, dtype: torch.dtype, in_features: int, head_dim: int, rotary_dim: int) -> bool:
     """Whether `qkv_rope` has a kernel for these sizes (else the caller runs `linear` and
     `rope_and_cache_write`)."""
@@ -323,12 +349,51 @@ def gated_activation(gate_up: torch.Tensor, out: torch.Tensor, activation: str) 
         backend().gated_activation(gate_up, out, activation)
 
 
-def gated_linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, activation: str,
-                 scratch: torch.Tensor, tiles: Optional[torch.Tensor] = None) -> None:
+class NormOnLoad:
+    """The input of a product as something the product kernel computes while it reads it:
+    rms_norm(residual) with the rows' sums of squares already known.  residual float32 [m, k];
+    sumsq float32 [m, c] whose rows add up to the rows' sums of squares (`linear_residual` leaves
+    it); weight float32 [k]; the result is what `rms_norm(residual, weight, eps, offset)` gives in
+    dtype T."""
+
+    def __init__(self, residual: torch.Tensor, sumsq: torch.Tensor, weight: torch.Tensor, eps: float, offset: float,
+                 dtype: torch.dtype):
+        _dense(residual, "residual", torch.float32)
+        _need(residual.dim() == 2, "residual: expected [rows, hidden]")
+        _dense(sumsq, "sumsq", torch.float32)
+        _need(sumsq.dim() == 2 and sumsq.shape[0] == residual.shape[0] and sumsq.shape[1] >= 1,
+              "sumsq: expected [rows, columns]")
+        _dense(weight, "weight", torch.float32, (residual.shape[1],))
+        self.residual, self.sumsq, self.weight = residual, sumsq, weight
+        self.eps, self.offset, self.dtype = float(eps), float(offset), dtype
+
+    @property
+    def shape(self):
+        return self.residual.shape
+
+
+def gated_linear_norm_takes(rows: int, dtype: torch.dtype, in_features: int) -> bool:
+    """Whether `gated_linear` can take its input as a `NormOnLoad` at these sizes."""
+    return bool(backend().gated_linear_norm_takes(rows, dtype, in_features))
+
+
+def gated_linear(x, weight: torch.Tensor, out: torch.Tensor, activation: str,
+                 scratch: Optional[torch.Tensor], tiles: Optional[torch.Tensor] = None) -> None:
     """out = act(x @ Wg^T) * (x @ Wu^T) with weight = [Wg; Wu] stacked, T [2I, k]; x T [m, k];
     out T [m, I]; scratch T [m, 2I] may be used for the unfused product.  `tiles` is
-    `tile_weight(weight, halves=2)`."""
+    `tile_weight(weight, halves=2)`.  x may be a `NormOnLoad` where `gated_linear_norm_takes` says so:
+    the norm is then applied as the kernel reads the residual stream (scratch is not used)."""
     _need(activation in ACTIVATIONS, f"activation {activation!r}: expected one of {ACTIVATIONS}")
+    if isinstance(x, NormOnLoad):
+        _need(gated_linear_norm_takes(x.shape[0], x.dtype, x.shape[1]), "gated_linear: no kernel with the norm on load for these sizes")
+        _dense(weight, "weight", x.dtype)
+        _need(weight.dim() == 2 and weight.shape[1] == x.shape[1] and weight.shape[0] % 2 == 0,
+              f"weight: shape {tuple(weight.shape)}, expected [2*intermediate, {x.shape[1]}]")
+        _dense(out, "out", x.dtype, (x.shape[0], weight.shape[0] // 2))
+        _check_tiles(tiles, weight, 2)
+        if x.shape[0]:
+            backend().gated_linear_norm(x, weight, out, activation, tiles)
+        return
     _dense(x, "x", _ACT)
     _need(x.dim() == 2, "x: expected [rows, in]")
     _dense(weight, "weight", x.dtype)

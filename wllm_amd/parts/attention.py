@@ -17,7 +17,7 @@ import torch
 
 from wllm_amd.cache.manager import CacheNeed
 from wllm_amd.kernels import ops
-from wllm_amd.parts.common import load_matrix, project
+from wllm_amd.parts.common import Product, load_matrix, project
 from wllm_amd.parts.registry import build_position, register_mixer
 from wllm_amd.parts.specs import AttentionSpec
 from wllm_amd.weights.checkpoint import ExpectedTensor
@@ -103,5 +103,5 @@ class PagedAttention:
             max_q_len=ctx.max_q_len, max_ctx_len=ctx.max_ctx_len,
             plan=ctx.attention_plan(num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim,
                                     page_size=pages.page_size, window=s.window or 0))
-        # the next norm adds the contribution to the residual stream, partial sums and all
-        return project(ctx, "mixer_out", attn, self.w_o, tiles=self.t_o)
+        # the stream adds the output projection: at once, or through the next norm, partial sums and all
+        return Product("mixer_out", attn, self.w_o, self.t_o)

@@ -26,6 +26,19 @@ def project(ctx, name: str, x: torch.Tensor, weight: torch.Tensor, out: Optional
     return out
 
 
+class Product:
+    """A part's contribution to the residual stream that is still a product to be made:
+    x @ weight^T.  The stream it is added to chooses how: into the stream at once by a kernel that
+    also leaves what the next norm needs (`ops.linear_residual`), or as a tensor (or a stack of
+    partial sums) that the next norm kernel adds."""
+
+    def __init__(self, name: str, x: torch.Tensor, weight: torch.Tensor, tiles: Optional[torch.Tensor] = None):
+        self.name, self.x, self.weight, self.tiles = name, x, weight, tiles
+
+    def make(self, ctx) -> torch.Tensor:
+        return project(ctx, self.name, self.x, self.weight, tiles=self.tiles)
+
+
 def load_matrix(fetch, matrix: torch.Tensor, halves: int = 1):
     """A weight matrix on the device as the product kernels want it: (the matrix, row by row, for
     products of many rows; its tile-major copy for the few rows of a decode step, or None).  The

@@ -7,7 +7,7 @@ from __future__ import annotations
 import torch
 
 from wllm_amd.kernels import ops
-from wllm_amd.parts.common import load_matrix, project
+from wllm_amd.parts.common import Product, load_matrix
 from wllm_amd.parts.registry import register_feed_forward
 from wllm_amd.parts.specs import GatedMLPSpec
 from wllm_amd.weights.checkpoint import ExpectedTensor
@@ -36,10 +36,17 @@ class GatedMLP:
             fetch, torch.cat([fetch.matrix(s.gate_weight), fetch.matrix(s.up_weight)], dim=0), halves=2)
         self.w_down, self.t_down = load_matrix(fetch, fetch.matrix(s.down_weight))
 
-    def forward(self, ctx, h: torch.Tensor) -> torch.Tensor:
+    def takes_norm_on_load(self, rows: int, dtype: torch.dtype) -> bool:
+        """Whether `forward` may be given `ops.NormOnLoad` instead of the normalised tensor."""
+        return ops.gated_linear_norm_takes(rows, dtype, self.spec.hidden_size)
+
+    def forward(self, ctx, h):
         s = self.spec
         n = h.shape[0]
-        gate_up = ctx.buffer("gate_up", (n, 2 * s.intermediate_size), h.dtype)
         act = ctx.buffer("ffn_act", (n, s.intermediate_size), h.dtype)
-        ops.gated_linear(h, self.w_gate_up, act, s.activation, gate_up, self.t_gate_up)
-        return project(ctx, "ffn_out", act, self.w_down, tiles=self.t_down)
+        if isinstance(h, ops.NormOnLoad):
+            ops.gated_linear(h, self.w_gate_up, act, s.activation, None, self.t_gate_up)
+        else:
+            gate_up = ctx.buffer("gate_up", (n, 2 * s.intermediate_size), h.dtype)
+            ops.gated_linear(h, self.w_gate_up, act, s.activation, gate_up, self.t_gate_up)
+        return Product("ffn_out", act, self.w_down, self.t_down)

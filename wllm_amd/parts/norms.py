@@ -28,3 +28,7 @@ class RMSNorm:
     def forward(self, x: torch.Tensor, out: torch.Tensor, delta=None, rows=None) -> torch.Tensor:
         ops.rms_norm(x, self.weight, self.spec.eps, self.spec.weight_offset, out, delta=delta, rows=rows)
         return out
+
+    def on_load(self, residual: torch.Tensor, sumsq: torch.Tensor, dtype: torch.dtype):
+        """This norm of `residual` as a recipe for a kernel that applies it while it reads."""
+        return ops.NormOnLoad(residual, sumsq, self.weight, self.spec.eps, self.spec.weight_offset, dtype)

@@ -13,7 +13,11 @@ block         built from a BlockSpec and the parts above; forward(ctx, entry, st
 
 `ctx` is the step's `StepContext`, `entry` the index of the schedule entry being
 run, `h` the normalised input [tokens, hidden] in the activation dtype, `y` the
-part's contribution to the residual stream, same shape and dtype.
+part's contribution to the residual stream: a tensor of the same shape and dtype, a
+float32 stack of partial sums [S, tokens, hidden], or a `common.Product` (a last
+product x @ W^T that the stream makes itself).  A part that defines
+`takes_norm_on_load(rows, dtype) -> bool` may be given `ops.NormOnLoad` as `h` when it
+says yes: the recipe of the norm, for a kernel that applies it while it reads.
 """
 from __future__ import annotations
 
