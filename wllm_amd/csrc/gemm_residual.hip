@@ -87,7 +87,7 @@ WLLM_API int wllm_gemm_residual(const void* x, const void* w, int tiled, float* 
     gemm_residual_kernel<W, T><<<bands, W * 64, 0, stream>>>(static_cast<const bf16*>(x), static_cast<const bf16*>(w), \
                                                              residual, sumsq, M, N, K)
     // sixteen wavefronts a band where the K axis is long, so that enough of them stream at once
-    if (K > 4096) {
+    if (K > 2048) {
         if (tiled) LAUNCH(16, true);
         else LAUNCH(16, false);
     } else {
