@@ -1,6 +1,6 @@
 """Command line.  Options carry the reference's names and meanings where it has them
 (src/wllm/cli.py:21-56): --model, --device, --dtype, --num-blocks, --block-size,
---chunked-prefill-tokens; --cuda-graphs is --hip-graphs here.  The reference's command
+--chunked-prefill-tokens, --cuda-graphs (also spelled --hip-graphs here).  The reference's command
 starts a server; this engine is token ids in, token ids out, so the commands are
 
     python -m wllm_amd.cli generate --model DIR --prompt-ids 5,17,3 [--prompt-ids ...]
@@ -38,7 +38,9 @@ def _engine_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--num-blocks", type=int, default=256, help="KV cache blocks (block_size tokens each)")
     ap.add_argument("--block-size", type=int, default=16)
-    ap.add_argument("--hip-graphs", action="store_true", help="replay captured HIP graphs for decode steps")
+    # the reference's name for the option (src/wllm/cli.py:21-56) and this engine's
+    ap.add_argument("--cuda-graphs", "--hip-graphs", dest="hip_graphs", action="store_true",
+                    help="replay captured HIP graphs for decode steps")
     ap.add_argument("--chunked-prefill-tokens", type=int, default=None,
                     help="max prompt tokens processed per scheduler step (enables chunked prefill)")
 
