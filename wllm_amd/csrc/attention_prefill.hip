@@ -1,8 +1,10 @@
 // Paged attention for long segments (prompt portions) on the matrix cores, bfloat16: the keys
 // and values of a block of 32 keys are staged through shared memory once per workgroup and read
-// by all four wavefronts; a wavefront owns 32 query rows (two tiles of 16), so every fragment it
-// reads from shared memory feeds two products.  A workgroup is 128 rows of one (segment, key/value
-// head): rows are (token, query head of the group) pairs, row r = token * G + head.
+// by all four wavefronts; a wavefront owns one tile of 16 query rows.  A workgroup is 64 rows of one
+// (segment, key/value head): rows are (token, query head of the group) pairs, row r = token * G +
+// head.  (With two tiles a wavefront, every fragment read from shared memory would feed two
+// products, but the registers of 128 rows leave room for one workgroup a compute unit; with 64
+// rows two workgroups share it and hide each other's waits, which measured a quarter faster.)
 //
 // The products are those of `attention_mfma.hip` (v_mfma_f32_16x16x32_bf16, scores transposed so
 // that a lane's values all belong to one query row, probabilities fed to the second product from
@@ -42,7 +44,7 @@ struct PrefillSmem {
 // block of rows write, per tile of 16 rows, an unnormalised accumulator and (maximum, sum) into
 // slot `partial slot + tile`, which `attention_reduce_kernel` combines.
 template <int HD, int RTW>      // RTW: tiles of 16 rows per wavefront (1 or 2)
-__global__ void __launch_bounds__(kPrefillThreads)
+__global__ void __launch_bounds__(kPrefillThreads, RTW == 1 ? 2 : 1)
 paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restrict__ cache,
                                const int* __restrict__ block_tables, const int* __restrict__ items,
                                const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
@@ -322,7 +324,7 @@ WLLM_API int wllm_paged_attention_prefill(const void* qkv, const void* cache, co
                                           int window, hipStream_t stream) {
     if (head_dim % 32 != 0 || head_dim < 32 || head_dim > 256 || page_size % 4 != 0 || num_heads % num_kv_heads != 0)
         return -1;
-    if (rows_per_item != 64 && rows_per_item != 128) return -1;
+    if (rows_per_item != 64) return -1;
     if (num_items <= 0) return 0;
     const float scale_log2e = scale * 1.4426950408889634f;
 #define LAUNCH_RTW(HD, RTW)                                                                                         \
@@ -330,9 +332,7 @@ WLLM_API int wllm_paged_attention_prefill(const void* qkv, const void* cache, co
         static_cast<const bf16*>(qkv), static_cast<const bf16*>(cache), block_tables, items, seg_q_start, seg_q_len, \
         seg_ctx_len, static_cast<bf16*>(out), partial_o, partial_ml, num_heads, num_kv_heads, page_size, max_pages, \
         scale_log2e, window)
-#define LAUNCH(HD)                            \
-    if (rows_per_item == 64) LAUNCH_RTW(HD, 1); \
-    else LAUNCH_RTW(HD, 2)
+#define LAUNCH(HD) LAUNCH_RTW(HD, 1)
     switch (head_dim) {
         case 32: LAUNCH(32); break;
         case 64: LAUNCH(64); break;

@@ -5,13 +5,13 @@ head of the group): rows = q_len * group.  A segment of at most 16 rows (a decod
 tile of rows whose keys are split over workgroups in fixed chunks of `KEY_CHUNK` keys, the
 partial results combined by a second kernel; chunk boundaries are multiples of the chunk size
 counted from key 0, so they depend on the key index only.  Longer segments are cut into
-workgroups of up to four tiles of 16 rows that each walk all their keys.
+workgroups of four tiles of 16 rows (prefill items).
 
 A work item is 8 int32: segment, key/value head, first row, 1 (reserved), first key,
 end key, partial slot (-1: the workgroup writes the final result), unused.  A partial slot holds
 one tile of 16 rows.  A reduce item is 8 int32: segment, key/value head, first partial slot, number
 of splits, first row of the tile, slots between two splits, 2 unused.  A prefill item (long
-segments, 64 or 128 rows each, for the kernel that stages keys and values through shared memory) is
+segments, 64 rows each, for the kernel that stages keys and values through shared memory) is
 8 int32: segment, key/value head, first row, first key, end key, partial slot (-1: final), 2
 unused.  The keys of a block of rows are split over several prefill items when the step has too
 few blocks to fill the compute units (a portion of a prompt late in a long context) or when they
@@ -31,9 +31,9 @@ ROWS_PER_TILE = 16
 ITEM_INTS = 8
 PREFILL_TABLE_PAGES = 1024      # pages one prefill item may span (the kernel's shared block table)
 PREFILL_TARGET_ITEMS = 1024     # prefill items wanted in a step: about four for each compute unit
-PREFILL_MIN_CHUNK = 256         # keys; smaller pieces cost more in partial results than they gain
-PREFILL_WIDE_SPAN = 131072      # keys walked by all blocks of 128 rows together from which on a workgroup
-                                # takes 128 rows (more reuse of staged keys) instead of 64 (more workgroups)
+PREFILL_MIN_CHUNK = 512         # keys; smaller pieces cost more in partial results than they gain
+PREFILL_ROWS = 64               # rows of a prefill item: with 64 two workgroups share a compute unit (128 rows
+                                # reuse the staged keys more, but fill the register file with one workgroup)
 
 
 @dataclass
@@ -146,21 +146,19 @@ def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_
     # ---- long segments: workgroups of 64 or 128 rows of one key/value head ----
     prefill = []
     long_idx = np.nonzero(~short)[0]
-    prefill_rows = 64
+    prefill_rows = PREFILL_ROWS
     if long_idx.size:
-        for prefill_rows in (128, 64):
-            blocks = []              # (segment, first rows, lowest key, end key) per long segment
-            span_total = 0
-            for s in long_idx:
-                n_blocks = -(-int(rows[s]) // prefill_rows)
-                rb = np.arange(n_blocks, dtype=np.int64) * prefill_rows
-                first_pos = int(ctx_len[s] - q_len[s])
-                hi = first_pos + np.minimum(rows[s] - 1, rb + prefill_rows - 1) // group + 1
-                lo = np.maximum(0, first_pos + rb // group - window + 1) if window > 0 else np.zeros_like(rb)
-                blocks.append((int(s), rb, lo, hi))
-                span_total += int((hi - lo).sum()) * num_kv_heads
-            if span_total >= PREFILL_WIDE_SPAN:
-                break
+        prefill_rows = PREFILL_ROWS
+        blocks = []              # (segment, first rows, lowest key, end key) per long segment
+        span_total = 0
+        for s in long_idx:
+            n_blocks = -(-int(rows[s]) // prefill_rows)
+            rb = np.arange(n_blocks, dtype=np.int64) * prefill_rows
+            first_pos = int(ctx_len[s] - q_len[s])
+            hi = first_pos + np.minimum(rows[s] - 1, rb + prefill_rows - 1) // group + 1
+            lo = np.maximum(0, first_pos + rb // group - window + 1) if window > 0 else np.zeros_like(rb)
+            blocks.append((int(s), rb, lo, hi))
+            span_total += int((hi - lo).sum()) * num_kv_heads
         tiles = prefill_rows // ROWS_PER_TILE
         # a piece that starts inside a page touches up to two pages more than its keys fill
         max_chunk = max(KEY_CHUNK, (PREFILL_TABLE_PAGES - 2) * page_size // KEY_CHUNK * KEY_CHUNK)
