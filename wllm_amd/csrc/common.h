@@ -73,5 +73,12 @@ __device__ __forceinline__ float stack_sum(const float* __restrict__ p, int spli
     return total;
 }
 
+// One rotated pair (a, b) -> (a cos - b sin, b cos + a sin).  The products are fused in one fixed
+// way, so that every kernel that rotates gives the same bits for the same numbers.
+__device__ __forceinline__ void rotate_pair(float a, float b, float s, float c, float& ra, float& rb) {
+    ra = __fmaf_rn(a, c, -(b * s));
+    rb = __fmaf_rn(b, c, a * s);
+}
+
 // The error a launch left, as an int for the caller (0 = hipSuccess).
 __host__ inline int launch_status() { return static_cast<int>(hipGetLastError()); }

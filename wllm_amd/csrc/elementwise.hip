@@ -113,9 +113,81 @@ __global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ de
     }
 }
 
+// The same with 16-byte accesses, for a width that is a multiple of 4 and fits the registers: a
+// thread keeps up to kNormGroups groups of 4 consecutive elements.
+constexpr int kNormGroups = 2;
+
+template <typename T> struct alignas(4 * sizeof(T)) Quad { T v[4]; };
+
+template <typename TD, typename TO>
+__global__ void rms_norm_vec_kernel(float* __restrict__ x, const TD* __restrict__ delta, int splits,
+                                    size_t split_stride, const float* __restrict__ weight,
+                                    const int* __restrict__ rows, TO* __restrict__ out, int hidden, float eps,
+                                    float offset) {
+    __shared__ float scratch[16];
+    const int orow = blockIdx.x;
+    const int irow = rows ? rows[orow] : orow;
+    float* xr = x + static_cast<size_t>(irow) * hidden;
+    const TD* dr = delta ? delta + static_cast<size_t>(irow) * hidden : nullptr;
+    TO* o = out + static_cast<size_t>(orow) * hidden;
+    Quad<float> keep[kNormGroups];
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < kNormGroups; ++e) {
+        const int i = (threadIdx.x + e * blockDim.x) * 4;
+        Quad<float> v = {{0.f, 0.f, 0.f, 0.f}};
+        if (i < hidden) {
+            v = *reinterpret_cast<const Quad<float>*>(xr + i);
+            if (dr) {
+                // the partial sums of a stack are added in stack order, then their sum to x
+                const int stack = (sizeof(TD) == sizeof(float) && splits > 1) ? splits : 1;
+                Quad<float> d;
+                for (int sp = 0; sp < stack; ++sp) {
+                    const Quad<TD> q = *reinterpret_cast<const Quad<TD>*>(dr + sp * split_stride + i);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) d.v[k] = sp == 0 ? to_float(q.v[k]) : d.v[k] + to_float(q.v[k]);
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k) v.v[k] += d.v[k];
+                if (!rows) *reinterpret_cast<Quad<float>*>(xr + i) = v;
+            }
+        }
+        keep[e] = v;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) ss += v.v[k] * v.v[k];
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = rsqrtf(ss / static_cast<float>(hidden) + eps);
+#pragma unroll
+    for (int e = 0; e < kNormGroups; ++e) {
+        const int i = (threadIdx.x + e * blockDim.x) * 4;
+        if (i < hidden) {
+            const Quad<float> w = *reinterpret_cast<const Quad<float>*>(weight + i);
+            Quad<TO> r;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) r.v[k] = from_float<TO>(keep[e].v[k] * inv * (offset + w.v[k]));
+            *reinterpret_cast<Quad<TO>*>(o + i) = r;
+        }
+    }
+}
+
 WLLM_API int wllm_rms_norm(float* x, const void* delta, int delta_bf16, int splits, long long split_stride,
                            const float* weight, const int* rows, void* out, int out_bf16, int num_out_rows,
                            int hidden, float eps, float offset, hipStream_t stream) {
+    if (hidden % 4 == 0 && hidden <= 1024 * 4 * kNormGroups && (splits <= 1 || split_stride % 4 == 0)) {
+        const int quads = hidden / 4;
+        const int vthreads = quads >= 1024 ? 1024 : ((quads + 63) / 64) * 64;
+#define LAUNCH(TD, TO)                                                                                          \
+    rms_norm_vec_kernel<TD, TO><<<num_out_rows, vthreads, 0, stream>>>(                                         \
+        x, static_cast<const TD*>(delta), splits, static_cast<size_t>(split_stride), weight, rows,             \
+        static_cast<TO*>(out), hidden, eps, offset)
+        if (delta_bf16 && out_bf16) LAUNCH(bf16, bf16);
+        else if (delta_bf16) LAUNCH(bf16, float);
+        else if (out_bf16) LAUNCH(float, bf16);
+        else LAUNCH(float, float);
+#undef LAUNCH
+        return launch_status();
+    }
     const int threads = hidden >= 4096 ? 1024 : (hidden >= 1024 ? 512 : (hidden >= 256 ? 128 : 64));
 #define LAUNCH(TD, TO)                                                                                          \
     rms_norm_kernel<TD, TO><<<num_out_rows, threads, 0, stream>>>(x, static_cast<const TD*>(delta), splits,      \
@@ -183,7 +255,9 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, const float* __restrict__
                 a += bias[ia];
                 b += bias[ib];
             }
-            const T ra = from_float<T>(a * c - b * s), rb = from_float<T>(b * c + a * s);
+            float fa, fb;
+            rotate_pair(a, b, s, c, fa, fb);
+            const T ra = from_float<T>(fa), rb = from_float<T>(fb);
             row[ia] = ra;
             row[ib] = rb;
             if (kpage && head >= num_heads) {
@@ -223,11 +297,105 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, const float* __restrict__
     }
 }
 
+// The same for the common case (the row holds the projection itself, no bias, every size a multiple
+// of 16 bytes): a thread moves 16 bytes at a time.  Sines and cosines of the token's angles are
+// computed once into LDS; then each thread takes units of W pairs (W elements at j and W at
+// j + rotary_dim/2 of one head), of W unrotated key elements or of W value elements.
+template <typename T>
+__global__ void rope_cache_vec_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
+                                      const float* __restrict__ inv_freq, const int* __restrict__ slots,
+                                      T* __restrict__ cache, int num_heads, int num_kv_heads, int head_dim,
+                                      int rotary_dim, int page_size, long long num_pages) {
+    constexpr int W = 16 / sizeof(T);
+    struct alignas(16) Vec { T v[W]; };
+    extern __shared__ float sincos_lds[];        // [rotary_dim/2] sines, then as many cosines
+    const int token = blockIdx.x;
+    const int width = (num_heads + 2 * num_kv_heads) * head_dim;
+    T* row = qkv + static_cast<size_t>(token) * width;
+    const int half = rotary_dim / 2;
+    const float pos = static_cast<float>(positions[token]);
+    for (int j = threadIdx.x; j < half; j += blockDim.x) {
+        float s, c;
+        sincosf(pos * inv_freq[j], &s, &c);
+        sincos_lds[j] = s;
+        sincos_lds[half + j] = c;
+    }
+    const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * head_dim;
+    T* kpage = nullptr;
+    T* vpage = nullptr;
+    int off = 0;
+    if (cache) {
+        const int slot = slots[token];
+        const long long page = slot / page_size;
+        off = slot % page_size;
+        if (slot >= 0 && page < num_pages) {
+            kpage = cache + page * page_elems;
+            vpage = kpage + static_cast<size_t>(num_kv_heads) * page_size * head_dim;
+        }
+    }
+    __syncthreads();
+    const int rot_heads = num_heads + num_kv_heads;
+    const int pair_units = half / W, rest_units = (head_dim - rotary_dim) / W, value_units = head_dim / W;
+    const int n_pairs = rot_heads * pair_units;
+    const int n_rest = kpage ? num_kv_heads * rest_units : 0;
+    const int n_values = vpage ? num_kv_heads * value_units : 0;
+    for (int unit = threadIdx.x; unit < n_pairs + n_rest + n_values; unit += blockDim.x) {
+        if (unit < n_pairs) {
+            const int head = unit / pair_units, j = (unit % pair_units) * W;
+            T* pa = row + head * head_dim + j;
+            const Vec a = *reinterpret_cast<const Vec*>(pa), b = *reinterpret_cast<const Vec*>(pa + half);
+            Vec ra, rb;
+#pragma unroll
+            for (int i = 0; i < W; ++i) {
+                const float s = sincos_lds[j + i], c = sincos_lds[half + j + i];
+                const float x = to_float(a.v[i]), y = to_float(b.v[i]);
+                float fa, fb;
+                rotate_pair(x, y, s, c, fa, fb);
+                ra.v[i] = from_float<T>(fa);
+                rb.v[i] = from_float<T>(fb);
+            }
+            *reinterpret_cast<Vec*>(pa) = ra;
+            *reinterpret_cast<Vec*>(pa + half) = rb;
+            if (kpage && head >= num_heads) {
+                T* dst = kpage + (static_cast<size_t>(head - num_heads) * page_size + off) * head_dim + j;
+                *reinterpret_cast<Vec*>(dst) = ra;
+                *reinterpret_cast<Vec*>(dst + half) = rb;
+            }
+        } else if (unit < n_pairs + n_rest) {
+            const int u = unit - n_pairs;
+            const int head = u / rest_units, j = rotary_dim + (u % rest_units) * W;
+            const Vec v = *reinterpret_cast<const Vec*>(row + (num_heads + head) * head_dim + j);
+            *reinterpret_cast<Vec*>(kpage + (static_cast<size_t>(head) * page_size + off) * head_dim + j) = v;
+        } else {
+            const int idx = (unit - n_pairs - n_rest) * W;       // element of the row's value part
+            const Vec v = *reinterpret_cast<const Vec*>(row + rot_heads * head_dim + idx);
+#pragma unroll
+            for (int i = 0; i < W; ++i) vpage[static_cast<size_t>(idx + i) * page_size + off] = v.v[i];
+        }
+    }
+}
+
 WLLM_API int wllm_rope_cache_write(void* qkv, int is_bf16, const float* parts, int splits, long long split_stride,
                                    const float* bias, const int* positions, const float* inv_freq, const int* slots,
                                    void* cache, long long num_pages, int n, int num_heads, int num_kv_heads,
                                    int head_dim, int rotary_dim, int page_size, hipStream_t stream) {
     const int pairs = (num_heads + num_kv_heads) * (rotary_dim / 2);
+    const int w = is_bf16 ? 8 : 4;          // elements in 16 bytes
+    if (!bias && !parts && head_dim % w == 0 && (rotary_dim / 2) % w == 0 && rotary_dim % 2 == 0 &&
+        rotary_dim / 2 <= 4096) {
+        const int units = (pairs + num_kv_heads * (2 * head_dim - rotary_dim)) / w;
+        const int vthreads = units >= 1024 ? 1024 : ((units + 63) / 64) * 64;
+        const size_t lds = static_cast<size_t>(rotary_dim) * sizeof(float);
+        if (is_bf16)
+            rope_cache_vec_kernel<bf16><<<n, vthreads, lds, stream>>>(
+                static_cast<bf16*>(qkv), positions, inv_freq, slots, static_cast<bf16*>(cache), num_heads,
+                num_kv_heads, head_dim, rotary_dim, page_size, num_pages);
+        else
+            rope_cache_vec_kernel<float><<<n, vthreads, lds, stream>>>(
+                static_cast<float*>(qkv), positions, inv_freq, slots, static_cast<float*>(cache), num_heads,
+                num_kv_heads, head_dim, rotary_dim, page_size, num_pages);
+        return launch_status();
+    }
     const int threads = pairs >= 1024 ? 1024 : (pairs >= 512 ? 512 : 256);
     if (is_bf16)
         rope_cache_kernel<bf16><<<n, threads, 0, stream>>>(static_cast<bf16*>(qkv), parts, splits,

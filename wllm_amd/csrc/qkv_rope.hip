@@ -109,8 +109,10 @@ qkv_rope_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const fl
             float s, c;
             sincosf(pos * fr[v], &s, &c);
             const float a = acc_lo[v], b = acc_hi[v];
-            acc_lo[v] = a * c - b * s;
-            acc_hi[v] = b * c + a * s;
+            float ra, rb;
+            rotate_pair(a, b, s, c, ra, rb);
+            acc_lo[v] = ra;
+            acc_hi[v] = rb;
         }
     }
     uint2 plo, phi;
