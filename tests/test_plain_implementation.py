@@ -45,7 +45,7 @@ def test_embedding_is_scaled_by_sqrt_hidden():
     table = torch.randn(10, 64, dtype=torch.float64)
     ids = torch.tensor([3, 3, 9])
     assert torch.equal(P.embed(ids, table, 64), table[ids] * 8.0)           # sqrt(64) exactly
-    # the factor held in bfloat16: sqrt(2048) = 45.2548... becomes 45.25
+    # the factor held in bfloat16: sqrt(2048) = 45.2548... becomes 45.25 (src/wllm/models/gemma.py:158-162)
     t = torch.ones(1, 2048, dtype=torch.float32)
     assert P.embed(torch.tensor([0]), t, 2048, torch.bfloat16)[0, 0].item() == 45.25
     assert abs(P.embed(torch.tensor([0]), t, 2048)[0, 0].item() - math.sqrt(2048)) < 1e-5
