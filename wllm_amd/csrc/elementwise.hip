@@ -141,11 +141,18 @@ __global__ void rms_norm_vec_kernel(float* __restrict__ x, const TD* __restrict_
             if (dr) {
                 // the partial sums of a stack are added in stack order, then their sum to x
                 const int stack = (sizeof(TD) == sizeof(float) && splits > 1) ? splits : 1;
-                Quad<float> d;
-                for (int sp = 0; sp < stack; ++sp) {
-                    const Quad<TD> q = *reinterpret_cast<const Quad<TD>*>(dr + sp * split_stride + i);
+                Quad<float> d = {{0.f, 0.f, 0.f, 0.f}};
+                for (int s0 = 0; s0 < stack; s0 += 8) {
+                    Quad<TD> q[8];       // eight loads in flight
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) d.v[k] = sp == 0 ? to_float(q.v[k]) : d.v[k] + to_float(q.v[k]);
+                    for (int j = 0; j < 8; ++j)
+                        q[j] = *reinterpret_cast<const Quad<TD>*>(dr + min(s0 + j, stack - 1) * split_stride + i);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        if (s0 + j >= stack) break;
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) d.v[k] = s0 + j == 0 ? to_float(q[j].v[k]) : d.v[k] + to_float(q[j].v[k]);
+                    }
                 }
 #pragma unroll
                 for (int k = 0; k < 4; ++k) v.v[k] += d.v[k];
