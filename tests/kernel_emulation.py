@@ -225,7 +225,8 @@ class EmulatedKernels:
         self._count("argmax_rows")
         out.copy_(logits.argmax(dim=-1).to(torch.int32))
 
-    def sample_rows(self, logits, params, seeds, penalty_ids, penalty_offsets, out_tokens, out_logprobs):
+    def sample_rows(self, logits, params, seeds, penalty_ids, penalty_offsets, out_tokens, out_logprobs,
+                    truncations=True):
         from plain.sampling_plain import philox_uniform, sample_row
         self._count("sample_rows")
         for r in range(logits.shape[0]):

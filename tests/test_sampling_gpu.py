@@ -123,3 +123,39 @@ def test_large_vocabulary():
     toks, lps = run(logits, [(0.0,), (1.0, 0, 0.5), (1.0, 50)], [(1, 1)] * 3)
     assert toks[0] == int(logits[0].argmax()) and toks[1] == 255999
     assert toks[2] in torch.topk(logits[2], 50).indices.tolist()
+
+
+@pytest.mark.parametrize("vocab", [777, 5000, 256000])
+def test_a_row_spread_over_workgroups_draws_what_one_workgroup_draws(vocab):
+    """A decode step's few rows are sampled by kernels that cut each row into segments; many rows by
+    one workgroup a row.  All sums that decide anything are integer sums, so the two give the same
+    token and the same log-probability, bit for bit."""
+    torch.manual_seed(vocab + 1)
+    rows = len(CASES) * 3
+    logits = torch.randn(rows, vocab) * 2.5
+    logits[1, vocab - 1] = logits[1].max() + 1.0           # the maximum in the last segment
+    logits[2, :] = logits[2, 0]                            # all equal
+    cases = [CASES[r % len(CASES)] for r in range(rows)]
+    cases[3] = (0.0,)                                      # a greedy row among the others
+    generated = [torch.randint(0, vocab, (9,)).tolist() for _ in range(rows)]
+    seeds = [(99 + r, r * 3) for r in range(rows)]
+    be = ops.backend()
+    limit = be.SAMPLE_SPLIT_ROWS
+    assert rows <= limit
+    split = run(logits, cases, seeds, generated)
+    try:
+        be.SAMPLE_SPLIT_ROWS = 0
+        whole = run(logits, cases, seeds, generated)
+    finally:
+        be.SAMPLE_SPLIT_ROWS = limit
+    assert split[0] == whole[0]
+    assert split[1] == whole[1]
+    # rows without top-k and top-p skip the passes for their thresholds
+    plain = [(0.9,), (1.2, 0, 1.0, 0.02), (0.0,)] * 2
+    a = run(logits[:6], plain, seeds[:6])
+    try:
+        be.SAMPLE_SPLIT_ROWS = 0
+        b = run(logits[:6], plain, seeds[:6])
+    finally:
+        be.SAMPLE_SPLIT_ROWS = limit
+    assert a == b

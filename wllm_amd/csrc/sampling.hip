@@ -1,4 +1,4 @@
-// Sampling kernels: one workgroup per row of float32 logits.
+// Sampling kernels over rows of float32 logits.
 #include "common.h"
 
 // ---- argmax: the largest value of a row, the lowest index among equals -------------------------
@@ -325,6 +325,390 @@ sample_rows_kernel(float* __restrict__ logits, const float* __restrict__ params,
         out_tokens[r] = tok;
         out_logprobs[r] = (row[tok] - row_max) * inv_t - log_z;
     }
+}
+
+// ---- the same sampler with a row spread over many workgroups -------------------------------------
+// One workgroup per row leaves most of the chip idle when a decode step has a few rows of a large
+// vocabulary: a pass over 256,000 logits with an exponential each takes one compute unit about
+// 60 us.  Here a row is cut into kSampleSegments contiguous segments, one workgroup each, and the
+// passes become kernels; what the segments of a row have to agree on goes through a scratch area
+// per row in integer sums, so every number is the one the kernel above computes and the token is
+// the same.  Kernels: prepare (zero the scratch, maximum per segment), histogram level 0 (which
+// also gives the normaliser), levels 1 to 3 (only when a row has top-k or top-p), kept mass per
+// segment, draw.
+constexpr int kSampleSegments = 32;
+constexpr int kSegmentThreads = 256;
+constexpr int kHistWords = 2 * 4 * 256;                  // [counts | mass][level][byte]
+constexpr int kRowWords = kHistWords + kSampleSegments   // kept mass per segment
+                          + kSampleSegments              // maximum per segment: (index << 32) | float bits
+                          + 8;                           // thresholds and normaliser for the draw
+typedef unsigned long long u64;
+
+struct RowSetup {
+    float temperature, top_p, min_p, inv_t, row_max;
+    int top_k, arg_max;
+    bool greedy;
+};
+
+__device__ __forceinline__ int segment_length(int vocab) {
+    return (((vocab + kSampleSegments - 1) / kSampleSegments) + 3) & ~3;
+}
+
+__device__ __forceinline__ RowSetup row_setup(const float* __restrict__ params, const u64* __restrict__ row_ws, int r) {
+    RowSetup rs;
+    rs.temperature = params[r * 5 + 0];
+    rs.top_k = static_cast<int>(params[r * 5 + 1]);
+    rs.top_p = params[r * 5 + 2];
+    rs.min_p = params[r * 5 + 3];
+    rs.greedy = rs.temperature == 0.0f;
+    rs.inv_t = rs.greedy ? 1.0f : 1.0f / fmaxf(rs.temperature, 1e-5f);
+    // the segments' maxima, in index order: the largest value, the lowest index among equals
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    const u64* seg_max = row_ws + kHistWords + kSampleSegments;
+    for (int sgm = 0; sgm < kSampleSegments; ++sgm) {
+        const u64 w = seg_max[sgm];
+        const float v = __uint_as_float(static_cast<uint32_t>(w));
+        const int i = static_cast<int>(w >> 32);
+        if (v > bv || (v == bv && i < bi)) {
+            bv = v;
+            bi = i;
+        }
+    }
+    rs.row_max = bv;
+    rs.arg_max = bi == 0x7fffffff ? 0 : bi;
+    return rs;
+}
+
+__device__ __forceinline__ u64 fixed_mass(float v, float row_max, float inv_t) {
+    return static_cast<u64>(static_cast<double>(expf((v - row_max) * inv_t)) * kFixedOne);
+}
+
+// One level of `radix_descend`, by a wavefront alone: the bin (descending) at which the running
+// total first goes beyond `target` (counts: reaches it), and the total above it.
+template <bool MASS>
+__device__ __forceinline__ bool descend_level(const u64* __restrict__ hist, u64 target, u64& above, int& sel) {
+    const int lane = threadIdx.x % kWave;
+    u64 c[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) c[j] = hist[255 - 4 * lane - j];
+    const u64 mine = c[0] + c[1] + c[2] + c[3];
+    u64 incl = mine;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const u64 o = __shfl_up(incl, off, kWave);
+        if (lane >= off) incl += o;
+    }
+    u64 cum = above + incl - mine;
+    int found = -1;
+    u64 found_above = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const u64 next = cum + c[j];
+        if (found < 0 && (MASS ? next > target : next >= target)) {
+            found = 255 - 4 * lane - j;
+            found_above = cum;
+        }
+        cum = next;
+    }
+    const u64 hits = __ballot(found >= 0);
+    if (hits == 0) return false;
+    const int first = __ffsll(static_cast<long long>(hits)) - 1;
+    sel = __shfl(found, first, kWave);
+    above = __shfl(found_above, first, kWave);
+    return true;
+}
+
+// The prefix of the threshold key after `levels` levels; false when the running total never gets there.
+template <bool MASS>
+__device__ __forceinline__ bool descend(const u64* __restrict__ hist4, int levels, u64 target, uint32_t& prefix,
+                                        uint32_t& mask) {
+    prefix = 0;
+    mask = 0;
+    u64 above = 0;
+    for (int level = 0; level < levels; ++level) {
+        int sel = -1;
+        if (!descend_level<MASS>(hist4 + level * 256, target, above, sel)) return false;
+        const int shift = 24 - 8 * level;
+        prefix |= static_cast<uint32_t>(sel) << shift;
+        mask |= 255u << shift;
+    }
+    return true;
+}
+
+__device__ __forceinline__ u64 wave_sum(u64 v) {
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// The normaliser: every element is in the level-0 histogram of mass.
+__device__ __forceinline__ u64 normaliser(const u64* __restrict__ row_ws) {
+    const int lane = threadIdx.x % kWave;
+    const u64* h = row_ws + 4 * 256;
+    return wave_sum(h[lane] + h[lane + 64] + h[lane + 128] + h[lane + 192]);
+}
+
+__global__ void sample_penalty_kernel(float* __restrict__ logits, const float* __restrict__ params,
+                                      const int* __restrict__ penalty_ids, const int* __restrict__ penalty_offsets,
+                                      int vocab) {
+    const int r = blockIdx.x;
+    const float penalty = params[r * 5 + 4];
+    if (penalty == 1.0f) return;
+    float* row = logits + static_cast<size_t>(r) * vocab;
+    for (int j = penalty_offsets[r] + threadIdx.x; j < penalty_offsets[r + 1]; j += blockDim.x) {
+        const int id = penalty_ids[j];
+        if (id >= 0 && id < vocab) {
+            const float v = row[id];
+            row[id] = v > 0.f ? v / penalty : v * penalty;
+        }
+    }
+}
+
+// Visits the elements of the workgroup's segment, four consecutive ones a thread at a time.
+template <typename F>
+__device__ __forceinline__ void for_segment(const float* __restrict__ row, int vocab, F&& f) {
+    const int len = segment_length(vocab);
+    const int begin = min(vocab, static_cast<int>(blockIdx.x) * len), end = min(vocab, begin + len);
+    const bool vec = vocab % 4 == 0;        // then rows and segments begin at multiples of 16 bytes
+    for (int i = begin + 4 * threadIdx.x; i < end; i += 4 * blockDim.x) {
+        float v[4];
+        if (vec) {
+            const float4 q = *reinterpret_cast<const float4*>(row + i);
+            v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = i + e < end ? row[i + e] : 0.f;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (i + e < end) f(i + e, v[e]);
+    }
+}
+
+__global__ void __launch_bounds__(kSegmentThreads)
+sample_prepare_kernel(const float* __restrict__ logits, u64* __restrict__ ws, int vocab) {
+    __shared__ float red_v[kSegmentThreads / kWave];
+    __shared__ int red_i[kSegmentThreads / kWave];
+    const int r = blockIdx.y, sgm = blockIdx.x, tid = threadIdx.x;
+    u64* row_ws = ws + static_cast<size_t>(r) * kRowWords;
+    for (int j = tid; j < kHistWords / kSampleSegments; j += blockDim.x) row_ws[sgm * (kHistWords / kSampleSegments) + j] = 0ull;
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for_segment(logits + static_cast<size_t>(r) * vocab, vocab, [&](int i, float v) { argmax_take(v, i, bv, bi); });
+    argmax_wave(bv, bi);
+    if (tid % kWave == 0) {
+        red_v[tid / kWave] = bv;
+        red_i[tid / kWave] = bi;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < kSegmentThreads / kWave; ++w)
+            if (red_v[w] > bv || (red_v[w] == bv && red_i[w] < bi)) {
+                bv = red_v[w];
+                bi = red_i[w];
+            }
+        row_ws[kHistWords + kSampleSegments + sgm] = (static_cast<u64>(static_cast<uint32_t>(bi)) << 32) | __float_as_uint(bv);
+    }
+}
+
+// Level `level` of both histograms: counts of keys for top-k, mass for top-p, of the elements whose
+// key has the prefix the levels before chose.  Level 0 of the mass always: it holds the normaliser.
+__global__ void __launch_bounds__(kSegmentThreads)
+sample_histogram_kernel(const float* __restrict__ logits, const float* __restrict__ params, u64* __restrict__ ws,
+                        int vocab, int level) {
+    __shared__ u64 hist[2][256];
+    const int r = blockIdx.y, tid = threadIdx.x;
+    u64* row_ws = ws + static_cast<size_t>(r) * kRowWords;
+    const RowSetup rs = row_setup(params, row_ws, r);
+    bool k_on = !rs.greedy && rs.top_k > 0 && rs.top_k < vocab, p_on = !rs.greedy && rs.top_p < 1.0f;
+    if (level > 0 && !k_on && !p_on) return;
+    uint32_t k_prefix = 0, k_mask = 0, p_prefix = 0, p_mask = 0;
+    if (level > 0) {
+        if (k_on) k_on = descend<false>(row_ws, level, static_cast<u64>(rs.top_k), k_prefix, k_mask);
+        if (p_on) {
+            const u64 z = normaliser(row_ws);
+            const u64 target = static_cast<u64>(static_cast<double>(rs.top_p) * static_cast<double>(z));
+            p_on = descend<true>(row_ws + 4 * 256, level, target, p_prefix, p_mask);
+        }
+        if (!k_on && !p_on) return;
+    }
+    const bool mass_on = level == 0 || p_on;
+    hist[0][tid] = 0ull;
+    hist[1][tid] = 0ull;
+    __syncthreads();
+    const int shift = 24 - 8 * level;
+    for_segment(logits + static_cast<size_t>(r) * vocab, vocab, [&](int, float v) {
+        const uint32_t key = sortable_key(v);
+        const int bin = (key >> shift) & 255u;
+        if (k_on && (key & k_mask) == k_prefix) atomicAdd(&hist[0][bin], 1ull);
+        if (mass_on && (key & p_mask) == p_prefix) atomicAdd(&hist[1][bin], fixed_mass(v, rs.row_max, rs.inv_t));
+    });
+    __syncthreads();
+#pragma unroll
+    for (int kind = 0; kind < 2; ++kind) {
+        const u64 v = hist[kind][tid];
+        if (v) atomicAdd(row_ws + (kind * 4 + level) * 256 + tid, v);
+    }
+}
+
+// The thresholds from the finished histograms, and the mass each segment keeps.
+__global__ void __launch_bounds__(kSegmentThreads)
+sample_kept_kernel(const float* __restrict__ logits, const float* __restrict__ params, u64* __restrict__ ws, int vocab) {
+    __shared__ u64 part_s[kSegmentThreads / kWave];
+    const int r = blockIdx.y, sgm = blockIdx.x, tid = threadIdx.x;
+    u64* row_ws = ws + static_cast<size_t>(r) * kRowWords;
+    const RowSetup rs = row_setup(params, row_ws, r);
+    const u64 z = normaliser(row_ws);
+    u64* out_words = row_ws + kHistWords + 2 * kSampleSegments;
+    if (rs.greedy) {
+        if (sgm == 0 && tid == 0) out_words[2] = z;
+        return;
+    }
+    bool k_on = rs.top_k > 0 && rs.top_k < vocab, p_on = rs.top_p < 1.0f;
+    uint32_t k_key = 0, p_key = 0, mask = 0;
+    if (k_on) k_on = descend<false>(row_ws, 4, static_cast<u64>(rs.top_k), k_key, mask);
+    if (p_on) {
+        const u64 target = static_cast<u64>(static_cast<double>(rs.top_p) * static_cast<double>(z));
+        p_on = descend<true>(row_ws + 4 * 256, 4, target, p_key, mask);
+    }
+    const bool mp_on = rs.min_p > 0.0f;
+    const uint32_t max_key = sortable_key(rs.row_max);
+    u64 mine = 0;
+    for_segment(logits + static_cast<size_t>(r) * vocab, vocab, [&](int, float v) {
+        const uint32_t key = sortable_key(v);
+        const float e = expf((v - rs.row_max) * rs.inv_t);
+        const bool keep = key == max_key || ((!k_on || key >= k_key) && (!p_on || key > p_key) && (!mp_on || e >= rs.min_p));
+        if (keep) mine += static_cast<u64>(static_cast<double>(e) * kFixedOne);
+    });
+    mine = wave_sum(mine);
+    if (tid % kWave == 0) part_s[tid / kWave] = mine;
+    __syncthreads();
+    if (tid == 0) {
+        u64 total = 0;
+        for (int w = 0; w < kSegmentThreads / kWave; ++w) total += part_s[w];
+        row_ws[kHistWords + sgm] = total;
+        if (sgm == 0) {
+            out_words[0] = k_on ? (1ull << 32) | k_key : 0ull;
+            out_words[1] = p_on ? (1ull << 32) | p_key : 0ull;
+            out_words[2] = z;
+        }
+    }
+}
+
+// The draw: the segment that holds the target, then, within it, the thread and the element, all in
+// index order.
+__global__ void __launch_bounds__(kSampleThreads)
+sample_draw_kernel(const float* __restrict__ logits, const float* __restrict__ params, const long long* __restrict__ seeds,
+                   const u64* __restrict__ ws, int* __restrict__ out_tokens, float* __restrict__ out_logprobs, int vocab) {
+    __shared__ u64 scan[kSampleThreads / kWave];
+    __shared__ int found_s;
+    const int r = blockIdx.x, tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    constexpr int kWavesHere = kSampleThreads / kWave;
+    const float* row = logits + static_cast<size_t>(r) * vocab;
+    const u64* row_ws = ws + static_cast<size_t>(r) * kRowWords;
+    const RowSetup rs = row_setup(params, row_ws, r);
+    const u64* words = row_ws + kHistWords + 2 * kSampleSegments;
+    const u64 z_fixed = words[2];
+    const float log_z = static_cast<float>(log(static_cast<double>(z_fixed) / kFixedOne));
+    if (rs.greedy) {
+        if (tid == 0) {
+            out_tokens[r] = rs.arg_max;
+            out_logprobs[r] = -log_z;
+        }
+        return;
+    }
+    const bool k_on = (words[0] >> 32) != 0, p_on = (words[1] >> 32) != 0, mp_on = rs.min_p > 0.0f;
+    const uint32_t k_key = static_cast<uint32_t>(words[0]), p_key = static_cast<uint32_t>(words[1]);
+    const uint32_t max_key = sortable_key(rs.row_max);
+    const u64* seg_kept = row_ws + kHistWords;
+    u64 total = 0;
+    for (int sgm = 0; sgm < kSampleSegments; ++sgm) total += seg_kept[sgm];
+
+    uint32_t ctr[4] = {static_cast<uint32_t>(seeds[r * 2 + 1]), static_cast<uint32_t>(seeds[r * 2 + 1] >> 32), 0u, 0u};
+    philox4x32_10(ctr, static_cast<uint32_t>(seeds[r * 2]), static_cast<uint32_t>(seeds[r * 2] >> 32));
+    const double u = static_cast<double>(((static_cast<u64>(ctr[0]) << 32) | ctr[1]) >> 11) * (1.0 / 9007199254740992.0);
+    u64 target = static_cast<u64>(u * static_cast<double>(total));
+    if (target >= total) target = total - 1;
+    // the segment whose interval holds the target
+    int sgm = 0;
+    u64 seg_base = 0;
+    for (; sgm < kSampleSegments - 1; ++sgm) {
+        if (target < seg_base + seg_kept[sgm]) break;
+        seg_base += seg_kept[sgm];
+    }
+    const int len = segment_length(vocab);
+    const int seg_begin = min(vocab, sgm * len), seg_end = min(vocab, seg_begin + len);
+    const int chunk = (len + kSampleThreads - 1) / kSampleThreads;
+    const int begin = min(seg_end, seg_begin + tid * chunk), end = min(seg_end, begin + chunk);
+    auto kept_mass = [&](int i) -> u64 {
+        const float v = row[i];
+        const uint32_t key = sortable_key(v);
+        const float e = expf((v - rs.row_max) * rs.inv_t);
+        const bool keep = key == max_key || ((!k_on || key >= k_key) && (!p_on || key > p_key) && (!mp_on || e >= rs.min_p));
+        return keep ? static_cast<u64>(static_cast<double>(e) * kFixedOne) : 0ull;
+    };
+    u64 mine = 0;
+    for (int i = begin; i < end; ++i) mine += kept_mass(i);
+    u64 incl = mine;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const u64 o = __shfl_up(incl, off, kWave);
+        if (lane >= off) incl += o;
+    }
+    if (lane == kWave - 1) scan[wave] = incl;
+    if (tid == 0) found_s = -1;
+    __syncthreads();
+    u64 wave_base = seg_base;
+    for (int w = 0; w < wave; ++w) wave_base += scan[w];
+    const u64 excl = wave_base + incl - mine;
+    if (mine > 0 && target >= excl && target < excl + mine) {
+        u64 cum = excl;
+        int tok = begin;
+        for (int i = begin; i < end; ++i) {
+            const u64 w = kept_mass(i);
+            if (w > 0 && target < cum + w) {
+                tok = i;
+                break;
+            }
+            cum += w;
+        }
+        found_s = tok;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        const int tok = found_s >= 0 ? found_s : rs.arg_max;
+        out_tokens[r] = tok;
+        out_logprobs[r] = (row[tok] - rs.row_max) * rs.inv_t - log_z;
+    }
+}
+
+// Words of scratch a row needs in `wllm_sample_rows_split`.
+WLLM_API int wllm_sample_split_row_words() { return kRowWords; }
+
+// The sampler with each row spread over kSampleSegments workgroups.  `scratch` holds rows *
+// wllm_sample_split_row_words() 8-byte words; `truncations` says whether any row has top-k or top-p
+// (then three more histogram levels run).  Same tokens and log-probabilities as `wllm_sample_rows`.
+WLLM_API int wllm_sample_rows_split(float* logits, const float* params, const long long* seeds, const int* penalty_ids,
+                                    const int* penalty_offsets, int* out_tokens, float* out_logprobs, void* scratch,
+                                    int rows, int vocab, int truncations, hipStream_t stream) {
+    if (rows < 1 || vocab < 1 || !scratch) return -1;
+    u64* ws = static_cast<u64*>(scratch);
+    if (penalty_ids) {
+        sample_penalty_kernel<<<rows, 256, 0, stream>>>(logits, params, penalty_ids, penalty_offsets, vocab);
+        if (int err = launch_status()) return err;
+    }
+    const dim3 grid(kSampleSegments, rows);
+    sample_prepare_kernel<<<grid, kSegmentThreads, 0, stream>>>(logits, ws, vocab);
+    if (int err = launch_status()) return err;
+    for (int level = 0; level < (truncations ? 4 : 1); ++level) {
+        sample_histogram_kernel<<<grid, kSegmentThreads, 0, stream>>>(logits, params, ws, vocab, level);
+        if (int err = launch_status()) return err;
+    }
+    sample_kept_kernel<<<grid, kSegmentThreads, 0, stream>>>(logits, params, ws, vocab);
+    if (int err = launch_status()) return err;
+    sample_draw_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, params, seeds, ws, out_tokens, out_logprobs, vocab);
+    return launch_status();
 }
 
 WLLM_API int wllm_sample_rows(float* logits, const float* params, const long long* seeds, const int* penalty_ids,

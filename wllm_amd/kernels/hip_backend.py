@@ -49,6 +49,9 @@ _SIGNATURES = {
     "wllm_gemm_skinny": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
                          c_void_p],
     "wllm_sample_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "wllm_sample_rows_split": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                               c_int, c_int, c_void_p],
+    "wllm_sample_split_row_words": [],
 }
 
 
@@ -60,6 +63,7 @@ class HipBackend:
         self._partial_o = None
         self._gemm_partials = None
         self._argmax_scratch = None
+        self._sample_scratch = None
         self._partial_ml = None
         for name, argtypes in _SIGNATURES.items():
             fn = getattr(self.lib, name)
@@ -333,8 +337,23 @@ class HipBackend:
                                                   _ptr(self._argmax_scratch), rows, logits.shape[1], self._stream()),
                         "argmax_rows")
 
-    def sample_rows(self, logits, params, seeds, penalty_ids, penalty_offsets, out_tokens, out_logprobs):
+    SAMPLE_SPLIT_ROWS = 256     # up to this many rows each row is spread over many workgroups
+
+    def sample_rows(self, logits, params, seeds, penalty_ids, penalty_offsets, out_tokens, out_logprobs,
+                    truncations=True):
         self._on_gpu(logits, params, seeds, penalty_ids, penalty_offsets, out_tokens, out_logprobs)
+        rows, vocab = logits.shape
+        if rows <= self.SAMPLE_SPLIT_ROWS:
+            # a decode step's few rows: one workgroup a row would leave the chip idle
+            if self._sample_scratch is None or self._sample_scratch.device != logits.device:
+                words = self.lib.wllm_sample_split_row_words()
+                self._sample_scratch = torch.empty(self.SAMPLE_SPLIT_ROWS * words, dtype=torch.int64,
+                                                   device=logits.device)
+            self._check(self.lib.wllm_sample_rows_split(
+                _ptr(logits), _ptr(params), _ptr(seeds), _ptr(penalty_ids), _ptr(penalty_offsets), _ptr(out_tokens),
+                _ptr(out_logprobs), _ptr(self._sample_scratch), rows, vocab, int(bool(truncations)), self._stream()),
+                "sample_rows (rows spread over workgroups)")
+            return
         self._check(self.lib.wllm_sample_rows(
             _ptr(logits), _ptr(params), _ptr(seeds), _ptr(penalty_ids), _ptr(penalty_offsets), _ptr(out_tokens),
-            _ptr(out_logprobs), logits.shape[0], logits.shape[1], self._stream()), "sample_rows")
+            _ptr(out_logprobs), rows, vocab, self._stream()), "sample_rows")

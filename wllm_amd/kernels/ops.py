@@ -419,7 +419,7 @@ def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> None:
 
 def sample_rows(logits: torch.Tensor, params: torch.Tensor, seeds: torch.Tensor,
                 penalty_ids: Optional[torch.Tensor], penalty_offsets: Optional[torch.Tensor],
-                out_tokens: torch.Tensor, out_logprobs: torch.Tensor) -> None:
+                out_tokens: torch.Tensor, out_logprobs: torch.Tensor, truncations: bool = True) -> None:
     """Samples one token per row.
 
     logits float32 [m, V].  params float32 [m, 5]: temperature (0: greedy), top_k (0: off),
@@ -428,7 +428,8 @@ def sample_rows(logits: torch.Tensor, params: torch.Tensor, seeds: torch.Tensor,
     int32 [m+1]: the ids the repetition penalty applies to, row by row (None: no row has
     any).  out_tokens int32 [m]; out_logprobs float32 [m]: log-probability of the token
     under the penalised, temperature-scaled distribution before truncation (temperature 1
-    for greedy rows).
+    for greedy rows).  `truncations` may be False only if no row has top_k or top_p on: the
+    kernels then skip the passes that find their thresholds.
     """
     _dense(logits, "logits", torch.float32)
     _need(logits.dim() == 2 and logits.shape[1] > 0, "logits: expected [rows, vocab]")
@@ -442,4 +443,5 @@ def sample_rows(logits: torch.Tensor, params: torch.Tensor, seeds: torch.Tensor,
     _dense(out_tokens, "out_tokens", torch.int32, (m,))
     _dense(out_logprobs, "out_logprobs", torch.float32, (m,))
     if m:
-        backend().sample_rows(logits, params, seeds, penalty_ids, penalty_offsets, out_tokens, out_logprobs)
+        backend().sample_rows(logits, params, seeds, penalty_ids, penalty_offsets, out_tokens, out_logprobs,
+                              truncations)

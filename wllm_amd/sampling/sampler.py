@@ -65,8 +65,9 @@ class Sampler:
                 pen_ids = torch.from_numpy(flat).to(logits.device)
                 pen_off = torch.from_numpy(offsets).to(logits.device)
         logprobs = torch.empty(m, dtype=torch.float32, device=logits.device)
+        truncations = any(not p.greedy and (p.top_k > 0 or p.top_p < 1.0) for p in params)
         ops.sample_rows(logits, torch.from_numpy(table).to(logits.device), torch.from_numpy(keys).to(logits.device),
-                        pen_ids, pen_off, tokens, logprobs)
+                        pen_ids, pen_off, tokens, logprobs, truncations=truncations)
         return PendingSample(tokens, logprobs)
 
     @staticmethod
