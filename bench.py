@@ -92,8 +92,8 @@ def measure_decode(model, batch: int, context: int, steps: int, warmup: int, blo
     import torch
 
     from wllm_amd.engine import ModelRunner, Request, Scheduler
-    # requests admitted first decode while the later ones are still prefilled, one prompt a step
-    total_new = batch + warmup + steps + 2
+    # requests admitted first decode while the later ones are still prefilled, one portion of a prompt a step
+    total_new = batch * (-(-context // chunk)) + warmup + steps + 2
     pages = batch * (-(-(context + total_new) // block_size)) + 2
     runner = ModelRunner.create(model, num_pages=pages, page_size=block_size, max_requests=batch)
     if hip_graphs and hasattr(runner, "enable_graphs"):
