@@ -315,6 +315,21 @@ def test_linear(dtype, m, n, k):
             close(g[2], r[2], out_dtype, f"product to {out_dtype}, tiled {tiled}")
 
 
+@pytest.mark.parametrize("n,k", [(777, 250), (2048, 2048), (100, 4128), (33, 64), (2560, 16384)])
+def test_float32_product_of_few_rows_has_the_bits_of_the_product_of_many(n, k):
+    """In float32 an element is the sum over k in ascending order whatever the number of rows, so a
+    token's projection in a decode step equals, bit for bit, its projection inside a long prompt."""
+    torch.manual_seed(14)
+    x = torch.randn(40, k, device=DEV)
+    w = torch.randn(n, k, device=DEV) / math.sqrt(k)
+    many = torch.zeros(40, n, device=DEV)
+    ops.linear(x, w, many)
+    for rows in (1, 7, 16):
+        few = torch.full((rows, n), 9.0, device=DEV)
+        ops.linear(x[11:11 + rows].contiguous(), w, few)
+        assert torch.equal(few, many[11:11 + rows]), f"{rows} rows"
+
+
 def test_tile_weight_is_the_documented_permutation():
     torch.manual_seed(12)
     for n, k, halves in ((40, 96, 1), (16, 32, 1), (2 * 23, 64, 2), (777, 2048, 1)):

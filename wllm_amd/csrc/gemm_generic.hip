@@ -63,8 +63,67 @@ gemm_nt_kernel(const TI* __restrict__ x, const TI* __restrict__ w, TO* __restric
     }
 }
 
+// The same product for at most 16 rows of float32 (the decode steps of the float32 path).  The big
+// tile would leave all but N/64 workgroups idle and seven eighths of each tile empty; here a
+// workgroup makes 16 rows x 16 columns, a thread one element, and the K axis is walked in chunks
+// of 128 through shared memory.  An element is still the sum over k in ascending order of fused
+// multiply-adds from zero, so it has the same bits as the kernel above gives it.
+constexpr int kFewRows = 16;
+constexpr int kFewChunk = 128;
+
+__global__ void __launch_bounds__(256)
+gemm_nt_few_rows_kernel(const float* __restrict__ x, const float* __restrict__ w, float* __restrict__ out, int M,
+                        int N, int K) {
+    __shared__ float4 xs[kFewRows][kFewChunk / 4 + 1];
+    __shared__ float4 ws[kFewRows][kFewChunk / 4 + 1];
+    const int tid = threadIdx.x;
+    const int col0 = blockIdx.x * kFewRows;
+    const int r = tid / 16, c = tid % 16;
+    // staging: a thread moves two 16-byte pieces of x and two of w per chunk
+    const int srow[2] = {tid / 32, tid / 32 + 8};
+    const int sk = (tid % 32) * 4;
+    float4 xreg[2], wreg[2];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const bool in_k = k0 + sk < K;
+            xreg[j] = (srow[j] < M && in_k) ? *reinterpret_cast<const float4*>(x + static_cast<size_t>(srow[j]) * K + k0 + sk)
+                                            : make_float4(0.f, 0.f, 0.f, 0.f);
+            wreg[j] = (col0 + srow[j] < N && in_k)
+                          ? *reinterpret_cast<const float4*>(w + static_cast<size_t>(col0 + srow[j]) * K + k0 + sk)
+                          : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    float acc = 0.f;
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += kFewChunk) {
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            xs[srow[j]][sk / 4] = xreg[j];
+            ws[srow[j]][sk / 4] = wreg[j];
+        }
+        __syncthreads();
+        if (k0 + kFewChunk < K) fetch(k0 + kFewChunk);
+        const int len = min(kFewChunk, K - k0);     // a multiple of 4
+        for (int k = 0; k < len; k += 4) {
+            const float4 a = xs[r][k / 4], b = ws[c][k / 4];
+            acc = fmaf(a.x, b.x, acc);
+            acc = fmaf(a.y, b.y, acc);
+            acc = fmaf(a.z, b.z, acc);
+            acc = fmaf(a.w, b.w, acc);
+        }
+    }
+    if (r < M && col0 + c < N) out[static_cast<size_t>(r) * N + col0 + c] = acc;
+}
+
 WLLM_API int wllm_gemm_generic(const void* x, const void* w, int in_bf16, void* out, int out_bf16, int M, int N,
                                int K, hipStream_t stream) {
+    if (!in_bf16 && !out_bf16 && M <= kFewRows && K % 4 == 0) {
+        gemm_nt_few_rows_kernel<<<(N + kFewRows - 1) / kFewRows, 256, 0, stream>>>(
+            static_cast<const float*>(x), static_cast<const float*>(w), static_cast<float*>(out), M, N, K);
+        return launch_status();
+    }
     const dim3 grid((N + kTile - 1) / kTile, (M + kTile - 1) / kTile);
     if (grid.y > 65535) return -1;
 #define LAUNCH(TI, TO)                                                                                  \
