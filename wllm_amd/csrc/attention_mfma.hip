@@ -188,7 +188,7 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
         float pe[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            pe[e] = ok[e] ? exp2f(fmaf(sv[e], scale_log2e, -mc)) : 0.f;
+            pe[e] = ok[e] ? exp2_probability(fmaf(sv[e], scale_log2e, -mc)) : 0.f;
             l_run += pe[e];
         }
         pv.u = make_uint4(pack2_bf16(pe[0], pe[1]), pack2_bf16(pe[2], pe[3]), pack2_bf16(pe[4], pe[5]),

@@ -261,11 +261,11 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
             const float m_new = fmaxf(m_run[rt], tile_max);
             const float m_use = m_new == -INFINITY ? 0.f : m_new;
             const float mc = m_use * scale_log2e;
-            alpha[rt] = exp2f(fmaf(m_run[rt], scale_log2e, -mc));
+            alpha[rt] = exp2_probability(fmaf(m_run[rt], scale_log2e, -mc));
             float pe[8], psum = 0.f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                pe[e] = exp2f(fmaf(sv[e], scale_log2e, -mc));       // exp2(-inf) = 0 for masked keys
+                pe[e] = exp2_probability(fmaf(sv[e], scale_log2e, -mc));       // exp2(-inf) = 0 for masked keys
                 psum += pe[e];
             }
             pv[rt].u = make_uint4(pack2_bf16(pe[0], pe[1]), pack2_bf16(pe[2], pe[3]), pack2_bf16(pe[4], pe[5]),

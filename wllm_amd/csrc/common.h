@@ -73,6 +73,11 @@ __device__ __forceinline__ float stack_sum(const float* __restrict__ p, int spli
     return total;
 }
 
+// 2^x by the hardware instruction alone, for the arguments of a softmax (x <= 0, -inf included):
+// results below the smallest normal number become 0 instead of passing through the library's
+// rescaling, which a probability does not need.
+__device__ __forceinline__ float exp2_probability(float x) { return __builtin_amdgcn_exp2f(x); }
+
 // One rotated pair (a, b) -> (a cos - b sin, b cos + a sin).  The products are fused in one fixed
 // way, so that every kernel that rotates gives the same bits for the same numbers.
 __device__ __forceinline__ void rotate_pair(float a, float b, float s, float c, float& ra, float& rb) {
