@@ -179,6 +179,28 @@ def test_captured_graphs_give_what_eager_steps_give(model_folders, dtype):
         assert torch.allclose(torch.tensor(a.logprobs), torch.tensor(b.logprobs), atol=1e-5 if dtype == "float32" else 2e-2)
 
 
+def test_a_full_batch_of_any_size_has_its_graph(model_folders):
+    """The largest number of requests the cache admits is a bucket of its own: a full batch of 3
+    (or 17) does not fall back to steps run kernel by kernel."""
+    model = load_model(model_folders["M"], "bfloat16", "cuda")
+    runner = ModelRunner.create(model, num_pages=40, page_size=16, max_requests=3)
+    runner.enable_graphs()
+    assert runner.graph_buckets == (1, 2, 3)
+    s = Scheduler(runner, max_prefill_tokens_per_step=64)
+    reqs = [Request(i, random_ids(90 + i, 11 + i, 1000), 12) for i in range(3)]
+    for r in reqs:
+        s.add_request(r)
+    s.run_to_completion()
+    assert 3 in runner.graphs and runner.graph_steps >= 8
+    plain = ModelRunner.create(model, num_pages=40, page_size=16, max_requests=3)
+    s2 = Scheduler(plain, max_prefill_tokens_per_step=64)
+    again = [Request(i, random_ids(90 + i, 11 + i, 1000), 12) for i in range(3)]
+    for r in again:
+        s2.add_request(r)
+    s2.run_to_completion()
+    assert [r.output_token_ids for r in reqs] == [r.output_token_ids for r in again]
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("graphs", [False, True])
 def test_looking_ahead_gives_the_same_tokens_on_the_gpu(model_folders, dtype, graphs):

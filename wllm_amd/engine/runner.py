@@ -39,16 +39,19 @@ class ModelRunner:
         self.dummy_pages: list = []
         self.graph_steps = 0
 
-    def enable_graphs(self, buckets=(1, 2, 4, 8, 16, 32, 64), max_context=None) -> None:
+    def enable_graphs(self, buckets=(1, 2, 4, 8, 16, 32, 64, 128, 256), max_context=None) -> None:
         """Decode-only steps of up to max(buckets) requests replay a captured graph of the
-        smallest bucket that holds them.  One page per group is set aside for padding rows."""
+        smallest bucket that holds them; the largest number of requests the cache admits, if it
+        is below max(buckets), is a bucket too, so that a full batch of any size has its graph.
+        One page per group is set aside for padding rows."""
         if self.graph_buckets:
             return
         if not self.model.graph_capturable():
             raise ValueError("a part of this model reads the step's arrays on the host; its steps cannot be captured")
         limit = min(self.model.plan.max_positions, min(g.pool.num_pages - 1 for g in self.cache.groups) * self.cache.page_size)
         self.graph_max_context = min(max_context or limit, limit)
-        self.graph_buckets = tuple(sorted(b for b in buckets if b <= self.cache.max_requests)) or (self.cache.max_requests,)
+        most = self.cache.max_requests
+        self.graph_buckets = tuple(sorted({b for b in buckets if b <= most} | ({most} if most <= max(buckets) else set())))
         self.dummy_pages = [self.cache.set_aside_page(gi) for gi in range(len(self.cache.groups))]
 
     def _graph_for(self, entries: list):
