@@ -17,6 +17,10 @@ class KernelError(RuntimeError):
     """A kernel launch failed or a kernel refused its operands."""
 
 
+# torch's own shortcut to the current stream's handle (what its compiled kernels call)
+_raw_current_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _ptr(t):
     return c_void_p(t.data_ptr()) if t is not None else c_void_p(0)
 
@@ -60,6 +64,7 @@ class HipBackend:
         if not torch.cuda.is_available():
             raise KernelError("no GPU is visible; the kernels run on gfx950 only and there is no other path")
         self.lib = load()
+        self._device_index = torch.cuda.current_device()
         self._partial_o = None
         self._gemm_partials = None
         self._argmax_scratch = None
@@ -76,8 +81,10 @@ class HipBackend:
             if t is not None and not t.is_cuda:
                 raise KernelError("a kernel operand is not on the GPU")
 
-    @staticmethod
-    def _stream() -> c_void_p:
+    def _stream(self) -> c_void_p:
+        # the raw handle of torch's current stream on this process's GPU, asked for at every launch
+        if _raw_current_stream is not None:
+            return c_void_p(_raw_current_stream(self._device_index))
         return c_void_p(torch.cuda.current_stream().cuda_stream)
 
     @staticmethod

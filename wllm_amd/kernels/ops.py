@@ -44,20 +44,25 @@ def use_backend(obj):
         _backend = old
 
 
-def _need(cond: bool, msg: str) -> None:
+def _need(cond: bool, msg) -> None:
+    """`msg` is the message or a function that makes it (so that it is made only on failure)."""
     if not cond:
-        raise KernelShapeError(msg)
+        raise KernelShapeError(msg() if callable(msg) else msg)
 
 
 def _dense(t: torch.Tensor, name: str, dtype, shape=None) -> None:
-    _need(isinstance(t, torch.Tensor), f"{name}: expected a tensor")
+    # the messages are made only when a check fails: this runs for every operand of every launch
+    if not isinstance(t, torch.Tensor):
+        raise KernelShapeError(f"{name}: expected a tensor")
     if isinstance(dtype, tuple):
-        _need(t.dtype in dtype, f"{name}: dtype {t.dtype}, expected one of {dtype}")
-    else:
-        _need(t.dtype == dtype, f"{name}: dtype {t.dtype}, expected {dtype}")
-    _need(t.is_contiguous(), f"{name}: must be contiguous")
-    if shape is not None:
-        _need(tuple(t.shape) == tuple(shape), f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
+        if t.dtype not in dtype:
+            raise KernelShapeError(f"{name}: dtype {t.dtype}, expected one of {dtype}")
+    elif t.dtype != dtype:
+        raise KernelShapeError(f"{name}: dtype {t.dtype}, expected {dtype}")
+    if not t.is_contiguous():
+        raise KernelShapeError(f"{name}: must be contiguous")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise KernelShapeError(f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
 
 
 def embed_lookup(ids: torch.Tensor, table: torch.Tensor, scale: float, out: torch.Tensor) -> None:
@@ -77,7 +82,7 @@ def feed_tokens(ids: torch.Tensor, dst: torch.Tensor, src: torch.Tensor, source:
     before it sampled on the device."""
     for t, name in ((ids, "ids"), (dst, "dst"), (src, "src"), (source, "source")):
         _dense(t, name, torch.int32)
-        _need(t.dim() == 1, f"{name}: expected one axis")
+        _need(t.dim() == 1, lambda: f"{name}: expected one axis")
     _need(dst.shape == src.shape, "dst and src: expected equal lengths")
     if dst.shape[0]:
         backend().feed_tokens(ids, dst, src, source)
@@ -132,7 +137,7 @@ def rope_and_cache_write(qkv: torch.Tensor, bias: Optional[torch.Tensor], positi
     """
     width = (num_heads + 2 * num_kv_heads) * head_dim
     _dense(qkv, "qkv", _ACT)
-    _need(qkv.dim() == 2 and qkv.shape[1] == width, f"qkv: shape {tuple(qkv.shape)}, expected [n, {width}]")
+    _need(qkv.dim() == 2 and qkv.shape[1] == width, lambda: f"qkv: shape {tuple(qkv.shape)}, expected [n, {width}]")
     n = qkv.shape[0]
     if bias is not None:
         _dense(bias, "bias", torch.float32, (width,))
@@ -145,13 +150,13 @@ def rope_and_cache_write(qkv: torch.Tensor, bias: Optional[torch.Tensor], positi
         _dense(inv_freq, "inv_freq", torch.float32)
         _need(inv_freq.dim() == 1, "inv_freq: expected one axis")
         rotary_dim = 2 * inv_freq.shape[0]
-        _need(0 < rotary_dim <= head_dim, f"rotary_dim {rotary_dim} does not fit head_dim {head_dim}")
+        _need(0 < rotary_dim <= head_dim, lambda: f"rotary_dim {rotary_dim} does not fit head_dim {head_dim}")
     _need((slots is None) == (cache is None), "slots and cache go together")
     if cache is not None:
         _dense(slots, "slots", torch.int32, (n,))
         _dense(cache, "cache", qkv.dtype)
         _need(cache.dim() == 4 and tuple(cache.shape[1:]) == (2, num_kv_heads, page_size * head_dim),
-              f"cache: shape {tuple(cache.shape)}, expected [pages, 2, {num_kv_heads}, {page_size * head_dim}]")
+              lambda: f"cache: shape {tuple(cache.shape)}, expected [pages, 2, {num_kv_heads}, {page_size * head_dim}]")
     if n:
         backend().rope_and_cache_write(qkv, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads,
                                        head_dim, rotary_dim, page_size, parts)
@@ -173,7 +178,7 @@ def linear_residual(x: torch.Tensor, weight: torch.Tensor, residual: torch.Tenso
     _need(x.dim() == 2, "x: expected [rows, in]")
     m, k = x.shape
     _dense(weight, "weight", x.dtype)
-    _need(weight.dim() == 2 and weight.shape[1] == k, f"weight: shape {tuple(weight.shape)}, expected [out, {k}]")
+    _need(weight.dim() == 2 and weight.shape[1] == k, lambda: f"weight: shape {tuple(weight.shape)}, expected [out, {k}]")
     n = weight.shape[0]
     _check_tiles(tiles, weight, 1)
     _need(linear_residual_takes(m, x.dtype, n, k), "linear_residual: no kernel for these sizes")
@@ -220,7 +225,7 @@ def qkv_rope(x: torch.Tensor, weight: torch.Tensor, qkv: torch.Tensor, bias: Opt
         _dense(slots, "slots", torch.int32, (n,))
         _dense(cache, "cache", x.dtype)
         _need(cache.dim() == 4 and tuple(cache.shape[1:]) == (2, num_kv_heads, page_size * head_dim),
-              f"cache: shape {tuple(cache.shape)}, expected [pages, 2, {num_kv_heads}, {page_size * head_dim}]")
+              lambda: f"cache: shape {tuple(cache.shape)}, expected [pages, 2, {num_kv_heads}, {page_size * head_dim}]")
     if n:
         backend().qkv_rope(x, weight, tiles, qkv, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads,
                            head_dim, page_size)
@@ -245,12 +250,12 @@ def paged_attention(qkv: torch.Tensor, cache: torch.Tensor, block_tables: torch.
     """
     width = (num_heads + 2 * num_kv_heads) * head_dim
     _dense(qkv, "qkv", _ACT)
-    _need(qkv.dim() == 2 and qkv.shape[1] == width, f"qkv: shape {tuple(qkv.shape)}, expected [n, {width}]")
+    _need(qkv.dim() == 2 and qkv.shape[1] == width, lambda: f"qkv: shape {tuple(qkv.shape)}, expected [n, {width}]")
     n = qkv.shape[0]
     _need(num_heads % num_kv_heads == 0, "num_heads must be a multiple of num_kv_heads")
     _dense(cache, "cache", qkv.dtype)
     _need(cache.dim() == 4 and tuple(cache.shape[1:]) == (2, num_kv_heads, page_size * head_dim),
-          f"cache: shape {tuple(cache.shape)}, expected [pages, 2, {num_kv_heads}, {page_size * head_dim}]")
+          lambda: f"cache: shape {tuple(cache.shape)}, expected [pages, 2, {num_kv_heads}, {page_size * head_dim}]")
     _dense(block_tables, "block_tables", torch.int32)
     _need(block_tables.dim() == 2, "block_tables: expected [segments, pages]")
     s = block_tables.shape[0]
@@ -324,7 +329,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, tiles: Opti
     _need(x.dim() == 2, "x: expected [rows, in]")
     _dense(weight, "weight", x.dtype)
     _need(weight.dim() == 2 and weight.shape[1] == x.shape[1],
-          f"weight: shape {tuple(weight.shape)}, expected [out, {x.shape[1]}]")
+          lambda: f"weight: shape {tuple(weight.shape)}, expected [out, {x.shape[1]}]")
     _check_tiles(tiles, weight, 1)
     if out.dim() == 3:
         s = linear_splits(x.shape[0], weight.shape[0], x.shape[1], x.dtype)
@@ -341,7 +346,7 @@ ACTIVATIONS = ("gelu_tanh", "silu")
 
 def gated_activation(gate_up: torch.Tensor, out: torch.Tensor, activation: str) -> None:
     """out = act(gate_up[:, :I]) * gate_up[:, I:], in float32, cast to T.  gate_up T [n, 2I]."""
-    _need(activation in ACTIVATIONS, f"activation {activation!r}: expected one of {ACTIVATIONS}")
+    _need(activation in ACTIVATIONS, lambda: f"activation {activation!r}: expected one of {ACTIVATIONS}")
     _dense(gate_up, "gate_up", _ACT)
     _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "gate_up: expected [n, 2*intermediate]")
     _dense(out, "out", gate_up.dtype, (gate_up.shape[0], gate_up.shape[1] // 2))
@@ -383,12 +388,12 @@ def gated_linear(x, weight: torch.Tensor, out: torch.Tensor, activation: str,
     out T [m, I]; scratch T [m, 2I] may be used for the unfused product.  `tiles` is
     `tile_weight(weight, halves=2)`.  x may be a `NormOnLoad` where `gated_linear_norm_takes` says so:
     the norm is then applied as the kernel reads the residual stream (scratch is not used)."""
-    _need(activation in ACTIVATIONS, f"activation {activation!r}: expected one of {ACTIVATIONS}")
+    _need(activation in ACTIVATIONS, lambda: f"activation {activation!r}: expected one of {ACTIVATIONS}")
     if isinstance(x, NormOnLoad):
         _need(gated_linear_norm_takes(x.shape[0], x.dtype, x.shape[1]), "gated_linear: no kernel with the norm on load for these sizes")
         _dense(weight, "weight", x.dtype)
         _need(weight.dim() == 2 and weight.shape[1] == x.shape[1] and weight.shape[0] % 2 == 0,
-              f"weight: shape {tuple(weight.shape)}, expected [2*intermediate, {x.shape[1]}]")
+              lambda: f"weight: shape {tuple(weight.shape)}, expected [2*intermediate, {x.shape[1]}]")
         _dense(out, "out", x.dtype, (x.shape[0], weight.shape[0] // 2))
         _check_tiles(tiles, weight, 2)
         if x.shape[0]:
@@ -398,7 +403,7 @@ def gated_linear(x, weight: torch.Tensor, out: torch.Tensor, activation: str,
     _need(x.dim() == 2, "x: expected [rows, in]")
     _dense(weight, "weight", x.dtype)
     _need(weight.dim() == 2 and weight.shape[1] == x.shape[1] and weight.shape[0] % 2 == 0,
-          f"weight: shape {tuple(weight.shape)}, expected [2*intermediate, {x.shape[1]}]")
+          lambda: f"weight: shape {tuple(weight.shape)}, expected [2*intermediate, {x.shape[1]}]")
     inter = weight.shape[0] // 2
     _dense(out, "out", x.dtype, (x.shape[0], inter))
     _dense(scratch, "scratch", x.dtype, (x.shape[0], 2 * inter))
