@@ -33,6 +33,7 @@
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));     // 16 bytes as one value (no aggregate copy)
 
 constexpr int kItemInts = 8;
 constexpr int kRowsPerTile = 16;
@@ -57,8 +58,17 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
                             int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window) {
     constexpr int DC = HD / 32;   // 32-wide chunks of the head for the score product
     constexpr int DT = HD / 16;   // 16-row tiles of out^T
-    // merge buffer: two slots of [16 rows][HD + 2] floats
-    __shared__ float merge_s[2][kRowsPerTile * (HD + 2)];
+    // Shared memory, used twice.  First each wavefront turns its block of keys, which it reads
+    // from the cache row by row (whole key rows: contiguous runs the memory system streams much
+    // faster than the 64-byte pieces a fragment load straight from the cache would ask for), into
+    // fragments: [4 wavefronts][32 keys][HD + 8] bfloat16, rows padded so that the fragment reads
+    // spread over the banks.  Then, after a barrier, the merge buffer: two slots of [16 rows][HD + 2]
+    // floats.
+    constexpr int kKeyStride = HD + 8;                                      // elements
+    constexpr int kStageBytes = 4 * kKeysPerBlock * kKeyStride * 2;
+    constexpr int kMergeBytes = 2 * kRowsPerTile * (HD + 2) * 4;
+    __shared__ __align__(16) unsigned char shared_raw[kStageBytes > kMergeBytes ? kStageBytes : kMergeBytes];
+    float (*merge_s)[kRowsPerTile * (HD + 2)] = reinterpret_cast<float (*)[kRowsPerTile * (HD + 2)]>(shared_raw);
 
     const int* item = items + static_cast<size_t>(blockIdx.x) * kItemInts;
     const int seg = item[0], kvh = item[1], row_begin = item[2];
@@ -83,20 +93,25 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
     const int* table = block_tables + static_cast<size_t>(seg) * max_pages;
     const int blk_first = key_begin / kKeysPerBlock;
     const int blk_end = (key_end + kKeysPerBlock - 1) / kKeysPerBlock;
-    Pack16 ka_[2][DC], va_[DT];
+    // a block's keys as the cache holds them: 32 rows of HD, 16 bytes a lane and load
+    constexpr int kPieces = HD / 8;                 // 16-byte pieces of a key row
+    uint4_t kraw[DT];                               // 32 * kPieces / 64 = HD / 16 loads a lane
+    Pack16 va_[DT];
     // All loads of a block are issued before the first product needs one, so a block costs one
     // trip to memory.  Keys beyond the request are masked later; their table entry is clamped to
     // the table's width (entries beyond a request's pages name a valid page), not to the length.
     auto issue = [&](int blk) {
         const int kbase = blk * kKeysPerBlock;
-        const bf16* krow[2];
+        const bf16* kpiece[DT];
 #pragma unroll
-        for (int t2 = 0; t2 < 2; ++t2) {
-            // which key the A row i of the score product is; see the header for why
-            const int kk = kbase + (V16 ? 8 * (i / 4) + 4 * t2 + (i % 4) : 16 * t2 + i);
+        for (int j = 0; j < DT; ++j) {
+            // piece f of the block: key f / kPieces, its 8 elements f % kPieces; a wavefront's load
+            // covers whole consecutive rows
+            const int f = j * kWave + lane;
+            const int kk = kbase + f / kPieces;
             const int page = table[min(kk / page_size, max_pages - 1)];
-            krow[t2] = cache + static_cast<size_t>(page) * page_elems + k_off +
-                       static_cast<size_t>(kk % page_size) * HD + 8 * g;
+            kpiece[j] = cache + static_cast<size_t>(page) * page_elems + k_off +
+                        static_cast<size_t>(kk % page_size) * HD + (f % kPieces) * 8;
         }
         int vpage0, vslot0, vpage1 = 0, vslot1 = 0;
         if (V16) {
@@ -113,9 +128,7 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
         const bf16* vbase0 = cache + static_cast<size_t>(vpage0) * page_elems + v_off + vslot0;
         const bf16* vbase1 = cache + static_cast<size_t>(vpage1) * page_elems + v_off + vslot1;
 #pragma unroll
-        for (int t2 = 0; t2 < 2; ++t2)
-#pragma unroll
-            for (int c = 0; c < DC; ++c) ka_[t2][c].u = *reinterpret_cast<const uint4*>(krow[t2] + c * 32);
+        for (int j = 0; j < DT; ++j) kraw[j] = *reinterpret_cast<const uint4_t*>(kpiece[j]);
 #pragma unroll
         for (int t = 0; t < DT; ++t) {
             const size_t drow = static_cast<size_t>(t * 16 + i) * page_size;
@@ -158,14 +171,32 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
         }
         const int kbase = blk * kKeysPerBlock;
         const bool edge = kbase < seg_lo || kbase + kKeysPerBlock > ctx;
-        // ---- scores of two tiles of 16 keys ----
+        // ---- the keys through this wavefront's part of shared memory, then the scores of two
+        //      tiles of 16 keys ----
+        uint16_t* stage = reinterpret_cast<uint16_t*>(shared_raw) + wave * (kKeysPerBlock * kKeyStride);
+        {
+            // piece f = j * 64 + lane lies (64 / kPieces) rows further with every j when 64 is a
+            // multiple of kPieces; in general its row and place are computed per piece
+            const int f0 = lane;
+#pragma unroll
+            for (int j = 0; j < DT; ++j) {
+                const int f = f0 + j * kWave;
+                uint16_t* dst = stage + (f / kPieces) * kKeyStride + (f % kPieces) * 8;
+                *reinterpret_cast<uint4_t*>(dst) = kraw[j];
+            }
+        }
         float4_t s[2];
 #pragma unroll
         for (int t2 = 0; t2 < 2; ++t2) {
+            // which key row i of the first operand is; see the header for why
+            const int key = V16 ? 8 * (i / 4) + 4 * t2 + (i % 4) : 16 * t2 + i;
             float4_t sc = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int c = 0; c < DC; ++c)
-                sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka_[t2][c].v, qreg[c], sc, 0, 0, 0);
+            for (int c = 0; c < DC; ++c) {
+                Pack16 a;
+                a.u = *reinterpret_cast<const uint4*>(stage + key * kKeyStride + c * 32 + 8 * g);
+                sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qreg[c], sc, 0, 0, 0);
+            }
             s[t2] = sc;
         }
         // ---- mask, maximum, probabilities ----
