@@ -16,6 +16,8 @@ No memset node is recorded: buffers are cleared, where they must be, by kernels.
 """
 from __future__ import annotations
 
+import gc
+
 import numpy as np
 import torch
 
@@ -122,8 +124,17 @@ class DecodeGraph:
             self.runner.model.forward(self.ctx)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                self.logits = self.runner.model.forward(self.ctx)
+            # No garbage collection while the stream is capturing: a collector run that frees an
+            # object with device resources of its own (an event, pinned memory, another graph)
+            # makes a call the capture does not allow, and the process aborts.
+            collecting = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(graph):
+                    self.logits = self.runner.model.forward(self.ctx)
+            finally:
+                if collecting:
+                    gc.enable()
             self.graph = graph
         self.graph.replay()
         return self.logits[:len(entries)]
