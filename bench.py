@@ -1,4 +1,4 @@
-"""Decode and prefill throughput of the engine at the Gemma-2B layer sizes, on one MI355X.
+"""Decode and prefill throughput of the engine at the Gemma-2B layer sizes (or `--shape`), on one MI355X.
 
     python bench.py --gpus 1 --steps K --warmup W
 
@@ -154,7 +154,8 @@ def run_stress(model, args) -> dict:
     runner.cache.check()
     generated = sum(len(r.output_token_ids) for r in finished)
     assert len(finished) == n and generated == int(outputs.sum())
-    return {"metric": "continuous-batching stress, Gemma-2B layer sizes", "value": round(generated / dt, 1),
+    sizes = {"gemma-2b": "Gemma-2B", "gemma-7b": "Gemma-7B"}.get(args.shape, os.path.basename(args.shape))
+    return {"metric": f"continuous-batching stress, {sizes} layer sizes", "value": round(generated / dt, 1),
             "unit": "generated tokens/s", "seconds": round(dt, 3), "requests": n, "steps": sched.stats["steps"],
             "prompt_tokens": int(prompts.sum()), "generated_tokens": generated,
             "total_tokens_per_s": round((generated + int(prompts.sum())) / dt, 1),
@@ -226,8 +227,9 @@ def main() -> int:
                 points[f"decode_b{b}"] = round(k * b / d, 1)
 
     c = model.config
+    sizes = {"gemma-2b": "Gemma-2B", "gemma-7b": "Gemma-7B"}.get(args.shape, os.path.basename(args.shape))
     line = {
-        "metric": "decode tokens/s, Gemma-2B layer sizes, after 2,048-token prompts",
+        "metric": f"decode tokens/s, {sizes} layer sizes, after {args.context:,}-token prompts",
         "value": round(value, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -240,7 +242,7 @@ def main() -> int:
         "dtype": args.dtype,
         "data": "synthetic: seeded random weights (normal, std 0.02) and seeded uniform token ids",
         "config": {
-            "model": "Gemma-2B layer sizes (GemmaForCausalLM), random weights",
+            "model": f"{sizes} layer sizes (GemmaForCausalLM), random weights",
             "global_batch": args.batch, "seq_len": args.context, "parallelism": "single GPU",
             "layers": c.num_hidden_layers, "layers_of_full_model": full_layers, "hidden_size": c.hidden_size,
             "intermediate_size": c.intermediate_size, "num_attention_heads": c.num_attention_heads,
