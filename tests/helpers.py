@@ -8,8 +8,8 @@ from wllm_amd.config import GemmaConfig
 from wllm_amd.parts import write_random_model_folder
 
 # Two tiny configurations that differ in every size and option, a third with
-# biases and an untied head, and a fourth whose head size and page size are the
-# ones the matrix-core attention kernels take.
+# biases and an untied head, a fourth whose head size and page size are the
+# ones the matrix-core attention kernels take, and a fifth without grouped heads.
 TINY = {
     "A": dict(config=GemmaConfig(vocab_size=512, hidden_size=64, intermediate_size=256, num_hidden_layers=2,
                                  num_attention_heads=4, num_key_value_heads=1, head_dim=32, rms_norm_eps=1e-6,
@@ -28,6 +28,12 @@ TINY = {
                                  num_attention_heads=8, num_key_value_heads=2, head_dim=64, rms_norm_eps=1e-6,
                                  rope_theta=10000.0, max_position_embeddings=512, tie_word_embeddings=True),
               seed=44, std=0.04, norm_std=0.1, page_size=16),
+    # every query head with its own key/value head, a head size the matrix-core kernels take, and
+    # heads * head_dim (160) unlike the width (96): the arrangement of the 7B sizes
+    "S": dict(config=GemmaConfig(vocab_size=1200, hidden_size=96, intermediate_size=192, num_hidden_layers=2,
+                                 num_attention_heads=5, num_key_value_heads=5, head_dim=32, rms_norm_eps=1e-6,
+                                 rope_theta=10000.0, max_position_embeddings=256, tie_word_embeddings=True),
+              seed=55, std=0.04, norm_std=0.1, page_size=8),
 }
 
 

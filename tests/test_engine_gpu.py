@@ -12,7 +12,8 @@ from wllm_amd.parts import load_model
 
 pytestmark = pytest.mark.gpu
 
-LENGTHS = {"A": [40, 57, 72, 33, 90, 64], "B": [45, 97, 64, 130, 51, 80], "C": [37, 66, 49, 100, 41], "M": [70, 130, 48, 97, 33]}
+LENGTHS = {"A": [40, 57, 72, 33, 90, 64], "B": [45, 97, 64, 130, 51, 80], "C": [37, 66, 49, 100, 41], "M": [70, 130, 48, 97, 33],
+           "S": [50, 33, 120, 64, 77]}
 FAMILIES = {"whole": trace_whole, "tail": trace_tail, "portions": trace_portions, "mixed": trace_mixed}
 # float32: the engine and the oracle differ by the order of float32 sums only.
 # bfloat16: activations between kernels are rounded to 8 bits of mantissa; logits of
