@@ -254,6 +254,28 @@ def test_prompt_portions_whose_keys_are_split_over_workgroups(nh, nkv, d, ps, se
     assert int((plan.prefill_items[:, 5] >= 0).sum()) > 0, "no block of rows was split"
 
 
+def test_a_requests_attention_has_the_same_bits_alone_and_beside_a_long_prompt(monkeypatch):
+    """With many tiles to combine the reduce runs as a kernel of 16-byte loads, with few as one thread
+    per element; both add a row's pieces in the same order, so a request's output does not change by
+    a bit when a long prompt joins the step."""
+    from wllm_amd.kernels import attention_plan
+    monkeypatch.setattr(attention_plan, "PREFILL_MIN_CHUNK", 128)
+    nh, nkv, d, ps = 8, 2, 64, 8
+    dtype = torch.bfloat16
+    args, kwargs = _attention_case(dtype, nh, nkv, d, ps, [(40, 700), (1, 600), (300, 900)], 0, seed=23)
+    both_kw = _with_plan(args, kwargs)
+    assert both_kw["plan"].num_reduce >= 64
+    ops.paged_attention(*args, **both_kw)
+    beside = args[7][:41].clone()
+    # the first two requests alone: the same rows of qkv, the same pages
+    alone = [args[0][:41].contiguous(), args[1], args[2][:2].contiguous(), args[3][:41].contiguous(),
+             args[4][:2].contiguous(), args[5][:2].contiguous(), args[6][:2].contiguous(), torch.zeros_like(args[7][:41])]
+    alone_kw = _with_plan(alone, dict(kwargs, max_q_len=40, max_ctx_len=700))
+    assert 0 < alone_kw["plan"].num_reduce < 64
+    ops.paged_attention(*alone, **alone_kw)
+    assert torch.equal(alone[7], beside)
+
+
 def _check_matrix_cores(nh, nkv, d, ps, segs, window):
     dtype = torch.bfloat16
     args, kwargs = _attention_case(dtype, nh, nkv, d, ps, segs, window, seed=11)

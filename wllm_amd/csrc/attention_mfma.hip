@@ -360,6 +360,64 @@ attention_reduce_kernel(const int* __restrict__ reduce_items, const float* __res
     out[(static_cast<size_t>(seg_q_start[seg] + tok) * num_heads + head) * HD + d] = from_float<bf16>(num / den);
 }
 
+// The same sums for steps with many tiles to combine (the pieces of a long prompt): a thread takes
+// four consecutive elements of a row (16-byte loads), a workgroup of HD threads four rows.  Every
+// element goes through the operations of the kernel above in the same order, so which of the two
+// runs changes no bit of the result.
+template <int HD>
+__global__ void __launch_bounds__(HD)
+attention_reduce_wide_kernel(const int* __restrict__ reduce_items, const float* __restrict__ partial_o,
+                             const float* __restrict__ partial_ml, const int* __restrict__ seg_q_start,
+                             const int* __restrict__ seg_q_len, bf16* __restrict__ out, int num_heads,
+                             int num_kv_heads, float scale_log2e) {
+    const int* item = reduce_items + static_cast<size_t>(blockIdx.x) * kItemInts;
+    const int seg = item[0], kvh = item[1], first = item[2], splits = item[3], row0 = item[4];
+    if (seg < 0) return;
+    const size_t stride = static_cast<size_t>(item[5]) * kRowsPerTile;     // rows between two splits
+    const int group = num_heads / num_kv_heads;
+    constexpr int kQuads = HD / 4;
+    const int r = blockIdx.y * 4 + threadIdx.x / kQuads, d = (threadIdx.x % kQuads) * 4;
+    if (row0 + r >= seg_q_len[seg] * group) return;
+    const float* ml = partial_ml + (static_cast<size_t>(first) * kRowsPerTile + r) * 2;
+    const float* po = partial_o + (static_cast<size_t>(first) * kRowsPerTile + r) * HD + d;
+    float m = -INFINITY, den = 0.f;
+    float4_t num = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < splits; s0 += 8) {
+        float ms[8], ls[8];
+        float4_t ps[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const bool ok = s0 + u < splits;
+            const size_t at = static_cast<size_t>(ok ? s0 + u : splits - 1) * stride;
+            const float2 pair = *reinterpret_cast<const float2*>(ml + at * 2);
+            ms[u] = ok ? pair.x : -INFINITY;
+            ls[u] = pair.y;
+            ps[u] = *reinterpret_cast<const float4_t*>(po + at * HD);
+        }
+        float m_new = m;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) m_new = fmaxf(m_new, ms[u]);
+        if (m_new == -INFINITY) continue;       // nothing seen yet
+        const float keep = m == -INFINITY ? 0.f : exp2f((m - m_new) * scale_log2e);
+        num *= keep;
+        den *= keep;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const float f = ms[u] == -INFINITY ? 0.f : exp2f((ms[u] - m_new) * scale_log2e);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) num[v] = fmaf(ps[u][v], f, num[v]);
+            den = fmaf(ls[u], f, den);
+        }
+        m = m_new;
+    }
+    const int row = row0 + r;
+    const int tok = row / group, head = kvh * group + row % group;
+    uint2 w;
+    w.x = pack2_bf16(num[0] / den, num[1] / den);
+    w.y = pack2_bf16(num[2] / den, num[3] / den);
+    *reinterpret_cast<uint2*>(out + (static_cast<size_t>(seg_q_start[seg] + tok) * num_heads + head) * HD + d) = w;
+}
+
 // Returns 0, a HIP error code, or -1 for sizes these kernels do not take.
 WLLM_API int wllm_paged_attention_mfma(const void* qkv, const void* cache, const int* block_tables, const int* items,
                                        int num_items, const int* reduce_items, int num_reduce_items,
@@ -377,9 +435,15 @@ WLLM_API int wllm_paged_attention_mfma(const void* qkv, const void* cache, const
         seg_ctx_len, static_cast<bf16*>(out), partial_o, partial_ml, num_heads, num_kv_heads, page_size, max_pages,  \
         scale_log2e, window)
 #define LAUNCH_R(HD)                                                                                                 \
-    attention_reduce_kernel<HD><<<dim3(num_reduce_items, kRowsPerTile), HD, 0, stream>>>(reduce_items, partial_o, partial_ml, seg_q_start, \
-                                                                      seg_q_len, static_cast<bf16*>(out), num_heads,  \
-                                                                      num_kv_heads, scale_log2e)
+    if (num_reduce_items >= 64) {                                                                                    \
+        attention_reduce_wide_kernel<HD><<<dim3(num_reduce_items, kRowsPerTile / 4), HD, 0, stream>>>(               \
+            reduce_items, partial_o, partial_ml, seg_q_start, seg_q_len, static_cast<bf16*>(out), num_heads,         \
+            num_kv_heads, scale_log2e);                                                                              \
+    } else {                                                                                                         \
+        attention_reduce_kernel<HD><<<dim3(num_reduce_items, kRowsPerTile), HD, 0, stream>>>(                        \
+            reduce_items, partial_o, partial_ml, seg_q_start, seg_q_len, static_cast<bf16*>(out), num_heads,         \
+            num_kv_heads, scale_log2e);                                                                              \
+    }
 #define CASE(HD)                                   \
     case HD:                                       \
         if (num_items > 0) {                       \
