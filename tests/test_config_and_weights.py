@@ -175,3 +175,11 @@ def test_missing_files_are_clear_errors(tmp_path):
     (tmp_path / "config.json").write_text(json.dumps(TINY["A"]["config"].to_dict()))
     with pytest.raises(WeightError, match="safetensors"):
         load_model(str(tmp_path), "float32", "cpu")
+
+
+def test_a_head_size_beyond_the_kernels_is_refused_when_the_model_is_built():
+    from wllm_amd.parts import build_model
+    c = TINY["A"]["config"].to_dict()
+    c["head_dim"] = 272
+    with pytest.raises(ValueError, match="head_dim 272"):
+        build_model(c)

@@ -19,6 +19,7 @@ from typing import Optional
 import torch
 
 _ACT = (torch.float32, torch.bfloat16)
+HEAD_DIM_STEP, MAX_HEAD_DIM = 4, 256      # what `paged_attention` takes: multiples of 4 up to 256
 _backend = None
 
 

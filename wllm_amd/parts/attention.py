@@ -32,6 +32,9 @@ class PagedAttention:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
         if spec.window is not None and spec.window <= 0:
             raise ValueError(f"window must be positive or None, got {spec.window}")
+        if spec.head_dim % ops.HEAD_DIM_STEP or not 0 < spec.head_dim <= ops.MAX_HEAD_DIM:
+            raise ValueError(f"head_dim {spec.head_dim}: the attention kernels take multiples of "
+                             f"{ops.HEAD_DIM_STEP} up to {ops.MAX_HEAD_DIM}")
         self.spec = spec
         self.position = build_position(spec.position)
         self.w_qkv = None
