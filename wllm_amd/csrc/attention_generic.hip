@@ -2,7 +2,7 @@
 // and grouping of heads, in float32 arithmetic throughout.  It is the kernel of the float32
 // path and of sizes the matrix-core kernels refuse.
 //
-// One workgroup (4 wavefronts) per (token, key/value head).  The token's position p follows
+// One workgroup (16 wavefronts) per (token, key/value head).  The token's position p follows
 // from its segment: p = ctx_len - q_len + i; it sees keys lo..p with lo = max(0, p - window + 1).
 // Each wavefront takes tiles of 64 consecutive keys: lane = key for the scores (a lane reads
 // its key's row of the page, [page_size, head_dim]), lane = element of the head for the
@@ -14,7 +14,7 @@
 #include "common.h"
 
 constexpr int kGroupMax = 8;     // query heads handled per pass over the keys
-constexpr int kWaves = 4;
+constexpr int kWaves = 16;      // a decode step has few (token, key/value head) pairs: many wavefronts each
 constexpr int kMaxHeadDim = 256;
 
 template <typename T> struct Vec4;
@@ -138,10 +138,11 @@ paged_attention_generic_kernel(const T* __restrict__ qkv, const T* __restrict__ 
         __builtin_amdgcn_wave_barrier();
     }
 
-    // merge the wavefronts: (m, l) per head and the accumulators through shared memory
+    // merge the wavefronts, in their order: (m, l) of all heads at once, the accumulators head by
+    // head through one buffer of [waves][head_dim]
     __syncthreads();
     float* ml_s = smem;                                              // [waves][g][2]
-    float* acc_s = smem + kWaves * kGroupMax * 2;                    // [waves][g][head_dim]
+    float* acc_s = smem + kWaves * kGroupMax * 2;                    // [waves][head_dim]
     if (lane == 0) {
 #pragma unroll
         for (int g = 0; g < kGroupMax; ++g) {
@@ -149,36 +150,36 @@ paged_attention_generic_kernel(const T* __restrict__ qkv, const T* __restrict__ 
             ml_s[(wave * kGroupMax + g) * 2 + 1] = l[g];
         }
     }
-#pragma unroll
-    for (int k = 0; k < DPL; ++k) {
-        const int d = lane + k * kWave;
-        if (d < head_dim) {
-#pragma unroll
-            for (int g = 0; g < kGroupMax; ++g)
-                if (g < g_count) acc_s[(wave * kGroupMax + g) * head_dim + d] = acc[g][k];
-        }
-    }
-    __syncthreads();
     T* orow = out + static_cast<size_t>(token) * num_heads * head_dim + static_cast<size_t>(kvh * group + group_begin) * head_dim;
-    for (int i = threadIdx.x; i < g_count * head_dim; i += blockDim.x) {
-        const int g = i / head_dim, d = i % head_dim;
-        float mm = -INFINITY;
-        for (int w = 0; w < kWaves; ++w) mm = fmaxf(mm, ml_s[(w * kGroupMax + g) * 2]);
-        float num = 0.f, den = 0.f;
-        for (int w = 0; w < kWaves; ++w) {
-            const float mw = ml_s[(w * kGroupMax + g) * 2];
-            const float f = mw == -INFINITY ? 0.f : expf(mw - mm);
-            num = fmaf(acc_s[(w * kGroupMax + g) * head_dim + d], f, num);
-            den = fmaf(ml_s[(w * kGroupMax + g) * 2 + 1], f, den);
+#pragma unroll
+    for (int g = 0; g < kGroupMax; ++g) {
+        if (g >= g_count) break;
+#pragma unroll
+        for (int k = 0; k < DPL; ++k) {
+            const int d = lane + k * kWave;
+            if (d < head_dim) acc_s[wave * head_dim + d] = acc[g][k];
         }
-        orow[i] = from_float<T>(num / den);
+        __syncthreads();
+        for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+            float mm = -INFINITY;
+            for (int w = 0; w < kWaves; ++w) mm = fmaxf(mm, ml_s[(w * kGroupMax + g) * 2]);
+            float num = 0.f, den = 0.f;
+            for (int w = 0; w < kWaves; ++w) {
+                const float mw = ml_s[(w * kGroupMax + g) * 2];
+                const float f = mw == -INFINITY ? 0.f : expf(mw - mm);
+                num = fmaf(acc_s[w * head_dim + d], f, num);
+                den = fmaf(ml_s[(w * kGroupMax + g) * 2 + 1], f, den);
+            }
+            orow[g * head_dim + d] = from_float<T>(num / den);
+        }
+        __syncthreads();
     }
 }
 
 static size_t generic_smem_bytes(int head_dim) {
     const size_t main_loop = sizeof(float) * (kGroupMax * head_dim + kWaves * kGroupMax * kWave) +
                              sizeof(long long) * kWaves * kWave + sizeof(int) * kWaves * kWave;
-    const size_t merge = sizeof(float) * (kWaves * kGroupMax * 2 + kWaves * kGroupMax * head_dim);
+    const size_t merge = sizeof(float) * (kWaves * kGroupMax * 2 + kWaves * head_dim);
     return main_loop > merge ? main_loop : merge;
 }
 
