@@ -87,15 +87,24 @@ paged_attention_generic_kernel(const T* __restrict__ qkv, const T* __restrict__ 
             slot = key % page_size;
             page_base = static_cast<long long>(page) * static_cast<long long>(page_elems);
             const T* krow = cache + page_base + k_off + static_cast<size_t>(slot) * head_dim;
-            for (int d = 0; d < head_dim; d += 4) {
-                Vec4<T> kv;
-                kv.v = *reinterpret_cast<const decltype(kv.v)*>(krow + d);
+            // four loads of the key's row are asked for before the first is used
+            for (int d0 = 0; d0 < head_dim; d0 += 16) {
+                Vec4<T> kv[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float kf = kv.get(e);
+                for (int u = 0; u < 4; ++u)
+                    kv[u].v = *reinterpret_cast<const decltype(kv[u].v)*>(krow + min(d0 + 4 * u, head_dim - 4));
 #pragma unroll
-                    for (int g = 0; g < kGroupMax; ++g)
-                        if (g < g_count) s[g] = fmaf(q_s[g * head_dim + d + e], kf, s[g]);
+                for (int u = 0; u < 4; ++u) {
+                    const int d = d0 + 4 * u;
+                    if (d < head_dim) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float kf = kv[u].get(e);
+#pragma unroll
+                            for (int g = 0; g < kGroupMax; ++g)
+                                if (g < g_count) s[g] = fmaf(q_s[g * head_dim + d + e], kf, s[g]);
+                        }
+                    }
                 }
             }
         }
@@ -125,11 +134,20 @@ paged_attention_generic_kernel(const T* __restrict__ qkv, const T* __restrict__ 
                 float a[kGroupMax];
 #pragma unroll
                 for (int g = 0; g < kGroupMax; ++g) a[g] = acc[g][k] * (g < g_count ? alpha[g] : 0.f);
-                for (int j = 0; j < keys_here; ++j) {
-                    const float vf = to_float(cache[koff_s[j] + v_off + static_cast<size_t>(d) * page_size + slot_s[j]]);
+                // eight keys' values are asked for before the first is used; beyond the tile's last
+                // key the last one is read again and meets a probability of zero
+                for (int j0 = 0; j0 < keys_here; j0 += 8) {
+                    float vf[8];
 #pragma unroll
-                    for (int g = 0; g < kGroupMax; ++g)
-                        if (g < g_count) a[g] = fmaf(p_s[g * kWave + j], vf, a[g]);
+                    for (int u = 0; u < 8; ++u) {
+                        const int j = min(j0 + u, keys_here - 1);
+                        vf[u] = to_float(cache[koff_s[j] + v_off + static_cast<size_t>(d) * page_size + slot_s[j]]);
+                    }
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+#pragma unroll
+                        for (int g = 0; g < kGroupMax; ++g)
+                            if (g < g_count) a[g] = fmaf(p_s[g * kWave + j0 + u], vf[u], a[g]);
                 }
 #pragma unroll
                 for (int g = 0; g < kGroupMax; ++g) acc[g][k] = a[g];
