@@ -26,9 +26,13 @@
 //   out^T[d, row] = V^T[d, keys] . P^T[keys, row]  A = V^T: lane (i, g) holds V^T[16t + i][8 keys of g]
 //                                                  B = P^T: the lane's own 8 probabilities of row_i
 // so every value a lane holds belongs to one query row, softmax needs two shuffles per tile, and the
-// probabilities feed the second product from the registers they were computed in.  Keys are read as
-// [page_size, head_dim] rows, values transposed as [head_dim, page_size] rows (16-byte loads when the
-// page size is a multiple of 8).  Scores, maxima, sums and accumulators are float32.
+// probabilities feed the second product from the registers they were computed in.  The cache holds
+// keys as [page_size, head_dim] rows and values transposed as [head_dim, page_size] rows.  Values are
+// loaded as fragments (16-byte loads when the page size is a multiple of 8: per instruction two runs
+// of 512 bytes).  Keys are loaded as whole rows, 16 bytes a lane in the order they lie in the page,
+// and become fragments in the wavefront's part of shared memory: a fragment load straight from the
+// cache asks for 64-byte pieces of 16 rows, a pattern the memory system serves more slowly.
+// Scores, maxima, sums and accumulators are float32.
 #include "common.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
