@@ -142,7 +142,8 @@ def run_stress(model, args) -> dict:
     runner = ModelRunner.create(model, num_pages=pages, page_size=args.block_size, max_requests=n)
     if not args.no_graphs:
         runner.enable_graphs()
-    sched = Scheduler(runner, max_prefill_tokens_per_step=512, seed=args.seed, lookahead=True)
+    sched = Scheduler(runner, max_prefill_tokens_per_step=512, seed=args.seed, lookahead=True,
+                      row_multiple=args.row_multiple or None)
     for i in range(n):
         ids = rng.integers(0, vocab, size=int(prompts[i])).tolist()
         sched.add_request(Request(i, ids, int(outputs[i]), sampling_params=SamplingParams(temperature=0.7, seed=1000 + i)))
@@ -182,6 +183,8 @@ def main() -> int:
     ap.add_argument("--workload", default="decode", choices=["decode", "stress"],
                     help="decode: the contract's line; stress: continuous batching of 64 mixed requests")
     ap.add_argument("--stress-requests", type=int, default=64)
+    ap.add_argument("--row-multiple", type=int, default=256,
+                    help="stress: a step's rows are trimmed to a multiple of this where the budget cuts a portion (0: off)")
     ap.add_argument("--stress-pool-fraction", type=float, default=0.5,
                     help="page pool as a fraction of what all requests together would need")
     args = ap.parse_args()

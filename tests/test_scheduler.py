@@ -361,3 +361,35 @@ def test_a_repetition_penalty_is_never_run_ahead(tiny):
             assert s._started is None, "a penalised request waits for its tokens"
         outs.append(r.output_token_ids)
     assert outs[0] == outs[1]
+
+
+def test_a_steps_rows_are_trimmed_to_the_products_tiles_where_the_budget_cuts_anyway(tiny):
+    """With `row_multiple`, a portion that the budget cuts is shortened so that the step's rows
+    (decoded tokens and prompt tokens) are a multiple of it; a portion that ends its prompt is not,
+    and the tokens are the same either way."""
+    model, cfg, w = tiny
+    prompts = prompts_of([5, 6, 7, 90])
+    outs = {}
+    for multiple in (None, 8):
+        s = make(model, num_pages=96, max_prefill_tokens_per_step=16, row_multiple=multiple)
+        seen = []
+        real_step = s.runner.step
+        s.runner.step = lambda entries, *a, real=real_step, log=seen: (
+            log.append([len(e.tokens) for e in entries]), real(entries, *a))[1]
+        for i, p in enumerate(prompts[:3]):
+            s.add_request(Request(i, p, 30))
+        s.step()
+        s.step()                                    # three requests decode
+        s.add_request(Request(3, prompts[3], 4))
+        done = s.run_to_completion()
+        outs[multiple] = {r.request_id: r.output_token_ids for r in done}
+        mixed = [b for b in seen if max(b) > 1 and b.count(1) == 3]
+        assert mixed, "portions of the long prompt ran beside three decoded tokens"
+        if multiple is None:
+            assert mixed[0] == [1, 1, 1, 16]
+        else:
+            # 3 + 16 rows would be 19: the portion gives 3 up; the last portion (90 = 13 * 6 + 12) ends
+            # the prompt and is left alone
+            assert mixed[0] == [1, 1, 1, 13] and all(sum(b) % 8 == 0 for b in mixed[:-1])
+            assert sum(b[-1] for b in mixed) == 90 and sum(mixed[-1]) % 8 != 0
+    assert outs[None] == outs[8]

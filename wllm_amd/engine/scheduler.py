@@ -62,7 +62,8 @@ class _StartedStep:
 
 class Scheduler:
     def __init__(self, runner, max_prefill_tokens_per_step: Optional[int] = None, admission: str = "pledged",
-                 seed: int = 0, compute_logprobs: bool = True, lookahead: bool = False):
+                 seed: int = 0, compute_logprobs: bool = True, lookahead: bool = False,
+                 row_multiple: Optional[int] = None):
         if admission not in ("pledged", "prompt_only"):
             raise ValueError(f"admission {admission!r}: expected 'pledged' or 'prompt_only'")
         if max_prefill_tokens_per_step is not None and max_prefill_tokens_per_step <= 0:
@@ -70,6 +71,10 @@ class Scheduler:
         self.runner = runner
         self.cache = runner.cache
         self.max_prefill_tokens_per_step = max_prefill_tokens_per_step
+        # A step's rows (decoded tokens and prompt tokens) are trimmed to a multiple of this where a
+        # portion is cut by the budget anyway: the library's products of many rows work in tiles of
+        # rows, and a step of 530 rows costs as much as one of 768.
+        self.row_multiple = row_multiple
         self.admission = admission
         self.compute_logprobs = compute_logprobs
         self.sampler = Sampler(runner.device, seed)
@@ -183,6 +188,13 @@ class Scheduler:
             plan.append((r, take))
             if not unlimited:
                 budget -= take
+        if self.row_multiple and not unlimited and plan:
+            rows = sum(n for _, n in plan)
+            extra = rows % self.row_multiple
+            r, take = plan[-1]
+            cut_by_budget = r.status == RequestStatus.PREFILLING and r.num_tokens - r.num_computed > take
+            if rows > self.row_multiple and extra and cut_by_budget and take - extra >= max(2, take // 2):
+                plan[-1] = (r, take - extra)
         return plan
 
     def _preempt(self, request: Request) -> None:
