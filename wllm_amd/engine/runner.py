@@ -39,7 +39,7 @@ class ModelRunner:
         self.dummy_pages: list = []
         self.graph_steps = 0
 
-    def enable_graphs(self, buckets=(1, 2, 4, 8, 16, 32, 64, 128, 256), max_context=None) -> None:
+    def enable_graphs(self, buckets=(1, 2, 4, 8, 16, 32, 48, 64, 128, 256), max_context=None) -> None:
         """Decode-only steps of up to max(buckets) requests replay a captured graph of the
         smallest bucket that holds them; the largest number of requests the cache admits, if it
         is below max(buckets), is a bucket too, so that a full batch of any size has its graph.
