@@ -149,6 +149,26 @@ def test_trace_run_program(model_folders, tmp_path, dtype):
         assert ((got.double() - ref.double()).abs() <= atol + rtol * ref.double().abs()).all(), f"step {step}"
 
 
+def test_trace_run_says_when_a_trace_holds_more_than_max_tokens(model_folders, tmp_path):
+    """Two live requests of 100 tokens against --max-tokens 128: one line that names the step and
+    the limit, a non-zero exit, and the steps before it done."""
+    folder = model_folders["A"]
+    a, b = random_ids(3, 100, 512), random_ids(4, 100, 512)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a, "want": [99]}], "end": []},
+        {"step": 1, "entries": [{"id": "b", "tokens": b, "want": [99]}], "end": ["a", "b"]},
+    ]
+    out = tmp_path / "out"
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
+                           "--out", str(out), "--max-tokens", "128"],
+                          input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert proc.returncode != 0
+    assert proc.stdout.split() == ["done", "0"]
+    assert "step 1" in proc.stderr and "--max-tokens 128" in proc.stderr
+    assert "Traceback" not in proc.stderr
+    assert (out / "0.f32").exists() and not (out / "1.f32").exists()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_captured_graphs_give_what_eager_steps_give(model_folders, dtype):
     """Decode steps replayed from captured graphs against the same steps run kernel by kernel:
