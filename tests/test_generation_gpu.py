@@ -26,7 +26,7 @@ def plain_model(folder):
 
 @pytest.mark.parametrize("name,lengths,new", [("A", [7, 16, 23], 8), ("B", [5, 31, 64], 6), ("C", [9, 20], 6), ("M", [33, 70], 6)])
 def test_greedy_generation_through_the_entry_point_float32(model_folders, name, lengths, new):
-    # BASELINE's tiny workload: prompts of 7/16/23 ids, 8 greedy tokens each, pages of 4
+    # the first case is a tiny workload of its own: prompts of 7/16/23 ids, 8 greedy tokens each, pages of 4
     cfg, w = plain_model(model_folders[name])
     prompts = [random_ids(i + 1, n, cfg["vocab_size"]) for i, n in enumerate(lengths)]
     llm = LLM(model_folders[name], dtype="float32", num_blocks=64, block_size=TINY[name]["page_size"])
@@ -58,7 +58,7 @@ def test_greedy_generation_bfloat16_follows_the_plain_implementation_up_to_near_
 
 
 def test_chunked_prefill_beside_decodes_with_seeded_temperature(model_folders):
-    """BASELINE's second tiny workload: four prompts of 5/31/64/97 ids, portions of 16 beside
+    """A second tiny workload: four prompts of 5/31/64/97 ids, portions of 16 beside
     decoding requests, temperature 0.8 from a seeded generator, pages of 8.  Each request's tokens
     equal those it gets alone, and each token is one the plain implementation's distribution gives
     the request's uniform number."""
