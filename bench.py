@@ -228,6 +228,11 @@ def main() -> int:
             for b, k in ((1, args.steps), (64, max(8, args.steps // 2))):
                 d, _ = measure_decode(model, b, args.context, k, min(args.warmup, 4), args.block_size, graphs)
                 points[f"decode_b{b}"] = round(k * b / d, 1)
+            # the same batch near the longest context the configuration allows
+            long_context = model.config.max_position_embeddings - 1024
+            if long_context > args.context:
+                d, _ = measure_decode(model, args.batch, long_context, args.steps, min(args.warmup, 4), args.block_size, graphs)
+                points[f"decode_b{args.batch}_context_{long_context}"] = round(args.steps * args.batch / d, 1)
 
     c = model.config
     sizes = {"gemma-2b": "Gemma-2B", "gemma-7b": "Gemma-7B"}.get(args.shape, os.path.basename(args.shape))
