@@ -159,3 +159,24 @@ def test_a_row_spread_over_workgroups_draws_what_one_workgroup_draws(vocab):
     finally:
         be.SAMPLE_SPLIT_ROWS = limit
     assert a == b
+
+
+def test_starting_a_sampling_does_not_wait_for_the_gpu():
+    """`Sampler.start` only enqueues: behind a tenth of a second of queued products it returns
+    while they still run (its per-row numbers travel from page-locked memory), and what it then
+    gives is what a sampling of its own gives."""
+    torch.manual_seed(5)
+    logits = torch.randn(6, 3000, device=DEV)
+    params = [SamplingParams(temperature=0.8, top_k=40, repetition_penalty=1.3 if i % 2 else 1.0, seed=i) for i in range(6)]
+    generated = [[i, 2 * i + 1, 17] for i in range(6)]
+    sampler = Sampler(DEV)
+    expect = sampler.sample(logits.clone(), params, list(range(6)), [3] * 6, generated)
+    big = torch.randn(8192, 8192, device=DEV)
+    torch.cuda.synchronize()
+    for _ in range(12):
+        big @ big
+    queued = torch.cuda.Event()
+    queued.record()
+    pending = sampler.start(logits.clone(), params, list(range(6)), [3] * 6, generated)
+    assert not queued.query(), "start came back only after the work queued before it had run"
+    assert Sampler.finish(pending) == expect

@@ -128,22 +128,3 @@ class StepContext:
         """[max_requests, *shape] float32 state of a schedule entry; row state_slots[s]
         belongs to segment s."""
         return self._cache.state.get(entry)
-
-
-def pack_int32(arrays: list, device, pinned: Optional[torch.Tensor] = None):
-    """Concatenates int32 arrays, copies them to the device at once and returns the
-    device views in order."""
-    sizes = [a.size for a in arrays]
-    total = sum(sizes)
-    host = torch.empty(max(total, 1), dtype=torch.int32, pin_memory=(torch.device(device).type == "cuda"))
-    buf = host.numpy()
-    o = 0
-    for a, s in zip(arrays, sizes):
-        buf[o:o + s] = a.reshape(-1)
-        o += s
-    dev = host.to(device, non_blocking=True)
-    views, o = [], 0
-    for a, s in zip(arrays, sizes):
-        views.append(dev[o:o + s].view(a.shape))
-        o += s
-    return views

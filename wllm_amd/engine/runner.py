@@ -17,8 +17,9 @@ import torch
 
 from wllm_amd.cache.manager import CacheManager
 from wllm_amd.cache.pages import OutOfPages
-from wllm_amd.engine.batch import StepContext, StepEntry, Workspace, pack_int32
+from wllm_amd.engine.batch import StepContext, StepEntry, Workspace
 from wllm_amd.kernels import ops
+from wllm_amd.kernels.staging import pack_int32
 
 
 class StepError(ValueError):

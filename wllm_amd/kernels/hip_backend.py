@@ -11,6 +11,7 @@ import torch
 
 from wllm_amd.kernels.attention_plan import AttentionPlan, build_work_items
 from wllm_amd.kernels.library import load
+from wllm_amd.kernels.staging import pack_int32
 
 
 class KernelError(RuntimeError):
@@ -167,7 +168,7 @@ class HipBackend:
         items, reduces, slots, prefill, prefill_rows = build_work_items(
             host_q_len, host_ctx_len, num_heads // num_kv_heads, num_kv_heads, window, fixed_splits, page_size)
         flat = np.concatenate([items.reshape(-1), reduces.reshape(-1), prefill.reshape(-1)])
-        dev = torch.from_numpy(flat).to(device, non_blocking=True)
+        dev = pack_int32([flat], device)[0]
         n_i, n_r, n_p = items.shape[0], reduces.shape[0], prefill.shape[0]
         self._ensure_partials(slots, head_dim, device)
         a, b = n_i * 8, (n_i + n_r) * 8

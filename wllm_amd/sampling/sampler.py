@@ -15,6 +15,7 @@ import numpy as np
 import torch
 
 from wllm_amd.kernels import ops
+from wllm_amd.kernels.staging import pack_words
 from wllm_amd.sampling.params import SamplingParams
 
 
@@ -54,7 +55,9 @@ class Sampler:
         table = np.array([[p.temperature, p.top_k, p.top_p, p.min_p, p.repetition_penalty] for p in params],
                          dtype=np.float32)
         keys = np.array([[s, c] for s, c in zip(seeds, counters)], dtype=np.int64)
-        pen_ids = pen_off = None
+        # one copy from page-locked memory carries every per-row number, so the host goes on while
+        # the step's kernels still run
+        arrays = [keys, table]
         if generated is not None and any(p.repetition_penalty != 1.0 for p in params):
             # the penalty applies once per distinct generated id (sampling.py:55)
             lists = [sorted(set(g)) if p.repetition_penalty != 1.0 else [] for g, p in zip(generated, params)]
@@ -62,12 +65,12 @@ class Sampler:
             offsets[1:] = np.cumsum([len(x) for x in lists])
             flat = np.array([t for x in lists for t in x], dtype=np.int32)
             if flat.size:
-                pen_ids = torch.from_numpy(flat).to(logits.device)
-                pen_off = torch.from_numpy(offsets).to(logits.device)
+                arrays += [flat, offsets]
+        on_device = pack_words(arrays, logits.device)
+        pen_ids, pen_off = (on_device[2], on_device[3]) if len(on_device) == 4 else (None, None)
         logprobs = torch.empty(m, dtype=torch.float32, device=logits.device)
         truncations = any(not p.greedy and (p.top_k > 0 or p.top_p < 1.0) for p in params)
-        ops.sample_rows(logits, torch.from_numpy(table).to(logits.device), torch.from_numpy(keys).to(logits.device),
-                        pen_ids, pen_off, tokens, logprobs, truncations=truncations)
+        ops.sample_rows(logits, on_device[1], on_device[0], pen_ids, pen_off, tokens, logprobs, truncations=truncations)
         return PendingSample(tokens, logprobs)
 
     @staticmethod
