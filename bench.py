@@ -229,7 +229,9 @@ def main() -> int:
                 d, _ = measure_decode(model, b, args.context, k, min(args.warmup, 4), args.block_size, graphs)
                 points[f"decode_b{b}"] = round(k * b / d, 1)
             # the same batch near the longest context the configuration allows
-            long_context = model.config.max_position_embeddings - 1024
+            limit = model.config.max_position_embeddings
+            new_tokens = args.batch * (-(-limit // 2048)) + args.warmup + args.steps + 2      # as `measure_decode` counts them
+            long_context = min(limit - 1024, (limit - new_tokens) // 256 * 256)
             if long_context > args.context:
                 d, _ = measure_decode(model, args.batch, long_context, args.steps, min(args.warmup, 4), args.block_size, graphs)
                 points[f"decode_b{args.batch}_context_{long_context}"] = round(args.steps * args.batch / d, 1)
