@@ -32,3 +32,11 @@ def model_folders(tmp_path_factory):
     from helpers import TINY, write_tiny
     root = tmp_path_factory.mktemp("models")
     return {name: write_tiny(name, str(root / name)) for name in TINY}
+
+
+@pytest.fixture(scope="session")
+def varied_folders(tmp_path_factory):
+    """Model folders of the configurations whose greedy continuation varies."""
+    from helpers import VARIED, write_tiny
+    root = tmp_path_factory.mktemp("varied_models")
+    return {name: write_tiny(name, str(root / name)) for name in VARIED}

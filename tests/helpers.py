@@ -37,9 +37,54 @@ TINY = {
 }
 
 
+# Greedy decoding of the configurations above repeats the last prompt token for ever: with weights
+# this small the tied head's logit of a token for itself beats everything the context adds.  Tests
+# that compare generated tokens use these instead: the same sizes with weights large enough that
+# the context decides, so that a wrong key, page or position changes the tokens.
+VARIED = {"AV": dict(TINY["A"], std=0.3), "MV": dict(TINY["M"], std=0.3)}
+
+
+def assert_varied(tokens: list, least: int = 4) -> None:
+    """The generated tokens are not one token repeated (a test of token equality would be empty)."""
+    assert len(set(tokens)) >= min(least, len(tokens)), f"the generated tokens hardly vary: {tokens}"
+
+
 def write_tiny(name: str, folder: str) -> str:
-    t = TINY[name]
+    t = TINY[name] if name in TINY else VARIED[name]
     return write_random_model_folder(folder, t["config"], t["seed"], std=t["std"], norm_std=t["norm_std"])
+
+
+def degenerate_folder(src: str, out: str, kind: str) -> str:
+    """A copy of a model folder with some weights set to zero, so that the logits reduce to a formula
+    a test writes out by hand (through the framework's safetensors writer, not the model):
+    "no_contributions": every o_proj and down_proj zero and the layers' norm weights zero, so each
+        layer adds nothing: logits = final_norm(E[ids] * sqrt(H)) @ head^T;
+    "one_feed_forward": as above, but layer 0's down_proj and post-attention norm weight are kept:
+        logits = final_norm(x + mlp(norm(x))) @ head^T with x = E[ids] * sqrt(H);
+    "bias_only_queries_and_keys": q_proj and k_proj weights zero (the folder must have biases): queries
+        and keys are the rotated biases."""
+    import os
+    from wllm_amd.weights import Checkpoint, write_safetensors
+    ck = Checkpoint(src)
+    tensors = {n: ck.tensor(n).clone() for n in ck.names()}
+    ck.close()
+    for n, t in tensors.items():
+        if kind in ("no_contributions", "one_feed_forward"):
+            keep = kind == "one_feed_forward" and ".layers.0." in n
+            if n.endswith("o_proj.weight") or (n.endswith("down_proj.weight") and not keep):
+                t.zero_()
+            if n.endswith("input_layernorm.weight") or (n.endswith("post_attention_layernorm.weight") and not keep):
+                t.zero_()
+        elif kind == "bias_only_queries_and_keys":
+            if n.endswith(("q_proj.weight", "k_proj.weight")):
+                t.zero_()
+        else:
+            raise ValueError(kind)
+    os.makedirs(out, exist_ok=True)
+    write_safetensors(os.path.join(out, "model.safetensors"), tensors)
+    with open(os.path.join(src, "config.json")) as f, open(os.path.join(out, "config.json"), "w") as g:
+        g.write(f.read())
+    return out
 
 
 def random_ids(seed: int, length: int, vocab: int) -> list:

@@ -183,3 +183,30 @@ def test_a_head_size_beyond_the_kernels_is_refused_when_the_model_is_built():
     c["head_dim"] = 272
     with pytest.raises(ValueError, match="head_dim 272"):
         build_model(c)
+
+
+def test_the_index_file_names_files_of_its_own_folder_only(model_folders, tmp_path):
+    """model.safetensors.index.json belongs to a folder that may come from anywhere: a weight_map
+    entry that is absolute, climbs out of the folder or is no .safetensors file is refused; a plain
+    name is honoured (two shards, loaded as one checkpoint)."""
+    src = Checkpoint(model_folders["A"])
+    tensors = {n: src.tensor(n) for n in src.names()}
+    src.close()
+    names = sorted(tensors)
+    folder = tmp_path / "sharded"
+    folder.mkdir()
+    halves = {"part-1.safetensors": names[:5], "part-2.safetensors": names[5:]}
+    for file, part in halves.items():
+        write_safetensors(str(folder / file), {n: tensors[n] for n in part})
+    (folder / "config.json").write_text(json.dumps(TINY["A"]["config"].to_dict()))
+    (folder / "model.safetensors.index.json").write_text(
+        json.dumps({"weight_map": {n: file for file, part in halves.items() for n in part}}))
+    ck = Checkpoint(str(folder))
+    assert sorted(ck.names()) == names and torch.equal(ck.tensor(names[7]), tensors[names[7]])
+    ck.close()
+    outside = tmp_path / "outside.safetensors"
+    write_safetensors(str(outside), {"x": torch.zeros(1)})
+    for bad in (str(outside), "../outside.safetensors", "sub/part-1.safetensors", "config.json"):
+        (folder / "model.safetensors.index.json").write_text(json.dumps({"weight_map": {"x": bad}}))
+        with pytest.raises(WeightError, match="weight_map"):
+            Checkpoint(str(folder))

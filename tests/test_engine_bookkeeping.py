@@ -78,3 +78,48 @@ def test_partial_sums_of_split_products_reach_the_consumers(model_folders, plain
                                     max_requests=4)
         got = replay_and_collect(TraceReplayer(runner), trace)
     compare_with_plain(got, plain_logits["C"], atol=2e-5, rtol=1e-4)
+
+
+def test_the_garbage_collector_is_off_while_a_graph_is_captured(monkeypatch):
+    """A collector run inside a capture that frees an object with device resources aborts the
+    process; `capture` switches the collector off for the capture and back on after it, also when
+    the captured body raises, and leaves it off if it was off."""
+    import contextlib
+    import gc
+
+    from wllm_amd.engine import graphs
+
+    seen = []
+
+    class StandInGraph:
+        pass
+
+    @contextlib.contextmanager
+    def stand_in_capture(graph):
+        assert isinstance(graph, StandInGraph)
+        seen.append(("enter", gc.isenabled()))
+        yield
+        seen.append(("exit", gc.isenabled()))
+
+    monkeypatch.setattr(torch.cuda, "CUDAGraph", StandInGraph)
+    monkeypatch.setattr(torch.cuda, "graph", stand_in_capture)
+    assert gc.isenabled()
+
+    graph, result = graphs.capture(lambda: (seen.append(("body", gc.isenabled())), 42)[1])
+    assert isinstance(graph, StandInGraph) and result == 42
+    assert seen == [("enter", False), ("body", False), ("exit", False)] and gc.isenabled()
+
+    def failing():
+        assert not gc.isenabled()
+        raise KeyError("inside the capture")
+
+    with pytest.raises(KeyError):
+        graphs.capture(failing)
+    assert gc.isenabled(), "switched back on after a body that raised"
+
+    gc.disable()
+    try:
+        graphs.capture(lambda: None)
+        assert not gc.isenabled(), "a collector that was off stays off"
+    finally:
+        gc.enable()

@@ -104,3 +104,26 @@ def test_sharp_attention_over_hundreds_of_keys(model_folders, tmp_path_factory, 
         runner = ModelRunner.create(model, num_pages=pages, page_size=16, max_requests=4, poison_freed_pages=True)
         got = replay_and_collect(TraceReplayer(runner), trace)
         compare_with_plain(got, plain, **tol)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,kind", [("A", "no_contributions"), ("C", "no_contributions"), ("A", "one_feed_forward"),
+                                       ("B", "one_feed_forward"), ("C", "bias_only_queries_and_keys")])
+def test_models_whose_logits_a_formula_gives(model_folders, tmp_path, name, kind, dtype):
+    """The folders that pin the plain implementation's wiring (layers that contribute nothing; one
+    feed-forward alone; queries and keys that are rotated biases), through the engine: whole prompts,
+    the last tokens one by one, and portions."""
+    from helpers import degenerate_folder
+    folder = degenerate_folder(model_folders[name], str(tmp_path / kind), kind)
+    cfg = gemma_plain.read_config(folder)
+    w = gemma_plain.read_weights(folder, torch.float32)
+    requests = {f"r{i}": random_ids(7 * i + 1, n, cfg["vocab_size"]) for i, n in enumerate([21, 40])}
+    rounding = torch.bfloat16 if dtype == "bfloat16" else None
+    plain = {rid: gemma_plain.forward_logits(cfg, w, t, scale_rounding=rounding) for rid, t in requests.items()}
+    model = load_model(folder, dtype, "cuda")
+    page_size = TINY[name]["page_size"]
+    for family in (trace_whole, lambda r: trace_tail(r, tail=8), trace_portions):
+        trace = family(requests)
+        runner = ModelRunner.create(model, num_pages=pages_for_max_tokens(max_live_tokens(trace), page_size),
+                                    page_size=page_size, max_requests=4, poison_freed_pages=True)
+        compare_with_plain(replay_and_collect(TraceReplayer(runner), trace), plain, **TOLERANCE[dtype])

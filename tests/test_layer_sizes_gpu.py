@@ -5,14 +5,16 @@ vocabulary so that the plain implementation stays fast.  The prompts are long en
 attention's work to be cut along the keys (several pieces of 128 keys in decode steps, a late
 portion of a prompt split over workgroups).
 
-float32 is held to the tolerance of the tiny configurations.  In bfloat16 an activation of these
+float32 is held to the tolerance of the tiny configurations.  The bfloat16 bound here is a second line
+behind the tiny configurations' element-wise one: it shows a wrong page, key or head, not a rounding
+made at another point than the plain implementation makes it.  In bfloat16 an activation of these
 widths is the sum of thousands of rounded terms, so single logits stray further than in the tiny
 models; the measure is each position's error against the length of its logits vector, which a
 missed key, a wrong page or a wrong head would raise to the order of one."""
 import pytest
 import torch
 
-from helpers import max_live_tokens, random_ids, replay_and_collect, trace_mixed, trace_tail, trace_whole
+from helpers import max_live_tokens, random_ids, replay_and_collect, trace_mixed, trace_portions, trace_tail, trace_whole
 from plain import gemma_plain
 from wllm_amd.config import GemmaConfig
 from wllm_amd.engine import ModelRunner
@@ -66,7 +68,7 @@ def test_layer_sizes_of_the_measured_models(folders, plain_logits, name, dtype):
     requests = _requests(name)
     plain = plain_logits[name][torch.bfloat16 if dtype == "bfloat16" else None]
     model = load_model(folders[name], dtype, "cuda")
-    for family in (trace_whole, trace_tail, trace_mixed):
+    for family in (trace_whole, trace_tail, trace_portions, trace_mixed):
         trace = family(requests)
         pages = pages_for_max_tokens(max_live_tokens(trace), PAGE_SIZE)
         runner = ModelRunner.create(model, num_pages=pages, page_size=PAGE_SIZE, max_requests=4, poison_freed_pages=True)

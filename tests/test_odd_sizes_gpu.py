@@ -1,12 +1,13 @@
 """Sizes the tiny configurations of the other tests do not have: head sizes in steps of 16 from 16
 to 144, widths and inner sizes that are no multiple of 32 (or of 4), an odd vocabulary, pages of
 4 to 32 tokens.  Whatever kernel a size selects, or refuses so that a general one runs, the
-logits follow the plain implementation: whole prompts, the last tokens one by one, and mixed
-portions with pages handed out again, in float32 and in bfloat16."""
+logits follow the plain implementation: whole prompts, the last tokens one by one, portions of
+changing size, and mixed portions with pages handed out again, in float32 and in bfloat16."""
 import pytest
 import torch
 
-from helpers import compare_with_plain, max_live_tokens, random_ids, replay_and_collect, trace_mixed, trace_tail, trace_whole
+from helpers import (compare_with_plain, max_live_tokens, random_ids, replay_and_collect, trace_mixed, trace_portions,
+                     trace_tail, trace_whole)
 from plain import gemma_plain
 from wllm_amd.config import GemmaConfig
 from wllm_amd.engine import ModelRunner
@@ -53,7 +54,7 @@ def test_odd_sizes_follow_the_plain_implementation(folders, name, dtype):
     plain = {rid: gemma_plain.forward_logits(plain_cfg, weights, toks, scale_rounding=rounding)
              for rid, toks in requests.items()}
     model = load_model(folders[name], dtype, "cuda")
-    for family in (trace_whole, trace_tail, trace_mixed):
+    for family in (trace_whole, trace_tail, trace_portions, trace_mixed):
         trace = family(requests)
         pages = pages_for_max_tokens(max_live_tokens(trace), page_size)
         runner = ModelRunner.create(model, num_pages=pages, page_size=page_size, max_requests=4,

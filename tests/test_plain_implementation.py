@@ -161,16 +161,97 @@ def test_logits_do_not_change_when_all_positions_move(model_folders, name):
     assert torch.allclose(a, b, atol=1e-9)
 
 
-def test_logits_are_causal_and_the_head_is_the_unscaled_table(model_folders):
+def test_logits_are_causal(model_folders):
     cfg = P.read_config(model_folders["A"])
     w = P.read_weights(model_folders["A"], torch.float64)
     ids = torch.randint(0, cfg["vocab_size"], (10,))
     full = P.forward_logits(cfg, w, ids)
     assert torch.allclose(P.forward_logits(cfg, w, ids[:6]), full[:6], atol=1e-10)
-    # doubling the table doubles the logits through the head but not through the (normalised) body
-    w2 = dict(w)
-    w2["model.embed_tokens.weight"] = w["model.embed_tokens.weight"] * 2
-    assert not torch.allclose(P.forward_logits(cfg, w2, ids), full, atol=1e-3)
+
+
+def _hand_norm(x, w, eps):
+    return x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * (1.0 + w)
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_layers_that_contribute_nothing_leave_one_final_norm_and_the_unscaled_head(model_folders, tmp_path, name):
+    """Every o_proj and down_proj zero: each layer must hand its input on unchanged (the residual
+    path, src/wllm/models/gemma.py:83-93), so logits = norm_f(E[ids] * sqrt(H)) @ head^T with exactly
+    one final norm (src/wllm/models/llama.py:415) and, when tied, the table as it is stored
+    (llama.py:443-446).  A head scaled like the embedding is off by sqrt(H); a second final norm, or
+    one left out, changes the (1 + w) factor; a layer that normalises the stream itself changes x."""
+    from helpers import degenerate_folder
+    folder = degenerate_folder(model_folders[name], str(tmp_path / "none"), "no_contributions")
+    cfg = P.read_config(folder)
+    w = P.read_weights(folder, torch.float64)
+    ids = torch.randint(0, cfg["vocab_size"], (9,))
+    table = w["model.embed_tokens.weight"]
+    x = table[ids] * math.sqrt(cfg["hidden_size"])
+    head = table if cfg["tie_word_embeddings"] else w["lm_head.weight"]
+    expected = _hand_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"]) @ head.T
+    got = P.forward_logits(cfg, w, ids)
+    assert torch.allclose(got, expected, atol=1e-10)
+    # the plausible mistakes are far away: a head scaled like the embedding, no final norm, two of them
+    assert not torch.allclose(got, expected * math.sqrt(cfg["hidden_size"]), atol=1e-3)
+    assert not torch.allclose(got, x @ head.T, atol=1e-3)
+    twice = _hand_norm(_hand_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"]), w["model.norm.weight"], cfg["rms_norm_eps"])
+    assert not torch.allclose(got, twice @ head.T, atol=1e-3)
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_one_feed_forward_is_added_to_the_stream_it_read_through_a_norm(model_folders, tmp_path, name):
+    """Only layer 0's feed-forward contributes: logits = norm_f(x + mlp(norm_2(x))) @ E^T, x = E[ids] * sqrt(H)
+    (src/wllm/models/gemma.py:89-93): the feed-forward reads the normalised stream and is added to the
+    stream as it was, not to its normalised copy, and nothing is normalised after the sum but the
+    final norm."""
+    from helpers import degenerate_folder
+    folder = degenerate_folder(model_folders[name], str(tmp_path / "one"), "one_feed_forward")
+    cfg = P.read_config(folder)
+    w = P.read_weights(folder, torch.float64)
+    ids = torch.randint(0, cfg["vocab_size"], (7,))
+    eps, p = cfg["rms_norm_eps"], "model.layers.0."
+    x = w["model.embed_tokens.weight"][ids] * math.sqrt(cfg["hidden_size"])
+    h = _hand_norm(x, w[p + "post_attention_layernorm.weight"], eps)
+    gate, up = h @ w[p + "mlp.gate_proj.weight"].T, h @ w[p + "mlp.up_proj.weight"].T
+    mlp = (torch.nn.functional.gelu(gate, approximate="tanh") * up) @ w[p + "mlp.down_proj.weight"].T
+    assert mlp.abs().max() > 1e-3 * x.abs().max(), "the feed-forward matters in this test"
+    expected = _hand_norm(x + mlp, w["model.norm.weight"], eps) @ w["model.embed_tokens.weight"].T
+    got = P.forward_logits(cfg, w, ids)
+    assert torch.allclose(got, expected, atol=1e-10)
+    # post-norm wiring (the sum normalised, or the feed-forward added to the normalised copy) is far away
+    assert not torch.allclose(got, _hand_norm(h + mlp, w["model.norm.weight"], eps) @ w["model.embed_tokens.weight"].T, atol=1e-3)
+    unnormed = (torch.nn.functional.gelu(x @ w[p + "mlp.gate_proj.weight"].T, approximate="tanh")
+                * (x @ w[p + "mlp.up_proj.weight"].T)) @ w[p + "mlp.down_proj.weight"].T
+    assert not torch.allclose(got, _hand_norm(x + unnormed, w["model.norm.weight"], eps) @ w["model.embed_tokens.weight"].T, atol=1e-3)
+
+
+def test_biases_are_added_before_the_rotation():
+    """q_proj and k_proj weights zero, biases b_q and b_k: the query at position p is rope(b_q, p) and the
+    key at s is rope(b_k, s) (src/wllm/models/llama.py:95-98,103-110: the Linear with its bias, then
+    apply_rotary_pos_emb), so the scores depend on p - s.  Added after the rotation the biases would
+    give every key of a head the same score and the output the running mean of v."""
+    torch.manual_seed(3)
+    T, nh, nkv, d, H = 9, 4, 2, 8, 12
+    cfg = dict(num_attention_heads=nh, num_key_value_heads=nkv, head_dim=d, attention_bias=True)
+    w = {"q_proj.weight": torch.zeros(nh * d, H, dtype=torch.float64), "k_proj.weight": torch.zeros(nkv * d, H, dtype=torch.float64),
+         "v_proj.weight": torch.randn(nkv * d, H, dtype=torch.float64), "o_proj.weight": torch.eye(nh * d, dtype=torch.float64),
+         "q_proj.bias": torch.randn(nh * d, dtype=torch.float64) * 2, "k_proj.bias": torch.randn(nkv * d, dtype=torch.float64) * 2,
+         "v_proj.bias": torch.zeros(nkv * d, dtype=torch.float64)}
+    h = torch.randn(T, H, dtype=torch.float64)
+    cos, sin = P.rope_cos_sin(torch.arange(T), d, 100.0, torch.float64)
+    got = P.attention_block(h, w, "", cfg, cos, sin).view(T, nh, d)
+    v = (h @ w["v_proj.weight"].T).view(T, nkv, d)
+    # by hand: the rotated biases as queries and keys, one head and one position at a time
+    for head in range(nh):
+        kv = head // (nh // nkv)
+        for p in range(T):
+            q = P.apply_rope(w["q_proj.bias"].view(1, nh, d), cos[p:p + 1], sin[p:p + 1])[0, head]
+            keys = torch.stack([P.apply_rope(w["k_proj.bias"].view(1, nkv, d), cos[s:s + 1], sin[s:s + 1])[0, kv]
+                                for s in range(p + 1)])
+            probs = torch.softmax(keys @ q / math.sqrt(d), -1)
+            assert torch.allclose(got[p, head], probs @ v[:p + 1, kv], atol=1e-12)
+    running_mean = v.cumsum(0) / torch.arange(1, T + 1, dtype=torch.float64)[:, None, None]
+    assert not torch.allclose(got[:, 0], running_mean[:, 0], atol=1e-3), "biases after the rotation would give this"
 
 
 def test_head_dim_key_wins_over_the_derived_value(tmp_path):

@@ -4,7 +4,7 @@ implementation's full recomputation."""
 import pytest
 import torch
 
-from helpers import TINY, random_ids
+from helpers import assert_varied, random_ids
 from kernel_emulation import EmulatedKernels
 from plain import gemma_plain
 from wllm_amd.cache import OutOfPages
@@ -21,11 +21,13 @@ def emulated():
 
 
 @pytest.fixture(scope="module")
-def tiny(model_folders):
+def tiny(varied_folders):
+    # weights large enough that greedy decoding does not just repeat the last prompt token
+    folder = varied_folders["AV"]
     with ops.use_backend(EmulatedKernels()):
-        model = load_model(model_folders["A"], "float32", "cpu")
-    cfg = gemma_plain.read_config(model_folders["A"])
-    w = gemma_plain.read_weights(model_folders["A"], torch.float32)
+        model = load_model(folder, "float32", "cpu")
+    cfg = gemma_plain.read_config(folder)
+    w = gemma_plain.read_weights(folder, torch.float32)
     return model, cfg, w
 
 
@@ -52,6 +54,7 @@ def test_batched_generation_equals_each_request_alone_and_the_plain_implementati
         alone.add_request(Request(0, p, 8))
         assert alone.run_to_completion()[0].output_token_ids == together[i]
         assert gemma_plain.generate_greedy(cfg, w, p, 8) == together[i]
+        assert_varied(together[i])
     s.cache.check()
     assert s.cache.num_free_pages(0) == 64
 
@@ -202,6 +205,7 @@ def test_finishing_rules(tiny):
     model, cfg, w = tiny
     prompt = prompts_of([9])[0]
     plain = gemma_plain.generate_greedy(cfg, w, prompt, 6)
+    assert len(set(plain[:3])) == 3, "the stops below are in the middle of what is generated"
     s = make(model)
     one = Request("one", prompt, 1)
     s.add_request(one)
@@ -323,8 +327,84 @@ def test_looking_ahead_gives_every_request_the_same_tokens(tiny, admission, page
                               [r.output_token_ids for r in first], s.stats["preemptions"])
     assert results[True][:3] == results[False][:3]
     assert any(reason == "stop" for reason in results[True][1]), "the workload has requests that stop early"
+    assert any(reason == "stop" and len(out) > 1 for out, reason in zip(*results[True][:2])), "and not only at once"
+    for out in results[True][2]:
+        assert_varied(out, least=3)
     if admission == "prompt_only":
         assert results[True][3] > 0, "the small pool forces preemptions"
+
+
+@pytest.mark.parametrize("sampled", [False, True])
+def test_a_stop_at_any_output_index_ends_the_request_there_with_and_without_looking_ahead(tiny, sampled):
+    """The token that stops a request may come at any place among its outputs, the last but one
+    (where the step run ahead has already filled the request's length and closed it) and the last
+    included: the request ends with that token and "stop", and every page comes back."""
+    model, _, _ = tiny
+    prompt = prompts_of([11], 4)[0]
+    sp = SamplingParams(temperature=1.0, seed=77) if sampled else SamplingParams()
+    max_new = 6
+    free = make(model, lookahead=False)
+    r = Request("free", prompt, max_new, sampling_params=sp)
+    free.add_request(r)
+    free.run_to_completion()
+    out = list(r.output_token_ids)
+    assert len(set(out)) == max_new, f"every output token is its own stop: {out}"
+    for index in range(max_new):
+        for lookahead in (False, True):
+            for other in (False, True):      # alone, and beside a request that keeps the batch going
+                s = make(model, lookahead=lookahead)
+                stop = Request("stop", prompt, max_new, sampling_params=sp, stop_token_ids=frozenset([out[index]]))
+                s.add_request(stop)
+                if other:
+                    s.add_request(Request("other", prompts_of([5], 3)[0], 12))
+                s.run_to_completion()
+                assert stop.output_token_ids == out[:index + 1], (index, lookahead, other)
+                assert stop.finish_reason == "stop" and len(stop.logprobs) == index + 1 and stop.num_unread == 0
+                s.cache.check()
+                assert s.cache.num_free_pages(0) == 64 and not s.cache.requests
+
+
+def test_a_request_that_needs_the_page_set_aside_for_graphs_is_refused_when_added(tiny):
+    """Captured graphs keep one page per group for their padding rows; a request that would need
+    every page of the pool can then never be admitted and is refused at once instead of waiting
+    for ever (the reference's scheduler would spin to its step limit, scheduler.py:228-236,500-506)."""
+    model, _, _ = tiny
+    s = make(model, num_pages=8, page_size=4)
+    s.runner.enable_graphs()
+    assert s.cache.usable_pages(0) == 7
+    with pytest.raises(RequestRefused, match="pages"):
+        s.add_request(Request("all", prompts_of([24])[0], 8))      # 32 tokens: 8 pages
+    fits = Request("fits", prompts_of([20])[0], 8)                  # 28 tokens: 7 pages
+    s.add_request(fits)
+    assert not s.waiting[0].is_finished()
+
+
+def test_a_request_at_the_head_of_the_queue_that_can_never_fit_is_an_error_not_a_wait(tiny):
+    """Nothing runs, so no page can come back, and the head of the queue does not fit: the step
+    raises and names the request; the requests behind it are served afterwards."""
+    model, cfg, w = tiny
+    s = make(model, num_pages=6, page_size=4)
+    pool = s.cache.groups[0].pool
+    for _ in range(3):
+        pool.allocate("thief")        # pages lost behind the scheduler's back
+    s.add_request(Request("big", prompts_of([14])[0], 6))           # 5 pages of 3 free
+    small = Request("small", prompts_of([4], 2)[0], 4)
+    s.add_request(small)
+    with pytest.raises(RequestRefused, match="'big'"):
+        s.run_to_completion(max_steps=50)
+    assert [r.request_id for r in s.waiting] == ["small"]
+    s.run_to_completion()
+    assert small.output_token_ids == gemma_plain.generate_greedy(cfg, w, small.prompt_token_ids, 4)
+
+
+def test_run_to_completion_does_not_return_with_requests_unfinished(tiny):
+    model, _, _ = tiny
+    s = make(model)
+    s.add_request(Request("long", prompts_of([9])[0], 30))
+    with pytest.raises(RuntimeError, match="did not finish"):
+        s.run_to_completion(max_steps=5)
+    s.run_to_completion()
+    assert not s.has_unfinished_requests()
 
 
 def test_looking_ahead_starts_the_next_step_before_the_tokens_are_read(tiny):

@@ -71,7 +71,8 @@ def gemma_plan(cfg: GemmaConfig) -> ModelPlan:
         schedule=tuple(ScheduleEntry(layer=i) for i in range(cfg.num_hidden_layers)),
         final_norm=norm("model.norm.weight"),
         head=HeadSpec(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size,
-                      weight=None if cfg.tie_word_embeddings else "lm_head.weight"),
+                      weight=None if cfg.tie_word_embeddings else "lm_head.weight",
+                      tied_checkpoint_name="lm_head.weight"),
         max_positions=cfg.max_position_embeddings,
         # the rotation's frequencies are not persistent in the reference (llama.py:56);
         # checkpoints written by other tools sometimes carry them

@@ -16,9 +16,13 @@ contract of `reserve` and `commit` is the reference's `reserve`/`advance`
 without moving the request's length; `commit` moves it after all layers wrote.
 `reserve` is all-or-nothing across groups.
 
-A page of a group's storage is [2, kv_heads, page_size * head_dim]: the keys as
+What a page holds is the need's to say (`page_shape`).  For keys and values
+(`CacheNeed`) a page is [2, kv_heads, page_size * head_dim]: the keys as
 [page_size, head_dim] and the values transposed, [head_dim, page_size], which
-is the order the matrix-core attention kernels read them in.
+is the order the matrix-core attention kernels read them in.  A mixer that keeps
+something else per token (`PagedNeed`: a compressed vector, an integer code)
+gets pages of [page_size, *token_shape] in a dtype of its choice; the manager
+treats both alike.
 """
 from __future__ import annotations
 
@@ -42,10 +46,36 @@ class OutOfSlots(RuntimeError):
 class CacheNeed:
     """What one schedule entry keeps per token: keys and values of
     `num_kv_heads` heads of `head_dim`; all of them (window None) or the last
-    `window`."""
+    `window`.  Stored in the model's dtype."""
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    dtype = None
+
+    def page_shape(self, page_size: int) -> tuple:
+        return (2, self.num_kv_heads, page_size * self.head_dim)
+
+
+@dataclass(frozen=True)
+class PagedNeed:
+    """Any other per-token payload: `token_shape` numbers of `dtype` (None: the
+    model's) for every token, of all tokens (window None) or of the last `window`.
+    A page is [page_size, *token_shape]."""
+    token_shape: tuple
+    window: Optional[int] = None
+    dtype: Optional[torch.dtype] = None
+
+    def page_shape(self, page_size: int) -> tuple:
+        return (page_size,) + tuple(self.token_shape)
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """Per-request state of fixed size: one tensor of `shape` and `dtype` per
+    request, zeroed when the request is opened.  A mixer's `state_shape()` may
+    return this, or a plain shape for float32."""
+    shape: tuple
+    dtype: torch.dtype = torch.float32
 
 
 @dataclass
@@ -53,7 +83,7 @@ class LayerGroup:
     need: CacheNeed
     entries: list                      # schedule entries that own a cache here
     pool: PagePool
-    storage: Optional[torch.Tensor]    # [len(entries), pages, 2, kv_heads, page_size*head_dim]
+    storage: Optional[torch.Tensor]    # [len(entries), pages, *need.page_shape(page_size)]
     index_of_entry: dict = field(default_factory=dict)
 
 
@@ -71,9 +101,11 @@ class CacheManager:
     def __init__(self, needs: dict, page_size: int, num_pages, max_requests: int,
                  dtype: torch.dtype, device, state_shapes: Optional[dict] = None,
                  allocate_storage: bool = True, poison_freed_pages: bool = False):
-        """`needs`: {schedule entry: CacheNeed} for the entries that own a cache.
-        `num_pages`: pages of every group's pool (an int, or {CacheNeed: int}).
-        `state_shapes`: {schedule entry: shape} of fixed-size per-request state.
+        """`needs`: {schedule entry: need} for the entries that own a cache; a need is hashable
+        and has `window` (or None), `page_shape(page_size)` and `dtype` (None: the model's):
+        `CacheNeed`, `PagedNeed`.
+        `num_pages`: pages of every group's pool (an int, or {need: int}).
+        `state_shapes`: {schedule entry: shape or StateNeed} of fixed-size per-request state.
         `poison_freed_pages`: overwrite a page with NaN when it is given back, so
         that a read of a stale page shows in the results (for tests).
         """
@@ -95,8 +127,8 @@ class CacheManager:
             n = num_pages[need] if isinstance(num_pages, dict) else num_pages
             storage = None
             if allocate_storage:
-                storage = torch.zeros(len(entries), n, 2, need.num_kv_heads, page_size * need.head_dim,
-                                      dtype=dtype, device=device)
+                storage = torch.zeros(len(entries), n, *need.page_shape(page_size),
+                                      dtype=getattr(need, "dtype", None) or dtype, device=device)
             g = LayerGroup(need, entries, PagePool(n), storage, {e: i for i, e in enumerate(entries)})
             for e in entries:
                 self.group_of_entry[e] = len(self.groups)
@@ -105,8 +137,10 @@ class CacheManager:
         self._set_aside: dict = {}
         self._free_slots = list(range(max_requests - 1, -1, -1))
         self.state: dict = {}
-        for entry, shape in (state_shapes or {}).items():
-            self.state[entry] = torch.zeros((max_requests,) + tuple(shape), dtype=torch.float32, device=device)
+        for entry, need in (state_shapes or {}).items():
+            if not isinstance(need, StateNeed):
+                need = StateNeed(tuple(need))
+            self.state[entry] = torch.zeros((max_requests,) + tuple(need.shape), dtype=need.dtype, device=device)
 
     # ---- requests ----------------------------------------------------------
     def open(self, request) -> int:
@@ -159,6 +193,10 @@ class CacheManager:
 
     def num_free_pages(self, group_index: int = 0) -> int:
         return self.groups[group_index].pool.num_free
+
+    def usable_pages(self, group_index: int) -> int:
+        """Pages of a group that requests can ever hold: the pool without the pages set aside."""
+        return self.groups[group_index].pool.num_pages - len(self._set_aside.get(group_index, []))
 
     def set_aside_page(self, group_index: int) -> int:
         """Takes one page of a group out of circulation for good (captured graphs point
@@ -234,14 +272,17 @@ class CacheManager:
         return self.requests[request].tables[group_index]
 
     def entry_storage(self, entry: int) -> torch.Tensor:
-        """[pages, 2, kv_heads, page_size*head_dim] of one schedule entry."""
+        """[pages, *page_shape] of one schedule entry."""
         g = self.groups[self.group_of_entry[entry]]
         return g.storage[g.index_of_entry[entry]]
 
     def _release(self, g: LayerGroup, page: int, request) -> None:
         g.pool.free(page, request)
         if self.poison_freed_pages and g.storage is not None:
-            g.storage[:, page] = float("nan")
+            if g.storage.dtype.is_floating_point:
+                g.storage[:, page] = float("nan")
+            else:
+                g.storage[:, page] = torch.iinfo(g.storage.dtype).min
 
     # ---- invariants ------------------------------------------------------------
     def check(self) -> None:

@@ -16,8 +16,6 @@ import os
 import sys
 import time
 
-from wllm_amd.config import GemmaConfig
-
 SHAPES_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "config", "shapes")
 
 
@@ -78,13 +76,14 @@ def cmd_generate(args) -> int:
 def cmd_random_model(args) -> int:
     import torch
 
-    from wllm_amd.parts import write_random_model_folder
+    from wllm_amd.parts import write_random_model_from_config_json
     raw = read_shape(args.config)
     if args.num_hidden_layers is not None:
         raw["num_hidden_layers"] = args.num_hidden_layers
-    cfg = GemmaConfig.from_dict(raw)
     store = {"bfloat16": torch.bfloat16, "float32": torch.float32}[args.store_dtype]
-    write_random_model_folder(args.out, cfg, args.seed, std=args.std, norm_std=args.norm_std, store_dtype=store)
+    # the architecture named in the file parses and checks its own keys
+    write_random_model_from_config_json(args.out, raw, args.seed, std=args.std, norm_std=args.norm_std,
+                                        store_dtype=store)
     print(f"wrote {args.out}")
     return 0
 

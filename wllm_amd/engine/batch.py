@@ -31,7 +31,7 @@ class StepEntry:
 @dataclass
 class PageView:
     """The pages of one schedule entry as a mixer sees them."""
-    storage: torch.Tensor          # [pages, 2, kv_heads, page_size*head_dim]
+    storage: torch.Tensor          # [pages, *page shape]; keys and values: [pages, 2, kv_heads, page_size*head_dim]
     block_tables: torch.Tensor     # int32 [segments, max_pages]
     slots: torch.Tensor            # int32 [tokens]
     page_size: int
@@ -125,6 +125,6 @@ class StepContext:
                         self._cache.page_size, writes)
 
     def state(self, entry: int) -> Optional[torch.Tensor]:
-        """[max_requests, *shape] float32 state of a schedule entry; row state_slots[s]
-        belongs to segment s."""
+        """[max_requests, *shape] state of a schedule entry (float32 unless the mixer asked for
+        another dtype); row state_slots[s] belongs to segment s."""
         return self._cache.state.get(entry)

@@ -25,6 +25,25 @@ from wllm_amd.engine.batch import StepContext, Workspace
 from wllm_amd.kernels import ops
 
 
+def capture(body):
+    """Captures what `body()` launches into a new graph; returns (graph, body's result).
+
+    No garbage collection while the stream is capturing: a collector run that frees an object with
+    device resources of its own (an event, pinned memory, another graph) makes a call the capture
+    does not allow, and the process aborts.  The collector is switched back on afterwards if it was
+    on, also when the body raises."""
+    graph = torch.cuda.CUDAGraph()
+    collecting = gc.isenabled()
+    gc.disable()
+    try:
+        with torch.cuda.graph(graph):
+            result = body()
+    finally:
+        if collecting:
+            gc.enable()
+    return graph, result
+
+
 class DecodeGraph:
     def __init__(self, runner, bucket: int, max_context: int):
         self.runner = runner
@@ -123,18 +142,6 @@ class DecodeGraph:
             # once eagerly: scratch tensors and plans come into being, lazy library state settles
             self.runner.model.forward(self.ctx)
             torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            # No garbage collection while the stream is capturing: a collector run that frees an
-            # object with device resources of its own (an event, pinned memory, another graph)
-            # makes a call the capture does not allow, and the process aborts.
-            collecting = gc.isenabled()
-            gc.disable()
-            try:
-                with torch.cuda.graph(graph):
-                    self.logits = self.runner.model.forward(self.ctx)
-            finally:
-                if collecting:
-                    gc.enable()
-            self.graph = graph
+            self.graph, self.logits = capture(lambda: self.runner.model.forward(self.ctx))
         self.graph.replay()
         return self.logits[:len(entries)]

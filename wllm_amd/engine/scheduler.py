@@ -99,8 +99,10 @@ class Scheduler:
                                  f"positions; the model allows {limit}")
         for gi, g in enumerate(self.cache.groups):
             need = self.cache.pages_for(gi, request.total_len_estimate, self._longest_portion(request))
-            if need > g.pool.num_pages:
-                raise RequestRefused(f"request {request.request_id!r} needs {need} pages; the pool has {g.pool.num_pages}")
+            usable = self.cache.usable_pages(gi)
+            if need > usable:
+                raise RequestRefused(f"request {request.request_id!r} needs {need} pages; the pool has {usable} "
+                                     f"that a request can ever hold")
         request.arrival_index = self._arrivals
         request.seed = self.sampler.seed_of(request.sampling_params, self._arrivals)
         self._arrivals += 1
@@ -176,6 +178,11 @@ class Scheduler:
         while self.waiting and (unlimited or budget > 0):
             r = self.waiting[0]
             if not self._fits(r):
+                if not self.running:
+                    # nothing holds a page that could come back: waiting would be for ever
+                    self.waiting.pop(0)
+                    raise RequestRefused(f"request {r.request_id!r} does not fit into the free pages although no "
+                                         f"request is running; it can never be admitted")
                 self.stats["admission_waits"] += 1
                 break       # first come, first served: the head is not skipped
             self.waiting.pop(0)
@@ -293,11 +300,9 @@ class Scheduler:
             got.append(r)
             if r.ends_with(tokens[row]):
                 # sequence.py:53-59: the stop rules come before the length rule
-                already_over = r.is_finished()
                 r.status, r.finish_reason = RequestStatus.FINISHED, "stop"
-                if already_over:
-                    continue
-                # the request may have been run ahead: that token does not count
+                # The request may have been run ahead: that token does not count, whether or not it
+                # was the one that filled the request's length (and closed it in the step run ahead).
                 ahead = self._started
                 if ahead is not None:
                     for row2, r2 in enumerate(ahead.sampled):
@@ -305,7 +310,7 @@ class Scheduler:
                             ahead.dropped.add(row2)
                             r.num_unread -= 1
                 del r.output_token_ids[place + 1:], r.logprobs[place + 1:]
-                if r in self.running:
+                if r in self.running:           # not there if its length had closed it already
                     self.running.remove(r)
                     self.cache.close(r.request_id)
                 elif r in self.waiting:         # preempted after it was sampled
@@ -313,9 +318,14 @@ class Scheduler:
         return got
 
     def run_to_completion(self, max_steps: int = 1_000_000) -> list:
+        """Steps until nothing is left (scheduler.py:500-506).  Ending with requests unfinished is an
+        error, not a result."""
         finished = []
         for _ in range(max_steps):
             if not self.has_unfinished_requests():
-                break
+                return finished
             finished.extend(r for r in self.step() if r.is_complete())
+        if self.has_unfinished_requests():
+            left = [r.request_id for r in self.running + self.waiting]
+            raise RuntimeError(f"{max_steps} steps did not finish requests {left!r}")
         return finished

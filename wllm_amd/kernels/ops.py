@@ -168,6 +168,14 @@ def linear_residual_takes(rows: int, dtype: torch.dtype, out_features: int, in_f
     return bool(backend().linear_residual_takes(rows, dtype, out_features, in_features))
 
 
+SUMSQ_BAND = 16      # columns whose squares `linear_residual` adds into one entry of `sumsq`
+
+
+def linear_residual_sumsq_shape(rows: int, out_features: int) -> tuple:
+    """The shape of the `sumsq` operand of `linear_residual` for a residual of [rows, out_features]."""
+    return (rows, out_features // SUMSQ_BAND)
+
+
 def linear_residual(x: torch.Tensor, weight: torch.Tensor, residual: torch.Tensor, sumsq: torch.Tensor,
                     tiles: Optional[torch.Tensor] = None) -> None:
     """residual += x @ weight^T in float32, and sumsq[m, b] = the sum of squares of the new
@@ -184,7 +192,7 @@ def linear_residual(x: torch.Tensor, weight: torch.Tensor, residual: torch.Tenso
     _check_tiles(tiles, weight, 1)
     _need(linear_residual_takes(m, x.dtype, n, k), "linear_residual: no kernel for these sizes")
     _dense(residual, "residual", torch.float32, (m, n))
-    _dense(sumsq, "sumsq", torch.float32, (m, n // 16))
+    _dense(sumsq, "sumsq", torch.float32, linear_residual_sumsq_shape(m, n))
     if m:
         backend().linear_residual(x, weight, tiles, residual, sumsq)
 

@@ -58,6 +58,8 @@ class PagedAttention:
         for name, width in ((s.q_bias, q), (s.k_bias, kv), (s.v_bias, kv)):
             if name is not None:
                 out[name] = ExpectedTensor((width,), role="vector")
+        if hasattr(self.position, "expected_tensors"):      # a position encoding with tensors of its own
+            out.update(self.position.expected_tensors())
         return out
 
     def load(self, fetch) -> None:
@@ -70,6 +72,8 @@ class PagedAttention:
             parts = [fetch.vector(name) if name is not None else torch.zeros(width)
                      for name, width in ((s.q_bias, q), (s.k_bias, kv), (s.v_bias, kv))]
             self.b_qkv = fetch.to_device(torch.cat(parts))
+        if hasattr(self.position, "load"):
+            self.position.load(fetch)
         self.position.prepare(fetch.device)
 
     def cache_need(self) -> Optional[CacheNeed]:
@@ -84,10 +88,23 @@ class PagedAttention:
         qkv = ctx.buffer("qkv", (n, self.qkv_width), h.dtype)
         pages = ctx.pages(entry)
         slots, storage = (pages.slots, pages.storage) if pages.writes else (None, None)
-        rotary_dim = 2 * self.position.inv_freq.shape[0] if self.position.inv_freq is not None else s.head_dim
-        if ops.qkv_rope_takes(n, h.dtype, h.shape[1], s.head_dim, rotary_dim):
+        # What the position encoding asks for: a table of frequencies that the rotation kernels turn
+        # queries and keys by (`inv_freq`, or None), and/or a step of its own on the projected rows
+        # before they are cached and read (`apply`).
+        inv_freq = self.position.inv_freq
+        apply = getattr(self.position, "apply", None)
+        rotary_dim = 2 * inv_freq.shape[0] if inv_freq is not None else s.head_dim
+        if apply is not None:
+            ops.linear(h, self.w_qkv, qkv, self.t_qkv)
+            if self.b_qkv is not None:
+                qkv += self.b_qkv.to(qkv.dtype)
+            apply(ctx, qkv, num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim)
+            ops.rope_and_cache_write(
+                qkv, None, ctx.positions, inv_freq, slots, storage,
+                num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim, page_size=pages.page_size)
+        elif ops.qkv_rope_takes(n, h.dtype, h.shape[1], s.head_dim, rotary_dim):
             # a decode step: projection, rotation and cache write in one kernel
-            ops.qkv_rope(h, self.w_qkv, qkv, self.b_qkv, ctx.positions, self.position.inv_freq, slots, storage,
+            ops.qkv_rope(h, self.w_qkv, qkv, self.b_qkv, ctx.positions, inv_freq, slots, storage,
                          num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim,
                          page_size=pages.page_size, tiles=self.t_qkv)
         else:
@@ -95,7 +112,7 @@ class PagedAttention:
             projected = project(ctx, "qkv", h, self.w_qkv, qkv, tiles=self.t_qkv)
             parts = projected if projected.dim() == 3 else None
             ops.rope_and_cache_write(
-                qkv, self.b_qkv, ctx.positions, self.position.inv_freq, slots, storage,
+                qkv, self.b_qkv, ctx.positions, inv_freq, slots, storage,
                 num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim, page_size=pages.page_size,
                 parts=parts)
         attn = ctx.buffer("attn", (n, s.num_heads * s.head_dim), h.dtype)

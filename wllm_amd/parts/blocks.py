@@ -32,7 +32,7 @@ class ResidualStream:
     def __init__(self, x: torch.Tensor, pending: Optional[torch.Tensor] = None):
         self.x = x
         self.pending = pending
-        self.sumsq: Optional[torch.Tensor] = None      # float32 [n, H / 16], valid for x as it is now
+        self.sumsq: Optional[torch.Tensor] = None      # float32 [n, bands]: sums of squares of x as it is now
 
     def normed(self, norm, out: torch.Tensor, rows=None) -> torch.Tensor:
         """norm(x + pending).  Without `rows` the sum becomes the new x."""
@@ -57,7 +57,7 @@ class ResidualStream:
         if isinstance(y, Product):
             n, hidden = self.x.shape
             if ops.linear_residual_takes(n, y.x.dtype, hidden, y.x.shape[1]):
-                sumsq = ctx.buffer("sumsq", (n, hidden // 16), torch.float32)
+                sumsq = ctx.buffer("sumsq", ops.linear_residual_sumsq_shape(n, hidden), torch.float32)
                 ops.linear_residual(y.x, y.weight, self.x, sumsq, y.tiles)
                 self.sumsq = sumsq
                 return

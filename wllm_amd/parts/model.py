@@ -61,16 +61,17 @@ class CausalLM:
             if e.reads_cache_of is not None:
                 mine = self.blocks[e.layer].mixer.cache_need()
                 theirs = needs.get(e.reads_cache_of)
-                if mine is None or theirs is None or (mine.num_kv_heads, mine.head_dim) != (theirs.num_kv_heads, theirs.head_dim):
+                if mine is None or theirs is None or type(mine) is not type(theirs) \
+                        or mine.page_shape(1) != theirs.page_shape(1):
                     raise ValueError(f"schedule entry {i} cannot read the cache of entry {e.reads_cache_of}: shapes differ")
         return needs
 
     def state_shapes(self) -> dict:
         shapes = {}
         for i, e in enumerate(self.plan.schedule):
-            shape = self.blocks[e.layer].mixer.state_shape()
+            shape = self.blocks[e.layer].mixer.state_shape()      # a shape (float32) or a StateNeed
             if shape is not None:
-                shapes[i] = tuple(shape)
+                shapes[i] = shape
         return shapes
 
     def graph_capturable(self) -> bool:
@@ -96,8 +97,8 @@ class CausalLM:
         emb, head = self.plan.embedding, self.plan.head
         # a tied checkpoint may still carry the head; it is accepted if it is the table
         extra = ()
-        tied_head_name = "lm_head.weight"
-        if head.weight is None and tied_head_name in checkpoint:
+        tied_head_name = head.tied_checkpoint_name
+        if head.weight is None and tied_head_name is not None and tied_head_name in checkpoint:
             extra = (tied_head_name,)
         checkpoint.check(self.expected_tensors(), self.plan.ignored_tensor_suffixes, allowed_extra=extra)
         fetch = TensorFetcher(checkpoint, dtype, device, tiled_copies=tiled_copies)
@@ -185,11 +186,19 @@ def load_model(folder: str, dtype="bfloat16", device="cuda", tiled_copies: Optio
     return model
 
 
+def write_random_model_from_config_json(folder: str, raw_config: dict, seed: int, *, std: float = 0.02,
+                                        norm_std: float = 0.1, store_dtype: torch.dtype = torch.bfloat16) -> str:
+    """The random-weights mode: the contents of a config.json (of any registered architecture) and a
+    seed to a model folder.  The configuration is parsed and checked by its architecture; what is
+    written as config.json is `raw_config` itself."""
+    from wllm_amd.weights.random_init import write_random_model
+    model = build_model(raw_config)
+    return write_random_model(folder, raw_config, model.expected_tensors(), seed, std=std, norm_std=norm_std,
+                              store_dtype=store_dtype)
+
+
 def write_random_model_folder(folder: str, config, seed: int, *, std: float = 0.02, norm_std: float = 0.1,
                               store_dtype: torch.dtype = torch.bfloat16) -> str:
-    """The random-weights mode: a typed configuration and a seed to a model folder."""
-    from wllm_amd.weights.random_init import write_random_model
-    raw = config.to_dict()
-    model = build_model(raw)
-    return write_random_model(folder, raw, model.expected_tensors(), seed, std=std, norm_std=norm_std,
-                              store_dtype=store_dtype)
+    """The same from a typed configuration that can write itself as config.json (`to_dict()`)."""
+    return write_random_model_from_config_json(folder, config.to_dict(), seed, std=std, norm_std=norm_std,
+                                               store_dtype=store_dtype)

@@ -5,7 +5,12 @@ tensors it expects, loads them, and runs on the flat batch of a step.  The
 interfaces:
 
 norm          expected_tensors(); load(fetch); forward(x, out, delta=None, rows=None)
-position      prepare(dtype, device); arguments for the mixer's rotation kernel
+position      prepare(device); `inv_freq`: float32 [rotary_dim / 2] that the mixer's rotation kernels
+              turn queries and keys by, or None; optionally `apply(ctx, qkv, *, num_heads,
+              num_kv_heads, head_dim)`, a step of its own on the projected rows [tokens,
+              (heads + 2 kv heads) * head_dim] in place (positions in `ctx.positions`) before keys
+              are cached, for encodings that are no rotation; optionally `expected_tensors()`
+              and `load(fetch)` for tensors of its own
 mixer         expected_tensors(); load(fetch); cache_need() -> CacheNeed | None;
               state_shape() -> tuple | None; forward(ctx, entry, h) -> y
 feed-forward  expected_tensors(); load(fetch); forward(ctx, h) -> y

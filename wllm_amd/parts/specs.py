@@ -106,10 +106,13 @@ class EmbeddingSpec:
 
 @dataclass(frozen=True)
 class HeadSpec:
-    """logits = hidden @ W^T; W is the embedding table when `weight` is None."""
+    """logits = hidden @ W^T; W is the embedding table when `weight` is None.  `tied_checkpoint_name`:
+    the name under which a checkpoint of tied weights may still store the head; such a tensor is
+    accepted if it equals the table."""
     vocab_size: int
     hidden_size: int
     weight: Optional[str] = None
+    tied_checkpoint_name: Optional[str] = None
 
 
 @dataclass(frozen=True)

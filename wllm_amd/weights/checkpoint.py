@@ -52,6 +52,11 @@ class Checkpoint:
         if os.path.isfile(index):
             with open(index, "r", encoding="utf-8") as f:
                 files = sorted(set(json.load(f).get("weight_map", {}).values()))
+            for p in files:
+                # the index is part of an untrusted folder: it names files of that folder, nothing else
+                if not isinstance(p, str) or os.path.basename(p) != p or not p.endswith(".safetensors"):
+                    raise WeightError(f"{index}: weight_map names {p!r}; expected the plain name of a "
+                                      f".safetensors file in the same folder")
             paths = [os.path.join(folder, p) for p in files]
         else:
             paths = sorted(glob.glob(os.path.join(folder, "*.safetensors")))
