@@ -200,7 +200,7 @@ def check_toy3(folder, device, dtype="float32"):
         assert tuple(latent_group.storage.shape[2:]) == (4, R) and latent_group.storage.dtype == torch.float32
         assert cache.state[0].dtype == torch.int32 and tuple(cache.state[0].shape) == (4, 1)
         got = replay_and_collect(TraceReplayer(runner), trace)
-        tol = dict(atol=5e-5, rtol=2e-4) if dtype == "float32" else dict(atol=3e-2, rtol=3e-2)
+        tol = dict(atol=5e-5, rtol=2e-4) if dtype == "float32" else dict(atol=8e-2, rtol=3e-2)      # logits up to 3 from weights of std 0.2
         compare_with_plain(got, plain, **tol)
         cache.check()
         assert all(g.pool.num_free == g.pool.num_pages for g in cache.groups)

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import TINY, compare_with_plain, random_ids, replay_and_collect, trace_tail, trace_whole
+from helpers import TINY, VARIED, assert_varied, compare_with_plain, random_ids, replay_and_collect, trace_tail, trace_whole
 from plain import gemma_plain
 from wllm_amd.engine import LLM, ModelRunner, Request, Scheduler
 from wllm_amd.engine.replay import TraceReplayer
@@ -24,13 +24,19 @@ def plain_model(folder):
     return gemma_plain.read_config(folder), gemma_plain.read_weights(folder, torch.float32)
 
 
-@pytest.mark.parametrize("name,lengths,new", [("A", [7, 16, 23], 8), ("B", [5, 31, 64], 6), ("C", [9, 20], 6), ("M", [33, 70], 6)])
-def test_greedy_generation_through_the_entry_point_float32(model_folders, name, lengths, new):
-    # the first case is a tiny workload of its own: prompts of 7/16/23 ids, 8 greedy tokens each, pages of 4
-    cfg, w = plain_model(model_folders[name])
+@pytest.mark.parametrize("name,lengths,new", [("A", [7, 16, 23], 8), ("B", [5, 31, 64], 6), ("C", [9, 20], 6), ("M", [33, 70], 6),
+                                              ("AV", [7, 16, 23], 12), ("MV", [33, 70, 12], 12)])
+def test_greedy_generation_through_the_entry_point_float32(model_folders, varied_folders, name, lengths, new):
+    # the first case is a tiny workload of its own: prompts of 7/16/23 ids, 8 greedy tokens each, pages of 4.
+    # A, B and M repeat their last prompt token (the tied head's self-logit wins); C, AV and MV do not.
+    folder = model_folders[name] if name in model_folders else varied_folders[name]
+    cfg, w = plain_model(folder)
     prompts = [random_ids(i + 1, n, cfg["vocab_size"]) for i, n in enumerate(lengths)]
-    llm = LLM(model_folders[name], dtype="float32", num_blocks=64, block_size=TINY[name]["page_size"])
+    llm = LLM(folder, dtype="float32", num_blocks=64, block_size=(TINY.get(name) or VARIED[name])["page_size"])
     outs = llm.generate(prompts, max_new_tokens=new)
+    if name in ("C", "AV", "MV"):
+        for o in outs:
+            assert_varied(o.token_ids)
     for p, o in zip(prompts, outs):
         assert o.token_ids == gemma_plain.generate_greedy(cfg, w, p, new)
         assert o.finish_reason == "length" and len(o.logprobs) == new
@@ -170,11 +176,11 @@ def test_trace_run_says_when_a_trace_holds_more_than_max_tokens(model_folders, t
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_captured_graphs_give_what_eager_steps_give(model_folders, dtype):
+def test_captured_graphs_give_what_eager_steps_give(varied_folders, dtype):
     """Decode steps replayed from captured graphs against the same steps run kernel by kernel:
     several replays with eager work (prompt portions of newly admitted requests) between them,
     batches that grow and shrink through the buckets, every replay checked."""
-    folder = model_folders["M"]
+    folder = varied_folders["MV"]
     model = load_model(folder, dtype, "cuda")
     prompts = [random_ids(40 + i, n, 1000) for i, n in enumerate([9, 33, 17, 70, 5, 41])]
     news = [30, 12, 25, 8, 40, 18]
@@ -196,13 +202,14 @@ def test_captured_graphs_give_what_eager_steps_give(model_folders, dtype):
     assert runner.graph_steps > 20 and len(runner.graphs) >= 2
     for a, b in zip(eager, graphed):
         assert a.output_token_ids == b.output_token_ids
+        assert_varied(a.output_token_ids)
         assert torch.allclose(torch.tensor(a.logprobs), torch.tensor(b.logprobs), atol=1e-5 if dtype == "float32" else 2e-2)
 
 
-def test_a_full_batch_of_any_size_has_its_graph(model_folders):
+def test_a_full_batch_of_any_size_has_its_graph(varied_folders):
     """The largest number of requests the cache admits is a bucket of its own: a full batch of 3
     (or 17) does not fall back to steps run kernel by kernel."""
-    model = load_model(model_folders["M"], "bfloat16", "cuda")
+    model = load_model(varied_folders["MV"], "bfloat16", "cuda")
     runner = ModelRunner.create(model, num_pages=40, page_size=16, max_requests=3)
     runner.enable_graphs()
     assert runner.graph_buckets == (1, 2, 3)
@@ -219,15 +226,18 @@ def test_a_full_batch_of_any_size_has_its_graph(model_folders):
         s2.add_request(r)
     s2.run_to_completion()
     assert [r.output_token_ids for r in reqs] == [r.output_token_ids for r in again]
+    assert_varied(reqs[0].output_token_ids)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("graphs", [False, True])
-def test_looking_ahead_gives_the_same_tokens_on_the_gpu(model_folders, dtype, graphs):
+def test_looking_ahead_gives_the_same_tokens_on_the_gpu(varied_folders, dtype, graphs):
     """Steps started before the step before them was read (token ids taken from the device, in
     eager steps and in replayed graphs) against the same requests run step by step: mixed greedy
-    and seeded sampling, prompt portions beside decoded tokens, requests that stop on a token."""
-    folder = model_folders["M"]
+    and seeded sampling, prompt portions beside decoded tokens, requests that stop on a token: in the
+    middle of what they generate, at the last output but one (the step run ahead has filled the
+    request's length by then) and at the last."""
+    folder = varied_folders["MV"]
     model = load_model(folder, dtype, "cuda")
     prompts = [random_ids(90 + i, n, 1000) for i, n in enumerate([9, 33, 17, 70, 5, 41, 12])]
     news = [30, 12, 25, 8, 40, 18, 22]
@@ -254,21 +264,36 @@ def test_looking_ahead_gives_the_same_tokens_on_the_gpu(model_folders, dtype, gr
         return reqs, runner
 
     free, _ = run(False, {})
-    # stop three of them in the middle of what they generate
-    stops = {0: dict(eos_token_id=free[0].output_token_ids[11]), 3: dict(stop_token_ids=frozenset([free[3].output_token_ids[2]])),
-             4: dict(eos_token_id=free[4].output_token_ids[20])}
+    for r in free:
+        assert_varied(r.output_token_ids)
+
+    def stop_at(i, index):
+        """A token of request i that first occurs at `index` of what it generates freely, or near it."""
+        out = free[i].output_token_ids
+        index = next(k for k in [index] + list(range(len(out) - 1, -1, -1)) if out.index(out[k]) == k)
+        return out[index], index
+
+    # three stop in the middle, one at its last output but one, one at its last
+    wanted = {0: 11, 3: 2, 4: 20, 1: news[1] - 2, 5: news[5] - 1}
+    stops, places = {}, {}
+    for i, index in wanted.items():
+        token, places[i] = stop_at(i, index)
+        stops[i] = dict(eos_token_id=token) if i % 2 == 0 else dict(stop_token_ids=frozenset([token]))
+    assert places[1] == news[1] - 2 or places[5] == news[5] - 1, "a stop at the end of a request's length is among them"
     stepwise, _ = run(False, stops)
     ahead, runner = run(True, stops)
     if graphs:
         assert runner.graph_steps > 20
-    assert sum(r.finish_reason == "stop" for r in ahead) == 3
+    assert sum(r.finish_reason == "stop" for r in ahead) == 5
+    for i, index in places.items():
+        assert ahead[i].output_token_ids == free[i].output_token_ids[:index + 1]
     for a, b in zip(stepwise, ahead):
         assert a.output_token_ids == b.output_token_ids and a.finish_reason == b.finish_reason
         assert torch.allclose(torch.tensor(a.logprobs), torch.tensor(b.logprobs), atol=1e-5 if dtype == "float32" else 2e-2)
 
 
-def test_command_line_generates_what_the_entry_point_generates(model_folders, tmp_path):
-    folder = model_folders["A"]
+def test_command_line_generates_what_the_entry_point_generates(varied_folders, tmp_path):
+    folder = varied_folders["AV"]
     cfg, w = plain_model(folder)
     prompts = [random_ids(5, 9, 512), random_ids(6, 14, 512)]
     args = [sys.executable, "-m", "wllm_amd.cli", "generate", "--model", folder, "--dtype", "float32", "--num-blocks", "32",
@@ -280,3 +305,4 @@ def test_command_line_generates_what_the_entry_point_generates(model_folders, tm
     lines = [json.loads(l) for l in proc.stdout.splitlines() if l.startswith("{")]
     assert [l["token_ids"] for l in lines] == [gemma_plain.generate_greedy(cfg, w, p, 6) for p in prompts]
     assert all(l["finish_reason"] == "length" for l in lines)
+    assert_varied(lines[0]["token_ids"])

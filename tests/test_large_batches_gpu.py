@@ -121,20 +121,21 @@ def test_mixed_steps_of_24_live_requests(models, plain_models, dtype):
 
 
 def test_forty_requests_generate_what_the_plain_implementation_generates(varied_folders):
-    """Continuous batching of 40 requests through the entry point, float32: prompt portions beside up to 32
-    decoding requests, captured graphs of the default buckets, steps started ahead; every request's greedy
+    """Continuous batching of 40 requests through the entry point, float32: prompt portions beside
+    decoding requests, then decode steps of all 32 admitted requests from captured graphs of the default
+    buckets, steps started ahead, the last 8 requests admitted as others finish; every request's greedy
     tokens equal the plain implementation's full recomputation."""
     folder = varied_folders["MV"]
     cfg = gemma_plain.read_config(folder)
     w = gemma_plain.read_weights(folder, torch.float32)
     rng = np.random.default_rng(11)
-    prompts = [random_ids(500 + i, int(n), cfg["vocab_size"]) for i, n in enumerate(rng.integers(3, 120, size=40))]
-    news = [int(n) for n in rng.integers(4, 14, size=40)]
+    prompts = [random_ids(500 + i, int(n), cfg["vocab_size"]) for i, n in enumerate(rng.integers(3, 60, size=40))]
+    news = [int(n) for n in rng.integers(24, 40, size=40)]
     llm = LLM(folder, dtype="float32", num_blocks=400, block_size=16, max_prefill_tokens_per_step=96, max_requests=32,
               hip_graphs=True, lookahead=True)
     outs = llm.generate(prompts, max_new_tokens=news)
     llm.runner.cache.check()
-    assert llm.runner.graph_steps > 0 and max(llm.runner.graphs) >= 32
+    assert llm.runner.graph_steps > 10 and max(llm.runner.graphs) == 32, sorted(llm.runner.graphs)
     for p, n, o in zip(prompts, news, outs):
         assert o.token_ids == gemma_plain.generate_greedy(cfg, w, p, n)
         assert o.finish_reason == "length"
