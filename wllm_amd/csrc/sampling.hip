@@ -1,5 +1,8 @@
 // Sampling kernels over rows of float32 logits.
 #include "common.h"
+#include "wllm_no_alloc.h"
+
+#include <mutex>
 
 // ---- argmax: the largest value of a row, the lowest index among equals -------------------------
 // Two stages, so that a handful of rows still use many compute units: a row is cut into
@@ -76,9 +79,9 @@ argmax_final_kernel(const float* __restrict__ part_v, const int* __restrict__ pa
     if (lane == 0) out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
 }
 
-// `scratch` holds rows * 64 four-byte words.
-WLLM_API int wllm_argmax_rows(const float* logits, int* out, void* scratch, int rows, int vocab, hipStream_t stream) {
-    float* part_v = static_cast<float*>(scratch);
+// `workspace` holds rows * 64 four-byte words.
+WLLM_API int wllm_argmax_rows(const float* logits, int* out, void* workspace, int rows, int vocab, hipStream_t stream) {
+    float* part_v = static_cast<float*>(workspace);
     int* part_i = reinterpret_cast<int*>(part_v + static_cast<size_t>(rows) * kArgmaxSplits);
     int segment = (vocab + kArgmaxSplits - 1) / kArgmaxSplits;
     segment = (segment + 3) / 4 * 4;
@@ -686,14 +689,11 @@ sample_draw_kernel(const float* __restrict__ logits, const float* __restrict__ p
 // Words of scratch a row needs in `wllm_sample_rows_split`.
 WLLM_API int wllm_sample_split_row_words() { return kRowWords; }
 
-// The sampler with each row spread over kSampleSegments workgroups.  `scratch` holds rows *
-// wllm_sample_split_row_words() 8-byte words; `truncations` says whether any row has top-k or top-p
-// (then three more histogram levels run).  Same tokens and log-probabilities as `wllm_sample_rows`.
-WLLM_API int wllm_sample_rows_split(float* logits, const float* params, const long long* seeds, const int* penalty_ids,
-                                    const int* penalty_offsets, int* out_tokens, float* out_logprobs, void* scratch,
-                                    int rows, int vocab, int truncations, hipStream_t stream) {
-    if (rows < 1 || vocab < 1 || !scratch) return -1;
-    u64* ws = static_cast<u64*>(scratch);
+// The launches of the sampler with each row spread over kSampleSegments workgroups; `ws` holds
+// rows * kRowWords words on the device.  The prepare kernel clears what must start at zero.
+static int launch_sample_rows_split(float* logits, const float* params, const long long* seeds, const int* penalty_ids,
+                                    const int* penalty_offsets, int* out_tokens, float* out_logprobs, u64* ws, int rows,
+                                    int vocab, int truncations, hipStream_t stream) {
     if (penalty_ids) {
         sample_penalty_kernel<<<rows, 256, 0, stream>>>(logits, params, penalty_ids, penalty_offsets, vocab);
         if (int err = launch_status()) return err;
@@ -709,6 +709,72 @@ WLLM_API int wllm_sample_rows_split(float* logits, const float* params, const lo
     if (int err = launch_status()) return err;
     sample_draw_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, params, seeds, ws, out_tokens, out_logprobs, vocab);
     return launch_status();
+}
+
+// The sampler with each row spread over kSampleSegments workgroups.  `workspace` holds rows *
+// wllm_sample_split_row_words() 8-byte words; `truncations` says whether any row has top-k or top-p
+// (then three more histogram levels run).  Same tokens and log-probabilities as `wllm_sample_rows`.
+WLLM_API int wllm_sample_rows_split(float* logits, const float* params, const long long* seeds, const int* penalty_ids,
+                                    const int* penalty_offsets, int* out_tokens, float* out_logprobs, void* workspace,
+                                    int rows, int vocab, int truncations, hipStream_t stream) {
+    if (rows < 1 || vocab < 1 || !workspace) return -1;
+    return launch_sample_rows_split(logits, params, seeds, penalty_ids, penalty_offsets, out_tokens, out_logprobs,
+                                    static_cast<u64*>(workspace), rows, vocab, truncations, stream);
+}
+
+// ---- the same sampler for callers that cannot allocate (wllm_no_alloc.h) -------------------------
+// The scratch area is a device array of the library's image.  In host code its name is only a
+// handle for the runtime, not a device address: the address of each GPU's copy comes from
+// hipGetSymbolAddress, once per device, and only that pointer is ever handed to a kernel.
+constexpr int kStaticSampleRows = 64;
+constexpr int kStaticMaxDevices = 64;
+static __device__ __align__(256) u64 scratch[static_cast<size_t>(kStaticSampleRows) * kRowWords];
+static u64* scratch_of_device[kStaticMaxDevices];       // host side: device address of `scratch` per GPU
+static std::mutex scratch_lock;
+
+// The current device's copy of `scratch`; resolved at the first call on that device.
+static int static_scratch(u64** out) {
+    int device = -1;
+    if (hipError_t err = hipGetDevice(&device)) return static_cast<int>(err);
+    if (device < 0 || device >= kStaticMaxDevices) return static_cast<int>(hipErrorInvalidDevice);
+    std::lock_guard<std::mutex> hold(scratch_lock);
+    if (!scratch_of_device[device]) {
+        void* address = nullptr;
+        if (hipError_t err = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch))) return static_cast<int>(err);
+        if (!address) return static_cast<int>(hipErrorInvalidSymbol);
+        scratch_of_device[device] = static_cast<u64*>(address);
+    }
+    *out = scratch_of_device[device];
+    return 0;
+}
+
+WLLM_NO_ALLOC_API int wllm_sample_static_max_rows(void) { return kStaticSampleRows; }
+
+WLLM_NO_ALLOC_API int wllm_sample_static_init(void) {
+    u64* ws = nullptr;
+    return static_scratch(&ws);
+}
+
+WLLM_NO_ALLOC_API const char* wllm_sample_static_error(int code) {
+    switch (code) {
+        case 0: return "success";
+        case WLLM_STATIC_BAD_ARGUMENT: return "wllm_sample_rows_static: rows < 1, vocab < 1 or a null pointer";
+        case WLLM_STATIC_TOO_MANY_ROWS: return "wllm_sample_rows_static: more rows than wllm_sample_static_max_rows() (64)";
+        default: return code > 0 ? hipGetErrorString(static_cast<hipError_t>(code)) : "wllm_sample_rows_static: unknown error code";
+    }
+}
+
+WLLM_NO_ALLOC_API int wllm_sample_rows_static(float* logits, const float* params, const long long* seeds,
+                                              const int* penalty_ids, const int* penalty_offsets, int* out_tokens,
+                                              float* out_logprobs, int rows, int vocab, int truncations,
+                                              hipStream_t stream) {
+    if (rows < 1 || vocab < 1 || !logits || !params || !seeds || !out_tokens || !out_logprobs) return WLLM_STATIC_BAD_ARGUMENT;
+    if ((penalty_ids == nullptr) != (penalty_offsets == nullptr)) return WLLM_STATIC_BAD_ARGUMENT;
+    if (rows > kStaticSampleRows) return WLLM_STATIC_TOO_MANY_ROWS;
+    u64* ws = nullptr;
+    if (int err = static_scratch(&ws)) return err;
+    return launch_sample_rows_split(logits, params, seeds, penalty_ids, penalty_offsets, out_tokens, out_logprobs, ws,
+                                    rows, vocab, truncations, stream);
 }
 
 WLLM_API int wllm_sample_rows(float* logits, const float* params, const long long* seeds, const int* penalty_ids,
