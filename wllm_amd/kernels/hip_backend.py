@@ -42,14 +42,17 @@ _SIGNATURES = {
     "wllm_tile_weight": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "wllm_gated_activation": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_paged_attention_generic": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                     c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+                                     c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                     c_float, c_int, c_void_p],
+    "wllm_paged_attention_generic_chunk_keys": [],
     "wllm_paged_attention_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
                                   c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
                                   c_int, c_void_p],
     "wllm_paged_attention_prefill": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                                      c_void_p],
-    "wllm_gemm_generic": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "wllm_gemm_generic": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
+    "wllm_gemm_generic_segments": [c_int],
     "wllm_argmax_rows": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "wllm_gemm_skinny": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
                          c_void_p],
@@ -71,6 +74,7 @@ class HipBackend:
         self._argmax_scratch = None
         self._sample_scratch = None
         self._partial_ml = None
+        self._generic_partial_o = None
         for name, argtypes in _SIGNATURES.items():
             fn = getattr(self.lib, name)
             fn.argtypes = argtypes
@@ -195,6 +199,8 @@ class HipBackend:
         if self._partial_ml is None or self._partial_ml.numel() < need or self._partial_ml.device != torch.device(device):
             self._partial_ml = torch.empty(need, dtype=torch.float32, device=device)
 
+    GENERIC_PARTIAL_FLOATS = 1 << 25       # 128 MiB of partial results for the general attention kernel
+
     def paged_attention(self, qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len, out,
                         num_heads, num_kv_heads, head_dim, page_size, scale, window, max_q_len, max_ctx_len,
                         plan=None):
@@ -220,9 +226,24 @@ class HipBackend:
             return
         if head_dim % 4 or head_dim > 256:
             raise KernelError(f"paged_attention: head_dim {head_dim} is not a multiple of 4 up to 256")
+        # The general kernel cuts a token's keys into chunks and leaves the chunks of a token that has
+        # several in a buffer for a second kernel.  The buffer is made once at a fixed size (captured
+        # graphs hold its address); the tokens of a step run in as many launches as it takes.
+        longest = block_tables.shape[1] * page_size
+        max_ctx_len = min(max_ctx_len, longest) if max_ctx_len > 0 else longest
+        chunks = -(-max_ctx_len // self.lib.wllm_paged_attention_generic_chunk_keys())
+        per_token = num_heads * chunks * (head_dim + 2)
+        if per_token > self.GENERIC_PARTIAL_FLOATS:
+            raise KernelError(f"paged_attention: one token of {num_heads} heads over {max_ctx_len} keys needs "
+                              f"{per_token} floats of partial results, {self.GENERIC_PARTIAL_FLOATS} are reserved")
+        if self._generic_partial_o is None or self._generic_partial_o.device != qkv.device:
+            self._generic_partial_o = torch.empty(self.GENERIC_PARTIAL_FLOATS, dtype=torch.float32, device=qkv.device)
+        partial_tokens = self.GENERIC_PARTIAL_FLOATS // per_token
+        partial_ml = self._generic_partial_o[partial_tokens * num_heads * chunks * head_dim:]
         self._check(self.lib.wllm_paged_attention_generic(
             _ptr(qkv), _ptr(cache), int(qkv.dtype == torch.bfloat16), _ptr(block_tables), _ptr(token_segment),
-            _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out), qkv.shape[0], num_heads, num_kv_heads,
+            _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out), _ptr(self._generic_partial_o),
+            _ptr(partial_ml), partial_tokens, max_ctx_len, qkv.shape[0], num_heads, num_kv_heads,
             head_dim, page_size, block_tables.shape[1], scale, window, self._stream()), "paged_attention")
 
     @staticmethod
@@ -297,9 +318,15 @@ class HipBackend:
                 # many rows: the library's matrix-core product (float32 accumulation)
                 torch.mm(x, weight.t(), out=out)
                 return
+        # float32, few rows, a long K axis: the segments of K are summed by workgroups of their own
+        partial = None
+        if x.dtype == torch.float32 and m <= 16:
+            segments = self.lib.wllm_gemm_generic_segments(k)
+            if segments > 1:
+                partial = self._gemm_partial(segments * m * weight.shape[0], x.device)
         self._check(self.lib.wllm_gemm_generic(
             _ptr(x), _ptr(weight), int(x.dtype == torch.bfloat16), _ptr(out), int(out.dtype == torch.bfloat16),
-            x.shape[0], weight.shape[0], x.shape[1], self._stream()), "linear")
+            _ptr(partial), x.shape[0], weight.shape[0], x.shape[1], self._stream()), "linear")
 
     def gated_linear(self, x, weight, out, activation, scratch, tiles=None):
         self._on_gpu(x, weight, out, scratch, tiles)
