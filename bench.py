@@ -122,6 +122,12 @@ def measure_decode(model, batch: int, context: int, steps: int, warmup: int, blo
     return dt, mean_ctx
 
 
+class _StressDefaults:
+    """The stress workload's options as the default line runs it."""
+    seed, stress_requests, block_size, stress_pool_fraction, no_graphs, row_multiple = 0, 64, 16, 0.5, False, 256
+    dtype, shape = "bf16", "gemma-2b"
+
+
 def run_stress(model, args) -> dict:
     """Continuous batching under pressure: 64 requests at once, prompt lengths uniform in
     [128, 4096], output lengths uniform in [16, 512] (seeded), prompt portions of at most 512
@@ -178,7 +184,10 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the shape has")
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--no-graphs", action="store_true", help="do not replay captured graphs for decode")
-    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
+    ap.add_argument("--no-points", action="store_true", help="skip every point beside the line's own batch")
+    ap.add_argument("--points", default="all", choices=["basic", "all"],
+                    help="basic: batch 1 and 64 and the long context; all (default): also batch 128 and 256, batch 64 at "
+                         "longer contexts, the stress workload, float32 decoding and the Gemma-7B layer sizes")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--workload", default="decode", choices=["decode", "stress"],
                     help="decode: the contract's line; stress: continuous batching of 64 mixed requests")
@@ -225,18 +234,54 @@ def main() -> int:
 
         points = {}
         if not args.no_points:
-            for b, k in ((1, args.steps), (64, max(8, args.steps // 2))):
-                d, _ = measure_decode(model, b, args.context, k, min(args.warmup, 4), args.block_size, graphs)
-                points[f"decode_b{b}"] = round(k * b / d, 1)
+            few = min(args.warmup, 4)
+
+            def point(b, context, k):
+                d, _ = measure_decode(model, b, context, k, few, args.block_size, graphs)
+                return round(k * b / d, 1)
+
+            half = max(8, args.steps // 2)
+            points["decode_b1"] = point(1, args.context, args.steps)
+            points["decode_b64"] = point(64, args.context, half)
             # the same batch near the longest context the configuration allows
             limit = model.config.max_position_embeddings
             new_tokens = args.batch * (-(-limit // 2048)) + args.warmup + args.steps + 2      # as `measure_decode` counts them
             long_context = min(limit - 1024, (limit - new_tokens) // 256 * 256)
             if long_context > args.context:
-                d, _ = measure_decode(model, args.batch, long_context, args.steps, min(args.warmup, 4), args.block_size, graphs)
-                points[f"decode_b{args.batch}_context_{long_context}"] = round(args.steps * args.batch / d, 1)
+                points[f"decode_b{args.batch}_context_{long_context}"] = point(args.batch, long_context, args.steps)
+            if args.points == "all":
+                # further batch sizes and context lengths of the same configuration
+                points["decode_b128"] = point(128, args.context, half)
+                points["decode_b256"] = point(256, args.context, half)
+                for context in (4096, long_context):
+                    if args.context < context <= limit - 1024:
+                        points[f"decode_b64_context_{context}"] = point(64, context, half)
+                if args.dtype == "bf16" and args.shape == "gemma-2b" and args.layers is None:
+                    # the continuous-batching stress workload on the same model: generated tokens a second
+                    stress = run_stress(model, _StressDefaults)
+                    points["stress_64_requests_generated_tokens_per_s"] = stress["value"]
+                    points["stress_64_requests_seconds"] = stress["seconds"]
+        if not args.no_points and args.points == "all" and args.dtype == "bf16" and args.shape == "gemma-2b" and args.layers is None:
+            # the other measured configurations, each with all its layers: the true 32-bit path of the same
+            # sizes, and decoding at the Gemma-7B layer sizes
+            c2 = model.config
+            del model
+            torch.cuda.empty_cache()
+            other = build_model(shape, "fp32", args.seed)
+            d, _ = measure_decode(other, args.batch, args.context, half, 2, args.block_size, graphs)
+            points[f"fp32_{c2.num_hidden_layers}_layers_decode_b{args.batch}"] = round(half * args.batch / d, 1)
+            del other
+            torch.cuda.empty_cache()
+            big_shape = read_shape("gemma-7b")
+            other = build_model(big_shape, "bf16", args.seed)
+            for b, k in ((1, half), (8, half), (64, max(8, half // 2))):
+                d, _ = measure_decode(other, b, args.context, k, 2, args.block_size, graphs)
+                points[f"gemma7b_{big_shape['num_hidden_layers']}_layers_decode_b{b}"] = round(k * b / d, 1)
+            del other
+            torch.cuda.empty_cache()
+            model = None
 
-    c = model.config
+    c = model.config if model is not None else c2
     sizes = {"gemma-2b": "Gemma-2B", "gemma-7b": "Gemma-7B"}.get(args.shape, os.path.basename(args.shape))
     line = {
         "metric": f"decode tokens/s, {sizes} layer sizes, after {args.context:,}-token prompts",
