@@ -276,14 +276,19 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
         }
         // ---- out^T += V^T . P^T; the accumulators are rescaled only when some row's maximum moved ----
 #pragma unroll
+        for (int rt = 0; rt < RTW; ++rt) {
+            if (__builtin_amdgcn_readfirstlane(rescale[rt])) {      // one branch for the wavefront, not a select per number
+#pragma unroll
+                for (int t = 0; t < DT; ++t) acc[rt][t] *= alpha[rt];
+            }
+        }
+#pragma unroll
         for (int t = 0; t < DT; ++t) {
             PPack a;
             a.u = *reinterpret_cast<const uint4*>(&v_s[(16 * t + i) * SV + 8 * g]);
 #pragma unroll
-            for (int rt = 0; rt < RTW; ++rt) {
-                if (rescale[rt]) acc[rt][t] *= alpha[rt];
+            for (int rt = 0; rt < RTW; ++rt)
                 acc[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pv[rt].v, acc[rt][t], 0, 0, 0);
-            }
         }
     }
 #pragma unroll
@@ -315,6 +320,266 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
     }
 }
 
+// ---- the same kernel with the tiles moved into shared memory by the memory pipeline itself -------
+// For head sizes 64, 128 and 256 and pages of a multiple of 8 keys.  A lane's 16-byte load goes
+// straight to shared memory (lane l of a wavefront to base + 16 l), so staging costs no registers,
+// no writes to shared memory and no second barrier; two tiles of keys and values are held, and
+// the loads of block b+1 run while block b is multiplied.  Since a lane chooses its address, the
+// 16-byte chunks of a tile are placed so that fragment reads are free of bank conflicts: chunk c
+// of key row r lies at position c ^ (r % 8) of the row, chunk q (8 keys) of value row d at q ^
+// ((d / 2) % 4).  The keys of a block are staged in the order the second product wants them: row
+// 16 t + 4 g + v of the tile holds key 8 g + 4 t + v, so that after the first product a lane's eight
+// scores are the keys 8 g .. 8 g + 7 of its row, the same eight keys that chunk g of a value row holds.
+// Nothing is cleared in flight: in the blocks at the edges of a request the stale keys' values are
+// cleared in shared memory after they have landed (their scores are masked in any case).
+// 16 bytes per lane from global memory to shared memory without passing through registers: lane l's
+// bytes land at dst + 16 l; dst is the same for the whole wavefront (its address goes through M0).
+// Written as assembly on purpose.  Given the intrinsic, the compiler cannot tell which tile a later
+// read of shared memory touches and makes every such read wait for all loads in flight, the next
+// block's included, which is the overlap this kernel exists for.  So the compiler does not see
+// these loads; the kernel waits for them itself (s_waitcnt vmcnt(0) and a barrier before a tile
+// is read).  Loads the compiler does not know of can only make its own waits longer, never too short:
+// loads return in order, and it waits for one of its own by counting the loads issued after it.
+__device__ __forceinline__ void load_to_shared(const void* src, void* dst) {
+    const uint32_t lds_address = __builtin_amdgcn_readfirstlane(
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) void*)dst)));
+    // M0 is put back as it was: naming it as clobbered instead makes the compiler wait for every load in
+    // flight before the next read of shared memory
+    uint32_t saved_m0;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
+                 : "=&s"(saved_m0) : "v"(src), "s"(lds_address) : "memory");
+}
+
+template <int HD>
+__global__ void __launch_bounds__(kPrefillThreads, 2)
+paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict__ cache,
+                                   const int* __restrict__ block_tables, const int* __restrict__ items,
+                                   const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
+                                   const int* __restrict__ seg_ctx_len, bf16* __restrict__ out,
+                                   float* __restrict__ partial_o, float* __restrict__ partial_ml, int num_heads,
+                                   int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window) {
+    constexpr int DC = HD / 32, DT = HD / 16, CPR = HD / 8;       // CPR: 16-byte chunks of a key row
+    constexpr int kKeyInstr = kBlockKeys * CPR / 64, kValInstr = HD * 4 / 64;    // wavefront loads per tile
+    __shared__ __align__(16) uint16_t k_s0[kBlockKeys * HD], k_s1[kBlockKeys * HD];
+    __shared__ __align__(16) uint16_t v_s0[HD * kBlockKeys], v_s1[HD * kBlockKeys];
+    __shared__ int table_s[kMaxTablePages];
+
+    const int* item = items + static_cast<size_t>(blockIdx.x) * kPrefillItemInts;
+    const int seg = item[0], kvh = item[1], row_begin = item[2];
+    const int key_begin = item[3], key_end = item[4], partial_slot = item[5];
+    if (seg < 0) return;
+    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const int i = lane % 16, g = lane / 16;
+    const int group = num_heads / num_kv_heads;
+    const int q_start = seg_q_start[seg], q_len = seg_q_len[seg], ctx = seg_ctx_len[seg];
+    const int total_rows = q_len * group;
+    const int first_pos = ctx - q_len;
+    const int seg_lo = window > 0 ? max(0, first_pos - window + 1) : 0;
+    const int width = (num_heads + 2 * num_kv_heads) * HD;
+    const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * HD;
+    const size_t k_off = static_cast<size_t>(kvh) * page_size * HD;
+    const size_t v_off = (static_cast<size_t>(num_kv_heads) + kvh) * page_size * HD;
+
+    constexpr int kPrefillRows = kPrefillWaves * 16;
+    const int wr0 = row_begin + wave * 16;
+    const int row = wr0 + i;
+    const bool row_valid = row < total_rows;
+    const int tok = row_valid ? row / group : 0;
+    const int head = kvh * group + (row_valid ? row % group : 0);
+    const int pos = first_pos + tok;
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    bf16x8_t qreg[DC];
+    {
+        const bf16* qrow = qkv + static_cast<size_t>(q_start + tok) * width + static_cast<size_t>(head) * HD;
+#pragma unroll
+        for (int c = 0; c < DC; ++c) {
+            PPack p;
+            p.u = row_valid ? *reinterpret_cast<const uint4*>(qrow + c * 32 + 8 * g) : make_uint4(0, 0, 0, 0);
+            qreg[c] = p.v;
+        }
+    }
+    // the lowest position and the highest window start of the wavefront's rows
+    int t_pos_min, t_lo_max;
+    {
+        const int last = min(total_rows - 1, wr0 + 15);
+        t_pos_min = wr0 < total_rows ? first_pos + wr0 / group : -1;
+        const int pmax = first_pos + max(last, 0) / group;
+        t_lo_max = window > 0 ? max(0, pmax - window + 1) : 0;
+        if (last < wr0 + 15) t_pos_min = -1;      // a tile with rows beyond the segment always masks
+    }
+    const bool wave_active = wr0 < total_rows;
+    const int w_last_row = min(total_rows - 1, wr0 + 15);
+    const int w_hi = wave_active ? first_pos + w_last_row / group + 1 : 0;                       // exclusive
+    const int w_lo = window > 0 ? max(0, first_pos + wr0 / group - window + 1) : 0;
+    const int b_last_row = min(total_rows - 1, row_begin + kPrefillRows - 1);
+    const int b_hi = first_pos + b_last_row / group + 1;
+    const int b_lo = window > 0 ? max(0, first_pos + row_begin / group - window + 1) : 0;
+    const int blk_first = max(b_lo, key_begin) / kBlockKeys;
+    const int blk_end = (min(b_hi, key_end) + kBlockKeys - 1) / kBlockKeys;
+    const int page_base = blk_first * kBlockKeys / page_size;
+    if (blk_first < blk_end) {
+        const int* table_g = block_tables + static_cast<size_t>(seg) * max_pages + page_base;
+        const int page_last = (min(blk_end * kBlockKeys, ctx) - 1) / page_size;
+        const int count = min(min(max_pages - 1, page_last) - page_base + 1, kMaxTablePages);
+        for (int p = tid; p < count; p += kPrefillThreads) table_s[p] = table_g[p];
+    }
+
+    float4_t acc[DT];
+    float m_run = -INFINITY, l_run = 0.f;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
+    auto page_of = [&](int key, int& slot) -> int {
+        if (page_shift >= 0) {
+            slot = key & (page_size - 1);
+            return table_s[(key >> page_shift) - page_base];
+        }
+        slot = key % page_size;
+        return table_s[key / page_size - page_base];
+    };
+    // this lane's part of the loads of one block.  Keys: wavefront load q of the tile carries the chunks
+    // 64 q .. 64 q + 63 of the tile in shared-memory order; values likewise.
+    int k_row[(kKeyInstr + kPrefillWaves - 1) / kPrefillWaves], k_chunk[(kKeyInstr + kPrefillWaves - 1) / kPrefillWaves];
+#pragma unroll
+    for (int u = 0; u < (kKeyInstr + kPrefillWaves - 1) / kPrefillWaves; ++u) {
+        const int chunk_index = (wave + u * kPrefillWaves) * 64 + lane;       // position in the tile, in chunks
+        const int r = chunk_index / CPR;                                      // row of the tile
+        k_chunk[u] = (chunk_index % CPR) ^ (r % 8);                           // the chunk of the key's row that lies there
+        k_row[u] = 8 * ((r % 16) / 4) + 4 * (r / 16) + r % 4;                 // the key of the block that row r holds
+    }
+    const int v_q = (lane % 4) ^ ((lane / 8) % 4);                            // the chunk of 8 keys this lane moves, in every load
+    auto issue = [&](uint16_t* k_dst, uint16_t* v_dst, int kbase) {
+#pragma unroll
+        for (int u = 0; u < (kKeyInstr + kPrefillWaves - 1) / kPrefillWaves; ++u) {
+            const int q = wave + u * kPrefillWaves;
+            if (q < kKeyInstr) {
+                const int key = min(kbase + k_row[u], ctx - 1);
+                int slot;
+                const int page = page_of(key, slot);
+                const bf16* src = cache + static_cast<size_t>(page) * page_elems + k_off + static_cast<size_t>(slot) * HD + k_chunk[u] * 8;
+                load_to_shared(src, k_dst + q * 512);
+            }
+        }
+        {
+            const int key = min(kbase + 8 * v_q, (ctx - 1) & ~7);
+            int slot;
+            const int page = page_of(key, slot);
+            const bf16* src0 = cache + static_cast<size_t>(page) * page_elems + v_off + slot;
+#pragma unroll
+            for (int u = 0; u < (kValInstr + kPrefillWaves - 1) / kPrefillWaves; ++u) {
+                const int q = wave + u * kPrefillWaves;
+                if (q < kValInstr) {
+                    const int d = q * 16 + lane / 4;
+                    load_to_shared(src0 + static_cast<size_t>(d) * page_size, v_dst + q * 512);
+                }
+            }
+        }
+    };
+
+    __syncthreads();      // the block table is in shared memory
+    if (blk_first < blk_end) issue(k_s0, v_s0, blk_first * kBlockKeys);
+    // One block: its tiles are k_s and v_s, the next block's loads go to k_next and v_next.  The loop below
+    // names the two pairs of tiles in turn, so every address in shared memory is a constant plus a lane's
+    // fixed offset.
+    auto block = [&](int blk, const uint16_t* k_s, uint16_t* v_s, uint16_t* k_next, uint16_t* v_next) {
+        const int kbase = blk * kBlockKeys;
+        __builtin_amdgcn_s_waitcnt(0);   // this lane's loads of the block have landed
+        __syncthreads();                 // everyone's have, and everyone is done with the block before
+        if (blk + 1 < blk_end) issue(k_next, v_next, kbase + kBlockKeys);
+        if (kbase + kBlockKeys > ctx || kbase < seg_lo) {
+            // a block at the edge of the request: the values of keys that are not the request's are cleared
+            if (tid < HD) {
+                for (int kib = 0; kib < kBlockKeys; ++kib) {
+                    const int key = kbase + kib;
+                    if (key >= ctx || key < seg_lo) v_s[(tid * 4 + ((kib / 8) ^ ((tid / 2) % 4))) * 8 + kib % 8] = 0;
+                }
+            }
+            __syncthreads();
+        }
+        if (!wave_active || kbase >= w_hi || kbase + kBlockKeys <= w_lo) return;
+        // ---- scores: tile t2, lane (i, g) gets the keys 8 g + 4 t2 + v of the block ----
+        float sv[8];
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2) {
+            float4_t sc = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < DC; ++c) {
+                PPack a;
+                a.u = *reinterpret_cast<const uint4*>(&k_s[((16 * t2 + i) * CPR + ((4 * c + g) ^ (i % 8))) * 8]);
+                sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qreg[c], sc, 0, 0, 0);
+            }
+#pragma unroll
+            for (int v = 0; v < 4; ++v) sv[4 * t2 + v] = sc[v];
+        }
+        // ---- softmax bookkeeping ----
+        const bool inside = kbase + kBlockKeys - 1 <= t_pos_min && kbase >= t_lo_max;
+        if (!inside) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int key = kbase + 8 * g + e;
+                if (!(row_valid && key <= pos && key >= lo)) sv[e] = -INFINITY;
+            }
+        }
+        float tile_max = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
+        const float m_new = fmaxf(m_run, tile_max);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float mc = m_use * scale_log2e;
+        const float alpha = exp2_probability(fmaf(m_run, scale_log2e, -mc));
+        float pe[8], psum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            pe[e] = exp2_probability(fmaf(sv[e], scale_log2e, -mc));       // exp2(-inf) = 0 for masked keys
+            psum += pe[e];
+        }
+        PPack pv;
+        pv.u = make_uint4(pack2_bf16(pe[0], pe[1]), pack2_bf16(pe[2], pe[3]), pack2_bf16(pe[4], pe[5]), pack2_bf16(pe[6], pe[7]));
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        // ---- out^T += V^T . P^T; the accumulators are rescaled only when some row's maximum moved: one
+        // branch for the whole wavefront around all of them (a test per accumulator becomes a multiply and a
+        // select for each of its 64 numbers, whether or not anything moved) ----
+        if (__builtin_amdgcn_readfirstlane(__any(alpha != 1.f))) {
+#pragma unroll
+            for (int t = 0; t < DT; ++t) acc[t] *= alpha;
+        }
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+            PPack a;
+            a.u = *reinterpret_cast<const uint4*>(&v_s[((16 * t + i) * 4 + (g ^ ((i / 2) % 4))) * 8]);
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pv.v, acc[t], 0, 0, 0);
+        }
+    };
+    for (int blk = blk_first; blk < blk_end; blk += 2) {
+        block(blk, k_s0, v_s0, k_s1, v_s1);
+        if (blk + 1 < blk_end) block(blk + 1, k_s1, v_s1, k_s0, v_s0);
+    }
+    float l = l_run;
+    l += __shfl_xor(l, 16, kWave);
+    l += __shfl_xor(l, 32, kWave);
+    if (!row_valid) return;
+    if (partial_slot >= 0) {
+        const size_t slot = static_cast<size_t>(partial_slot) + wave;
+        float* po = partial_o + (slot * 16 + i) * HD;
+#pragma unroll
+        for (int t = 0; t < DT; ++t)
+            *reinterpret_cast<float4*>(po + t * 16 + 4 * g) = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+        if (g == 0) *reinterpret_cast<float2*>(partial_ml + (slot * 16 + i) * 2) = make_float2(m_run, l);
+        return;
+    }
+    const float inv = 1.f / l;
+    bf16* orow = out + (static_cast<size_t>(q_start + tok) * num_heads + head) * HD;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+        uint2 w;
+        w.x = pack2_bf16(acc[t][0] * inv, acc[t][1] * inv);
+        w.y = pack2_bf16(acc[t][2] * inv, acc[t][3] * inv);
+        *reinterpret_cast<uint2*>(orow + t * 16 + 4 * g) = w;
+    }
+}
+
 // Returns 0, a HIP error code, or -1 for sizes this kernel does not take.
 WLLM_API int wllm_paged_attention_prefill(const void* qkv, const void* cache, const int* block_tables,
                                           const int* items, int num_items, int rows_per_item, const int* seg_q_start,
@@ -327,6 +592,18 @@ WLLM_API int wllm_paged_attention_prefill(const void* qkv, const void* cache, co
     if (rows_per_item != 64) return -1;
     if (num_items <= 0) return 0;
     const float scale_log2e = scale * 1.4426950408889634f;
+    if (page_size % 8 == 0 && (head_dim == 64 || head_dim == 128 || head_dim == 256)) {
+#define LAUNCH_DMA(HD)                                                                                              \
+    paged_attention_prefill_dma_kernel<HD><<<num_items, kPrefillThreads, 0, stream>>>(                              \
+        static_cast<const bf16*>(qkv), static_cast<const bf16*>(cache), block_tables, items, seg_q_start, seg_q_len, \
+        seg_ctx_len, static_cast<bf16*>(out), partial_o, partial_ml, num_heads, num_kv_heads, page_size, max_pages, \
+        scale_log2e, window)
+        if (head_dim == 64) LAUNCH_DMA(64);
+        else if (head_dim == 128) LAUNCH_DMA(128);
+        else LAUNCH_DMA(256);
+#undef LAUNCH_DMA
+        return launch_status();
+    }
 #define LAUNCH_RTW(HD, RTW)                                                                                         \
     paged_attention_prefill_kernel<HD, RTW><<<num_items, kPrefillThreads, 0, stream>>>(                             \
         static_cast<const bf16*>(qkv), static_cast<const bf16*>(cache), block_tables, items, seg_q_start, seg_q_len, \
