@@ -323,7 +323,9 @@ def test_paged_attention_finds_one_far_key(dtype):
 @pytest.mark.parametrize("m,n,k", [(1, 100, 64), (7, 777, 250), (65, 130, 96), (128, 64, 2048), (3, 2560, 2048),
                                    (8, 2048, 16384), (17, 777, 96), (33, 1000, 128), (64, 4099, 2048), (49, 32768, 256),
                                    (200, 777, 64), (2, 16, 32), (16, 20, 1056), (16, 2048, 8192), (12, 100, 4128),
-                                   (9, 3072, 24576), (11, 16500, 320)])
+                                   (9, 3072, 24576), (11, 16500, 320),
+                                   # more than 64 rows of an unsplit product (logits of many rows): groups of 64 rows in one launch
+                                   (65, 24600, 64), (130, 25001, 96), (256, 26000, 128), (200, 50000, 32)])
 def test_linear(dtype, m, n, k):
     torch.manual_seed(4)
     for out_dtype in {dtype, torch.float32}:

@@ -65,14 +65,28 @@ template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float4_t v) {
 // TILED: w is stored tile by tile (see `wllm_tile_weight`): a tile of 16 rows and 32 keys as the 16
 // bytes of each of the 64 lanes in lane order, the tiles of a band of 16 rows one after the other along
 // K, so a wavefront streams one contiguous run.
+//
+// More than 64 rows (row_groups > 1, unsplit products only): groups of 64 rows are made by workgroups of
+// their own that read the same weights.  The workgroups of a tile's row groups get indices that are 8
+// apart, so they are dispatched one after the other to the same XCD (workgroup index modulo 8) and the
+// later ones find the weights in that XCD's L2 instead of asking HBM for them again.
 template <int MT, int NT, typename TO, bool TILED>
 __global__ void __launch_bounds__(256)
 gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* __restrict__ out,
-                   float* __restrict__ partial, int M, int N, int K, int k_per_split, int chunk) {
+                   float* __restrict__ partial, int M, int N, int K, int k_per_split, int chunk, int row_groups) {
     extern __shared__ uint4 xs[];                 // [MT*16][chunk/8 + 1]
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const int i = lane % 16, g = lane / 16;
-    const int n0 = (blockIdx.x * 4 + wave) * 16 * NT;
+    int tile_group = blockIdx.x;                  // which 64 * NT weight rows
+    if (row_groups > 1) {
+        const int xcd = blockIdx.x % 8, j = blockIdx.x / 8;
+        const int rg = j % row_groups;
+        tile_group = (j / row_groups) * 8 + xcd;
+        x += static_cast<size_t>(rg) * 64 * K;
+        out += static_cast<size_t>(rg) * 64 * N;
+        M = min(64, M - rg * 64);
+    }
+    const int n0 = (tile_group * 4 + wave) * 16 * NT;
     const int k_begin = blockIdx.y * k_per_split, k_end = min(K, k_begin + k_per_split);
     const int stride = chunk / 8 + 1;             // in uint4; the odd stride spreads rows over the banks
     constexpr int kStep = TILED ? 512 : 32;       // elements from one step of 32 keys to the next
@@ -198,11 +212,14 @@ __global__ void split_sum_kernel(const float* __restrict__ partial, TO* __restri
 // are the result and nothing adds them.
 WLLM_API int wllm_gemm_skinny(const void* x, const void* w, int tiled, void* out, int out_bf16, float* partial, int M,
                               int N, int K, int splits, int chunk, hipStream_t stream) {
-    if (M < 1 || M > 64 || K % 32 != 0 || splits < 1 || K % splits != 0 || (K / splits) % 32 != 0 || chunk % 32 != 0)
+    if (M < 1 || K % 32 != 0 || splits < 1 || K % splits != 0 || (K / splits) % 32 != 0 || chunk % 32 != 0)
         return -1;
     // every result needs somewhere to go: a split product its partial sums, an unsplit one its output
     if ((splits > 1 && partial == nullptr) || (splits == 1 && out == nullptr)) return -1;
-    const int mt = (M + 15) / 16;
+    // more than 64 rows: groups of 64 rows by workgroups of their own, for unsplit products
+    const int row_groups = (M + 63) / 64;
+    if (row_groups > 1 && splits != 1) return -1;
+    const int mt = row_groups > 1 ? 4 : (M + 15) / 16;
     const int k_per_split = K / splits;
     if (chunk > k_per_split) chunk = k_per_split;
     const size_t smem = static_cast<size_t>(mt) * 16 * (chunk / 8 + 1) * sizeof(uint4);
@@ -220,10 +237,16 @@ WLLM_API int wllm_gemm_skinny(const void* x, const void* w, int tiled, void* out
         while (nt < 4 && chunk % ((16 / nt) * 32) != 0) nt *= 2;
         if (chunk % ((16 / nt) * 32) != 0) return -1;     // a register's step is fixed by its place in the batch
     }
-    const dim3 grid((N + 64 * nt - 1) / (64 * nt), splits);
+    // with row groups the tile groups are padded to a multiple of 8, one stripe per XCD (tile groups beyond
+    // the last hold no live weight rows and write nothing)
+    const int tile_groups = (N + 64 * nt - 1) / (64 * nt);
+    const long long blocks = row_groups > 1 ? static_cast<long long>((tile_groups + 7) / 8 * 8) * row_groups : tile_groups;
+    if (blocks > 0x7fffffffLL) return -1;
+    const dim3 grid(static_cast<unsigned>(blocks), splits);
 #define LAUNCH_T(MT, NT, TO, T)                                                                                  \
     gemm_skinny_kernel<MT, NT, TO, T><<<grid, 256, smem, stream>>>(static_cast<const bf16*>(x), static_cast<const bf16*>(w), \
-                                                                   static_cast<TO*>(out), partial, M, N, K, k_per_split, chunk)
+                                                                   static_cast<TO*>(out), partial, M, N, K, k_per_split, chunk, \
+                                                                   row_groups)
 #define LAUNCH(MT, NT, TO)                  \
     if (tiled) LAUNCH_T(MT, NT, TO, true);  \
     else LAUNCH_T(MT, NT, TO, false)

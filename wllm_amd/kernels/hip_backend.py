@@ -130,13 +130,14 @@ class HipBackend:
             _ptr(cache), cache.shape[0] if cache is not None else 0, qkv.shape[0], num_heads, num_kv_heads, head_dim,
             rotary_dim, page_size, self._stream()), "rope_and_cache_write")
 
-    @staticmethod
-    def linear_residual_takes(rows: int, dtype, out_features: int, in_features: int) -> bool:
+    RESIDUAL_MAX_K = 4096
+
+    def linear_residual_takes(self, rows: int, dtype, out_features: int, in_features: int) -> bool:
         """The product that adds into the residual stream: bfloat16, at most 16 rows, whole bands of
         16 columns.  Its workgroups are the bands; with a long K axis there are too few of them for the
         weight to stream from all compute units, and the split product with its norm kernel is faster."""
         return (dtype == torch.bfloat16 and 1 <= rows <= 16 and out_features % 16 == 0 and in_features % 32 == 0
-                and in_features <= 4096)
+                and in_features <= self.RESIDUAL_MAX_K)
 
     def linear_residual(self, x, weight, tiles, residual, sumsq):
         self._on_gpu(x, weight, tiles, residual, sumsq)
@@ -290,7 +291,7 @@ class HipBackend:
         m, k = x.shape
         n = weight.shape[0]
         splits = self.skinny_split(n, k)
-        chunk = self.SKINNY_CHUNK[-(-m // 16)]
+        chunk = self.SKINNY_CHUNK[min(4, -(-m // 16))]
         w, tiled = (tiles, 1) if tiles is not None else (weight, 0)
         if out.dim() == 3:      # the caller adds the partial sums later
             self._check(self.lib.wllm_gemm_skinny(_ptr(x), _ptr(w), tiled, c_void_p(0), 0, _ptr(out), m, n, k, splits,
@@ -308,9 +309,12 @@ class HipBackend:
             if self.skinny_takes(x.dtype, m, k):
                 self._skinny(x, weight, out, tiles)
                 return
+            if k % 32 == 0 and out.dtype == torch.float32 and self.skinny_split(weight.shape[0], k) == 1:
+                # float32 results from bfloat16 operands (logits at many rows): the few-row kernel with a
+                # workgroup per 64 rows, placed so that the weights come from HBM once
+                self._skinny(x, weight, out, tiles)
+                return
             if k % 32 == 0 and out.dtype == torch.float32:
-                # float32 results from bfloat16 operands (logits at many rows): the few-row kernel
-                # in blocks of 64 rows
                 for r in range(0, m, 64):
                     self._skinny(x[r:r + 64], weight, out[r:r + 64], tiles)
                 return
