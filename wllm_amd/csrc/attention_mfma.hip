@@ -62,75 +62,100 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
                             int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window) {
     constexpr int DC = HD / 32;   // 32-wide chunks of the head for the score product
     constexpr int DT = HD / 16;   // 16-row tiles of out^T
-    // Shared memory, used twice.  First each wavefront turns its block of keys, which it reads
-    // from the cache row by row (whole key rows: contiguous runs the memory system streams much
-    // faster than the 64-byte pieces a fragment load straight from the cache would ask for), into
-    // fragments: [4 wavefronts][32 keys][HD + 8] bfloat16, rows padded so that the fragment reads
-    // spread over the banks.  Then, after a barrier, the merge buffer: two slots of [16 rows][HD + 2]
-    // floats.
+    // Shared memory, a part for each wavefront, used twice.  First the wavefront turns its block of
+    // keys, which it reads from the cache row by row (whole key rows: contiguous runs the memory
+    // system streams much faster than the 64-byte pieces a fragment load straight from the cache
+    // would ask for), into fragments: [32 keys][HD + 8] bfloat16, rows padded so that the fragment
+    // reads spread over the banks.  Then it leaves its sums there for the merge: [16 rows][HD + 4]
+    // floats and the rows' maxima and sums.
     constexpr int kKeyStride = HD + 8;                                      // elements
-    constexpr int kStageBytes = 4 * kKeysPerBlock * kKeyStride * 2;
-    constexpr int kMergeBytes = 2 * kRowsPerTile * (HD + 2) * 4;
-    __shared__ __align__(16) unsigned char shared_raw[kStageBytes > kMergeBytes ? kStageBytes : kMergeBytes];
-    float (*merge_s)[kRowsPerTile * (HD + 2)] = reinterpret_cast<float (*)[kRowsPerTile * (HD + 2)]>(shared_raw);
+    constexpr int kPartBytes = kKeysPerBlock * kKeyStride * 2;
+    constexpr int kMergeStride = HD + 4;                                    // floats
+    static_assert(kRowsPerTile * kMergeStride * 4 + kRowsPerTile * 2 * 4 <= kPartBytes, "the merge fits a wavefront's part");
+    __shared__ __align__(16) unsigned char shared_raw[4 * kPartBytes];
 
     const int* item = items + static_cast<size_t>(blockIdx.x) * kItemInts;
     const int seg = item[0], kvh = item[1], row_begin = item[2];
-    constexpr int row_tiles = 1;            // one tile of 16 rows; the four wavefronts split the keys
     const int key_begin = item[4], key_end = item[5], partial_slot = item[6];
     if (seg < 0) return;    // padding item
-    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x % kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int i = lane % 16, g = lane / 16;
-    const int key_splits = 4 / row_tiles;           // wavefronts that share a row tile
-    const int rt = wave % row_tiles, ks = wave / row_tiles;
 
-    // ---- The walk over the keys depends on the item alone: the host cut the item's keys to what
-    //      its rows can need (from the lowest window start of the first row to the last row's
-    //      position).  The loads of the first block of keys and values are issued before anything
-    //      else is read, so they wait for the item and the block table only; the request's
-    //      lengths and the queries arrive while they are in flight. ----
+    // ---- The request's lengths and this lane's queries are asked for first: they arrive while the
+    //      addresses of the keys and values are worked out. ----
+    const int q_start = seg_q_start[seg], q_len = seg_q_len[seg], ctx = seg_ctx_len[seg];
     const int group = num_heads / num_kv_heads;
     const int width = (num_heads + 2 * num_kv_heads) * HD;
+    const int total_rows = q_len * group;
+    const int first_pos = ctx - q_len;
+    const int seg_lo = window > 0 ? max(0, first_pos - window + 1) : 0;   // keys below may be given back
+    const int row = row_begin + i;
+    const bool row_valid = row < total_rows;
+    const int tok = row_valid ? row / group : 0;
+    const int head = kvh * group + (row_valid ? row % group : 0);
+    const int pos = first_pos + tok;
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    // An item's keys lie within one aligned group of 128 (the host's chunk), so each of the four
+    // wavefronts has at most one block of 32 keys and nothing is carried from block to block.
+    const int blk_first = key_begin / kKeysPerBlock;
+    const int blk_end = (key_end + kKeysPerBlock - 1) / kKeysPerBlock;
+    const int blk = blk_first + wave;
+    const bool has_block = blk < blk_end;
+    bf16x8_t qreg[DC];
+    if (has_block) {
+        const bf16* qrow = qkv + static_cast<size_t>(q_start + tok) * width + static_cast<size_t>(head) * HD;
+#pragma unroll
+        for (int c = 0; c < DC; ++c) {
+            Pack16 p;
+            p.u = row_valid ? *reinterpret_cast<const uint4*>(qrow + c * 32 + 8 * g) : make_uint4(0, 0, 0, 0);
+            qreg[c] = p.v;
+        }
+    }
+
     const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * HD;
     const size_t k_off = static_cast<size_t>(kvh) * page_size * HD;
     const size_t v_off = (static_cast<size_t>(num_kv_heads) + kvh) * page_size * HD;
     const int* table = block_tables + static_cast<size_t>(seg) * max_pages;
-    const int blk_first = key_begin / kKeysPerBlock;
-    const int blk_end = (key_end + kKeysPerBlock - 1) / kKeysPerBlock;
     // a block's keys as the cache holds them: 32 rows of HD, 16 bytes a lane and load
     constexpr int kPieces = HD / 8;                 // 16-byte pieces of a key row
     uint4_t kraw[DT];                               // 32 * kPieces / 64 = HD / 16 loads a lane
     Pack16 va_[DT];
-    // All loads of a block are issued before the first product needs one, so a block costs one
-    // trip to memory.  Keys beyond the request are masked later; their table entry is clamped to
-    // the table's width (entries beyond a request's pages name a valid page), not to the length.
-    auto issue = [&](int blk) {
-        const int kbase = blk * kKeysPerBlock;
+    const int kbase = blk * kKeysPerBlock;
+    float4_t acc[DT];
+    float m_run = -INFINITY, l_run = 0.f;
+    uint16_t* stage = reinterpret_cast<uint16_t*>(shared_raw + wave * kPartBytes);
+    if (has_block) {
+        // All loads of the block are issued before the first product needs one, so a block costs
+        // one trip to memory after the block table's.  Keys beyond the request are masked later;
+        // their table entry is clamped to the table's width (entries beyond a request's pages name
+        // a valid page), not to the length.  A key's page and slot come from its place within the
+        // block and one division a wavefront: the quotient by the page size as a float product,
+        // exact for the few hundred values it is asked for here.
+        const int base_page = kbase / page_size, base_slot = kbase % page_size;     // the same for all lanes
+        const float inv_page = 1.f / static_cast<float>(page_size);
+        auto place = [&](int within, int& page_index, int& slot) {
+            const int x = base_slot + within;                                  // < page_size + 32
+            const int q = static_cast<int>((static_cast<float>(x) + 0.5f) * inv_page);
+            page_index = min(base_page + q, max_pages - 1);
+            slot = x - q * page_size;
+        };
         const bf16* kpiece[DT];
 #pragma unroll
         for (int j = 0; j < DT; ++j) {
             // piece f of the block: key f / kPieces, its 8 elements f % kPieces; a wavefront's load
             // covers whole consecutive rows
             const int f = j * kWave + lane;
-            const int kk = kbase + f / kPieces;
-            const int page = table[min(kk / page_size, max_pages - 1)];
-            kpiece[j] = cache + static_cast<size_t>(page) * page_elems + k_off +
-                        static_cast<size_t>(kk % page_size) * HD + (f % kPieces) * 8;
+            int page_index, slot;
+            place(f / kPieces, page_index, slot);
+            kpiece[j] = cache + static_cast<size_t>(table[page_index]) * page_elems + k_off +
+                        static_cast<size_t>(slot) * HD + (f % kPieces) * 8;
         }
         int vpage0, vslot0, vpage1 = 0, vslot1 = 0;
-        if (V16) {
-            const int kk = kbase + 8 * g;
-            vpage0 = table[min(kk / page_size, max_pages - 1)];
-            vslot0 = kk % page_size;
-        } else {
-            const int ka = kbase + 4 * g, kb = kbase + 16 + 4 * g;
-            vpage0 = table[min(ka / page_size, max_pages - 1)];
-            vslot0 = ka % page_size;
-            vpage1 = table[min(kb / page_size, max_pages - 1)];
-            vslot1 = kb % page_size;
-        }
-        const bf16* vbase0 = cache + static_cast<size_t>(vpage0) * page_elems + v_off + vslot0;
-        const bf16* vbase1 = cache + static_cast<size_t>(vpage1) * page_elems + v_off + vslot1;
+        place(V16 ? 8 * g : 4 * g, vpage0, vslot0);
+        if (!V16) place(16 + 4 * g, vpage1, vslot1);
+        const bf16* vbase0 = cache + static_cast<size_t>(table[vpage0]) * page_elems + v_off + vslot0;
+        const bf16* vbase1 = cache + static_cast<size_t>(V16 ? 0 : table[vpage1]) * page_elems + v_off + vslot1;
 #pragma unroll
         for (int j = 0; j < DT; ++j) kraw[j] = *reinterpret_cast<const uint4_t*>(kpiece[j]);
 #pragma unroll
@@ -143,51 +168,13 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
                 va_[t].half[1] = *reinterpret_cast<const uint2*>(vbase1 + drow);
             }
         }
-    };
-    // An item's keys lie within one aligned group of 128 (the host's chunk), so each of the four
-    // wavefronts has at most one block of 32 keys and nothing is carried from block to block.
-    const int blk = blk_first + ks;
-    const bool has_block = blk < blk_end && blk < blk_first + key_splits;
-    if (has_block) issue(blk);
-
-    const int q_start = seg_q_start[seg], q_len = seg_q_len[seg], ctx = seg_ctx_len[seg];
-    const int total_rows = q_len * group;
-    const int first_pos = ctx - q_len;
-    const int seg_lo = window > 0 ? max(0, first_pos - window + 1) : 0;   // keys below may be given back
-    const int row = row_begin + i;
-    const bool row_valid = row < total_rows;
-    const int tok = row_valid ? row / group : 0;
-    const int head = kvh * group + (row_valid ? row % group : 0);
-    const int pos = first_pos + tok;
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-
-    float4_t acc[DT];
-    float m_run = -INFINITY, l_run = 0.f;
-    if (has_block) {
-        // the queries of this lane's row
-        bf16x8_t qreg[DC];
-        const bf16* qrow = qkv + static_cast<size_t>(q_start + tok) * width + static_cast<size_t>(head) * HD;
-#pragma unroll
-        for (int c = 0; c < DC; ++c) {
-            Pack16 p;
-            p.u = row_valid ? *reinterpret_cast<const uint4*>(qrow + c * 32 + 8 * g) : make_uint4(0, 0, 0, 0);
-            qreg[c] = p.v;
-        }
-        const int kbase = blk * kKeysPerBlock;
         const bool edge = kbase < seg_lo || kbase + kKeysPerBlock > ctx;
         // ---- the keys through this wavefront's part of shared memory, then the scores of two
         //      tiles of 16 keys ----
-        uint16_t* stage = reinterpret_cast<uint16_t*>(shared_raw) + wave * (kKeysPerBlock * kKeyStride);
-        {
-            // piece f = j * 64 + lane lies (64 / kPieces) rows further with every j when 64 is a
-            // multiple of kPieces; in general its row and place are computed per piece
-            const int f0 = lane;
 #pragma unroll
-            for (int j = 0; j < DT; ++j) {
-                const int f = f0 + j * kWave;
-                uint16_t* dst = stage + (f / kPieces) * kKeyStride + (f % kPieces) * 8;
-                *reinterpret_cast<uint4_t*>(dst) = kraw[j];
-            }
+        for (int j = 0; j < DT; ++j) {
+            const int f = lane + j * kWave;
+            *reinterpret_cast<uint4_t*>(stage + (f / kPieces) * kKeyStride + (f % kPieces) * 8) = kraw[j];
         }
         float4_t s[2];
 #pragma unroll
@@ -251,61 +238,66 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
         for (int t = 0; t < DT; ++t) acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
     }
 
-    // ---- merge the wavefronts that split the keys of one row tile ----
-    // lane (i, g) holds out^T[16t + 4g + v][row i]: element d = 16t + 4g + v of row i
-    for (int step = key_splits / 2; step >= 1; step /= 2) {
-        // wavefronts with ks in [step, 2*step) hand over to ks - step
-        __syncthreads();
-        const bool sender = ks >= step && ks < 2 * step;
-        const bool receiver = ks < step;
-        const int slot = (rt + row_tiles * (ks % step)) % 2;   // at most two pairs are live per step
-        float* buf = merge_s[slot] + i * (HD + 2);
-        if (sender) {
-#pragma unroll
-            for (int t = 0; t < DT; ++t)
-#pragma unroll
-                for (int v = 0; v < 4; ++v) buf[t * 16 + 4 * g + v] = acc[t][v];
-            if (g == 0) {
-                buf[HD] = m_run;
-                buf[HD + 1] = l_run;
-            }
-        }
-        __syncthreads();
-        if (receiver) {
-            const float m_o = buf[HD], l_o = buf[HD + 1];
-            const float m_new = fmaxf(m_run, m_o);
-            const float m_use = m_new == -INFINITY ? 0.f : m_new;
-            const float a_me = exp2f((m_run - m_use) * scale_log2e), a_o = exp2f((m_o - m_use) * scale_log2e);
-#pragma unroll
-            for (int t = 0; t < DT; ++t)
-#pragma unroll
-                for (int v = 0; v < 4; ++v) acc[t][v] = acc[t][v] * a_me + buf[t * 16 + 4 * g + v] * a_o;
-            l_run = l_run * a_me + l_o * a_o;
-            m_run = m_new;
-        }
-    }
-
-    if (ks != 0 || !row_valid) return;
-    if (partial_slot < 0) {
-        const float inv = 1.f / l_run;
-        bf16* orow = out + (static_cast<size_t>(q_start + tok) * num_heads + head) * HD;
-#pragma unroll
-        for (int t = 0; t < DT; ++t) {
-            uint2 w;
-            w.x = pack2_bf16(acc[t][0] * inv, acc[t][1] * inv);
-            w.y = pack2_bf16(acc[t][2] * inv, acc[t][3] * inv);
-            *reinterpret_cast<uint2*>(orow + t * 16 + 4 * g) = w;
-        }
-    } else {
-        const size_t prow = static_cast<size_t>(partial_slot) * kRowsPerTile + (row - row_begin);
-        float* po = partial_o + prow * HD;
+    // ---- merge: every wavefront leaves its sums in its own part of shared memory (it has read its
+    //      keys from there already), then each takes every fourth tile of 16 elements of the head and
+    //      combines the four wavefronts' sums of that tile, always in the order 0, 1, 2, 3.
+    //      lane (i, g) holds out^T[16t + 4g + v][row i]: elements d = 16t + 4g + v of row i ----
+    {
+        float* mine = reinterpret_cast<float*>(stage);
 #pragma unroll
         for (int t = 0; t < DT; ++t)
-            *reinterpret_cast<float4_t*>(po + t * 16 + 4 * g) = acc[t];
+            *reinterpret_cast<float4_t*>(mine + i * kMergeStride + t * 16 + 4 * g) = acc[t];
         if (g == 0) {
-            partial_ml[prow * 2] = m_run;
-            partial_ml[prow * 2 + 1] = l_run;
+            mine[kRowsPerTile * kMergeStride + 2 * i] = m_run;
+            mine[kRowsPerTile * kMergeStride + 2 * i + 1] = l_run;
         }
+    }
+    __syncthreads();
+    if (!row_valid) return;
+    float m_of[4], l_of[4], f_of[4];
+    float m_all = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        const float* part = reinterpret_cast<const float*>(shared_raw + w * kPartBytes);
+        m_of[w] = part[kRowsPerTile * kMergeStride + 2 * i];
+        l_of[w] = part[kRowsPerTile * kMergeStride + 2 * i + 1];
+        m_all = fmaxf(m_all, m_of[w]);
+    }
+    const float m_use = m_all == -INFINITY ? 0.f : m_all;
+    float l_all = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        f_of[w] = exp2f((m_of[w] - m_use) * scale_log2e);       // 0 for a wavefront without keys
+        l_all = fmaf(l_of[w], f_of[w], l_all);
+    }
+    const float inv = 1.f / l_all;
+    bf16* orow = out + (static_cast<size_t>(q_start + tok) * num_heads + head) * HD;
+    const size_t prow = static_cast<size_t>(max(partial_slot, 0)) * kRowsPerTile + (row - row_begin);
+    float* po = partial_o + prow * HD;
+#pragma unroll
+    for (int t0 = 0; t0 < DT; t0 += 4) {
+        const int t = t0 + wave;
+        if (t >= DT) break;
+        float4_t sum = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float* part = reinterpret_cast<const float*>(shared_raw + w * kPartBytes);
+            const float4_t v = *reinterpret_cast<const float4_t*>(part + i * kMergeStride + t * 16 + 4 * g);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sum[e] = fmaf(v[e], f_of[w], sum[e]);
+        }
+        if (partial_slot < 0) {
+            uint2 w2;
+            w2.x = pack2_bf16(sum[0] * inv, sum[1] * inv);
+            w2.y = pack2_bf16(sum[2] * inv, sum[3] * inv);
+            *reinterpret_cast<uint2*>(orow + t * 16 + 4 * g) = w2;
+        } else {
+            *reinterpret_cast<float4_t*>(po + t * 16 + 4 * g) = sum;
+        }
+    }
+    if (partial_slot >= 0 && wave == 0 && g == 0) {
+        partial_ml[prow * 2] = m_all;
+        partial_ml[prow * 2 + 1] = l_all;
     }
 }
 
