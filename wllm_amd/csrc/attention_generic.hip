@@ -179,7 +179,10 @@ paged_attention_generic_kernel(const T* __restrict__ qkv, const T* __restrict__ 
             if (c == 0) p_s[g * kTileKeys + j] = p;
         }
     }
+    // lanes read below what other lanes of the wavefront wrote above: no reordering by the
+    // scheduler, and the compiler is told that the memory changed
     __builtin_amdgcn_wave_barrier();
+    asm volatile("" ::: "memory");
 
     // ---- weighted sum: lane = element of the head; the keys in ascending order ----
     float acc[kGroupMax][DPL];

@@ -53,7 +53,7 @@ union Pack16 {
 __device__ __forceinline__ uint16_t bf16_bits(float f) { return from_float<bf16>(f).bits; }
 
 template <int HD, bool V16>
-__global__ void __launch_bounds__(256, 2)
+__global__ void __launch_bounds__(256, 3)
 paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict__ cache,
                             const int* __restrict__ block_tables, const int* __restrict__ items,
                             const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
@@ -62,17 +62,19 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
                             int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window) {
     constexpr int DC = HD / 32;   // 32-wide chunks of the head for the score product
     constexpr int DT = HD / 16;   // 16-row tiles of out^T
-    // Shared memory, a part for each wavefront, used twice.  First the wavefront turns its block of
-    // keys, which it reads from the cache row by row (whole key rows: contiguous runs the memory
-    // system streams much faster than the 64-byte pieces a fragment load straight from the cache
-    // would ask for), into fragments: [32 keys][HD + 8] bfloat16, rows padded so that the fragment
-    // reads spread over the banks.  Then it leaves its sums there for the merge: [16 rows][HD + 4]
-    // floats and the rows' maxima and sums.
+    // Shared memory, a part for each wavefront, used four times: three workgroups share a compute
+    // unit's 160 KB.  The wavefront turns its block of keys, which it reads from the cache row by row
+    // (whole key rows: contiguous runs the memory system streams much faster than the 64-byte pieces
+    // a fragment load straight from the cache would ask for), into fragments, the 16 keys of the
+    // first score tile and then the 16 of the second: [16 keys][HD + 8] bfloat16, rows padded so that
+    // the fragment reads spread over the banks.  Then it leaves its sums there for the merge, one
+    // half of the head after the other: [16 rows][HD / 2 + 4] floats.
     constexpr int kKeyStride = HD + 8;                                      // elements
-    constexpr int kPartBytes = kKeysPerBlock * kKeyStride * 2;
-    constexpr int kMergeStride = HD + 4;                                    // floats
-    static_assert(kRowsPerTile * kMergeStride * 4 + kRowsPerTile * 2 * 4 <= kPartBytes, "the merge fits a wavefront's part");
+    constexpr int kPartBytes = 16 * kKeyStride * 2;
+    constexpr int kMergeStride = HD / 2 + 4;                                // floats
+    static_assert(kRowsPerTile * kMergeStride * 4 <= kPartBytes, "half of the sums fits a wavefront's part");
     __shared__ __align__(16) unsigned char shared_raw[4 * kPartBytes];
+    __shared__ float row_max_s[4][kRowsPerTile], row_sum_s[4][kRowsPerTile];
 
     const int* item = items + static_cast<size_t>(blockIdx.x) * kItemInts;
     const int seg = item[0], kvh = item[1], row_begin = item[2];
@@ -169,23 +171,30 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
             }
         }
         const bool edge = kbase < seg_lo || kbase + kKeysPerBlock > ctx;
-        // ---- the keys through this wavefront's part of shared memory, then the scores of two
-        //      tiles of 16 keys ----
-#pragma unroll
-        for (int j = 0; j < DT; ++j) {
-            const int f = lane + j * kWave;
-            *reinterpret_cast<uint4_t*>(stage + (f / kPieces) * kKeyStride + (f % kPieces) * 8) = kraw[j];
-        }
+        // ---- the keys through this wavefront's part of shared memory, then the scores: one tile
+        //      of 16 keys after the other.  Which keys row i of a tile's first operand is: see the
+        //      header for why. ----
         float4_t s[2];
 #pragma unroll
         for (int t2 = 0; t2 < 2; ++t2) {
-            // which key row i of the first operand is; see the header for why
-            const int key = V16 ? 8 * (i / 4) + 4 * t2 + (i % 4) : 16 * t2 + i;
+#pragma unroll
+            for (int j = 0; j < DT; ++j) {
+                const int f = lane + j * kWave;
+                const int key = f / kPieces;
+                const int tile = V16 ? (key / 4) % 2 : key / 16;
+                const int at = V16 ? 4 * (key / 8) + key % 4 : key % 16;
+                if (tile == t2)
+                    *reinterpret_cast<uint4_t*>(stage + at * kKeyStride + (f % kPieces) * 8) = kraw[j];
+            }
+            // Lanes read what other lanes of the wavefront wrote, with no barrier between (a
+            // wavefront's accesses to shared memory run in order): the compiler has to be told
+            // that the memory changed, or a lane that wrote nothing keeps what it read before.
+            asm volatile("" ::: "memory");
             float4_t sc = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int c = 0; c < DC; ++c) {
                 Pack16 a;
-                a.u = *reinterpret_cast<const uint4*>(stage + key * kKeyStride + c * 32 + 8 * g);
+                a.u = *reinterpret_cast<const uint4*>(stage + i * kKeyStride + c * 32 + 8 * g);
                 sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qreg[c], sc, 0, 0, 0);
             }
             s[t2] = sc;
@@ -239,63 +248,70 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
     }
 
     // ---- merge: every wavefront leaves its sums in its own part of shared memory (it has read its
-    //      keys from there already), then each takes every fourth tile of 16 elements of the head and
-    //      combines the four wavefronts' sums of that tile, always in the order 0, 1, 2, 3.
+    //      keys from there already), one half of the head after the other; of each half every
+    //      wavefront takes every fourth tile of 16 elements and combines the four wavefronts' sums of
+    //      that tile, always in the order 0, 1, 2, 3.
     //      lane (i, g) holds out^T[16t + 4g + v][row i]: elements d = 16t + 4g + v of row i ----
-    {
-        float* mine = reinterpret_cast<float*>(stage);
-#pragma unroll
-        for (int t = 0; t < DT; ++t)
-            *reinterpret_cast<float4_t*>(mine + i * kMergeStride + t * 16 + 4 * g) = acc[t];
-        if (g == 0) {
-            mine[kRowsPerTile * kMergeStride + 2 * i] = m_run;
-            mine[kRowsPerTile * kMergeStride + 2 * i + 1] = l_run;
-        }
+    float* mine = reinterpret_cast<float*>(stage);
+    if (g == 0) {
+        row_max_s[wave][i] = m_run;
+        row_sum_s[wave][i] = l_run;
     }
-    __syncthreads();
-    if (!row_valid) return;
-    float m_of[4], l_of[4], f_of[4];
-    float m_all = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-        const float* part = reinterpret_cast<const float*>(shared_raw + w * kPartBytes);
-        m_of[w] = part[kRowsPerTile * kMergeStride + 2 * i];
-        l_of[w] = part[kRowsPerTile * kMergeStride + 2 * i + 1];
-        m_all = fmaxf(m_all, m_of[w]);
-    }
-    const float m_use = m_all == -INFINITY ? 0.f : m_all;
-    float l_all = 0.f;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-        f_of[w] = exp2f((m_of[w] - m_use) * scale_log2e);       // 0 for a wavefront without keys
-        l_all = fmaf(l_of[w], f_of[w], l_all);
-    }
-    const float inv = 1.f / l_all;
+    float f_of[4] = {0.f, 0.f, 0.f, 0.f};
+    float m_all = -INFINITY, l_all = 0.f, inv = 0.f;
     bf16* orow = out + (static_cast<size_t>(q_start + tok) * num_heads + head) * HD;
     const size_t prow = static_cast<size_t>(max(partial_slot, 0)) * kRowsPerTile + (row - row_begin);
     float* po = partial_o + prow * HD;
 #pragma unroll
-    for (int t0 = 0; t0 < DT; t0 += 4) {
-        const int t = t0 + wave;
-        if (t >= DT) break;
-        float4_t sum = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int half = 0; half < 2; ++half) {
+        if (half) __syncthreads();          // the first half has been read
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const float* part = reinterpret_cast<const float*>(shared_raw + w * kPartBytes);
-            const float4_t v = *reinterpret_cast<const float4_t*>(part + i * kMergeStride + t * 16 + 4 * g);
+        for (int t = 0; t < DT / 2; ++t)
+            *reinterpret_cast<float4_t*>(mine + i * kMergeStride + t * 16 + 4 * g) = acc[half * (DT / 2) + t];
+        __syncthreads();
+        if (!half) {
+            float m_of[4], l_of[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) sum[e] = fmaf(v[e], f_of[w], sum[e]);
+            for (int w = 0; w < 4; ++w) {
+                m_of[w] = row_max_s[w][i];
+                l_of[w] = row_sum_s[w][i];
+                m_all = fmaxf(m_all, m_of[w]);
+            }
+            const float m_use = m_all == -INFINITY ? 0.f : m_all;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                f_of[w] = exp2f((m_of[w] - m_use) * scale_log2e);       // 0 for a wavefront without keys
+                l_all = fmaf(l_of[w], f_of[w], l_all);
+            }
+            inv = 1.f / l_all;
         }
-        if (partial_slot < 0) {
-            uint2 w2;
-            w2.x = pack2_bf16(sum[0] * inv, sum[1] * inv);
-            w2.y = pack2_bf16(sum[2] * inv, sum[3] * inv);
-            *reinterpret_cast<uint2*>(orow + t * 16 + 4 * g) = w2;
-        } else {
-            *reinterpret_cast<float4_t*>(po + t * 16 + 4 * g) = sum;
+        if (row_valid) {
+#pragma unroll
+            for (int t0 = 0; t0 < DT / 2; t0 += 4) {
+                const int t = t0 + wave;
+                if (t < DT / 2) {
+                    float4_t sum = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        const float* part = reinterpret_cast<const float*>(shared_raw + w * kPartBytes);
+                        const float4_t v = *reinterpret_cast<const float4_t*>(part + i * kMergeStride + t * 16 + 4 * g);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) sum[e] = fmaf(v[e], f_of[w], sum[e]);
+                    }
+                    const int d = (half * (DT / 2) + t) * 16 + 4 * g;
+                    if (partial_slot < 0) {
+                        uint2 w2;
+                        w2.x = pack2_bf16(sum[0] * inv, sum[1] * inv);
+                        w2.y = pack2_bf16(sum[2] * inv, sum[3] * inv);
+                        *reinterpret_cast<uint2*>(orow + d) = w2;
+                    } else {
+                        *reinterpret_cast<float4_t*>(po + d) = sum;
+                    }
+                }
+            }
         }
     }
-    if (partial_slot >= 0 && wave == 0 && g == 0) {
+    if (row_valid && partial_slot >= 0 && wave == 0 && g == 0) {
         partial_ml[prow * 2] = m_all;
         partial_ml[prow * 2 + 1] = l_all;
     }
