@@ -10,7 +10,7 @@ from wllm_amd.kernels import attention_plan as ap
 
 def covered(q_len, ctx_len, group, nkv, window, page_size):
     items, reduces, slots, prefill, prefill_rows = ap.build_work_items(
-        np.array(q_len), np.array(ctx_len), group, nkv, window, 0, page_size)
+        np.array(q_len), np.array(ctx_len), group, nkv, window, page_size)
     cover = {}          # (seg, kvh, row) -> list of (first key, end key, slot)
     slot_users = {}
     def hold(slot, who):

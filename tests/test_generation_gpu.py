@@ -206,6 +206,38 @@ def test_captured_graphs_give_what_eager_steps_give(varied_folders, dtype):
         assert torch.allclose(torch.tensor(a.logprobs), torch.tensor(b.logprobs), atol=1e-5 if dtype == "float32" else 2e-2)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graphs_for_classes_of_context_lengths(varied_folders, dtype):
+    """A bucket has a graph for each class of context lengths; requests that grow from 20 to 150
+    tokens pass through the graphs for at most 48, 96 and 200 tokens, beside a shorter request
+    that comes later, and generate what steps run kernel by kernel generate."""
+    model = load_model(varied_folders["MV"], dtype, "cuda")
+    prompts = [random_ids(70, 20, 1000), random_ids(71, 30, 1000), random_ids(72, 6, 1000)]
+    news = [130, 90, 25]
+
+    def run(graphs):
+        runner = ModelRunner.create(model, num_pages=40, page_size=16, max_requests=2)
+        if graphs:
+            runner.enable_graphs(buckets=(1, 2), max_context=200, contexts=(48, 96))
+            assert runner.graph_contexts == (48, 96, 200)
+        s = Scheduler(runner, max_prefill_tokens_per_step=32, lookahead=True)
+        reqs = [Request(i, p, n) for i, (p, n) in enumerate(zip(prompts, news))]
+        for r in reqs:
+            s.add_request(r)
+        s.run_to_completion()
+        runner.cache.check()
+        return reqs, runner
+
+    eager, _ = run(False)
+    graphed, runner = run(True)
+    assert sorted(runner.graphs[2]) == [48, 96, 200] and runner.graph_steps > 100, {b: sorted(g) for b, g in runner.graphs.items()}
+    widths = {c: g.table_width for c, g in runner.graphs[2].items()}
+    assert widths == {48: 3, 96: 6, 200: 13}
+    for a, b in zip(eager, graphed):
+        assert a.output_token_ids == b.output_token_ids
+        assert_varied(a.output_token_ids)
+
+
 def test_a_full_batch_of_any_size_has_its_graph(varied_folders):
     """The largest number of requests the cache admits is a bucket of its own: a full batch of 3
     (or 17) does not fall back to steps run kernel by kernel."""

@@ -17,7 +17,8 @@
 // four are merged through shared memory.  A segment with more keys than a chunk is split over
 // workgroups; those write partial results (maximum, sum, unnormalised accumulator) that
 // `attention_reduce_kernel` combines.  Chunk boundaries depend on the key index only, never on
-// the batch.
+// the batch.  A captured graph launches a workgroup for every item its plan has room for and reads
+// the number of live items, which come first, from device memory.
 //
 // Matrix products (v_mfma_f32_16x16x32_bf16, 64 lanes: i = lane % 16, g = lane / 16):
 //   scores^T[key, row] = K[key, :] . Q[row, :]     A = K: lane (i, g) holds K[key_i][32c + 8g ..+8]
@@ -56,7 +57,7 @@ template <int HD, bool V16>
 __global__ void __launch_bounds__(256, 3)
 paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict__ cache,
                             const int* __restrict__ block_tables, const int* __restrict__ items,
-                            const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
+                            const int* __restrict__ live_items, const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
                             const int* __restrict__ seg_ctx_len, bf16* __restrict__ out,
                             float* __restrict__ partial_o, float* __restrict__ partial_ml, int num_heads,
                             int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window) {
@@ -76,6 +77,8 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
     __shared__ __align__(16) unsigned char shared_raw[4 * kPartBytes];
     __shared__ float row_max_s[4][kRowsPerTile], row_sum_s[4][kRowsPerTile];
 
+    // a captured graph launches as many workgroups as its plan has room for items; the live ones come first
+    if (live_items != nullptr && static_cast<int>(blockIdx.x) >= live_items[0]) return;
     const int* item = items + static_cast<size_t>(blockIdx.x) * kItemInts;
     const int seg = item[0], kvh = item[1], row_begin = item[2];
     const int key_begin = item[4], key_end = item[5], partial_slot = item[6];
@@ -430,54 +433,80 @@ attention_reduce_wide_kernel(const int* __restrict__ reduce_items, const float* 
     *reinterpret_cast<uint2*>(out + (static_cast<size_t>(seg_q_start[seg] + tok) * num_heads + head) * HD + d) = w;
 }
 
-// Returns 0, a HIP error code, or -1 for sizes these kernels do not take.
+namespace {
+
+struct AttentionArguments {
+    const bf16* qkv;
+    const bf16* cache;
+    const int* block_tables;
+    const int* items;
+    const int* live_items;
+    int num_items;
+    const int* reduce_items;
+    int num_reduce_items;
+    const int* seg_q_start;
+    const int* seg_q_len;
+    const int* seg_ctx_len;
+    bf16* out;
+    float* partial_o;
+    float* partial_ml;
+    int num_heads, num_kv_heads, page_size, max_pages;
+    float scale_log2e;
+    int window;
+    hipStream_t stream;
+};
+
+template <int HD, bool V16>
+int launch_items(const AttentionArguments& a) {
+    paged_attention_mfma_kernel<HD, V16><<<a.num_items, 256, 0, a.stream>>>(
+        a.qkv, a.cache, a.block_tables, a.items, a.live_items, a.seg_q_start, a.seg_q_len, a.seg_ctx_len, a.out,
+        a.partial_o, a.partial_ml, a.num_heads, a.num_kv_heads, a.page_size, a.max_pages, a.scale_log2e, a.window);
+    return 0;
+}
+
+template <int HD>
+int launch_all(const AttentionArguments& a) {
+    if (a.num_items > 0) {
+        const int status = a.page_size % 8 == 0 ? launch_items<HD, true>(a) : launch_items<HD, false>(a);
+        if (status != 0) return status;
+    }
+    if (a.num_reduce_items >= 64) {
+        attention_reduce_wide_kernel<HD><<<dim3(a.num_reduce_items, kRowsPerTile / 4), HD, 0, a.stream>>>(
+            a.reduce_items, a.partial_o, a.partial_ml, a.seg_q_start, a.seg_q_len, a.out, a.num_heads, a.num_kv_heads,
+            a.scale_log2e);
+    } else if (a.num_reduce_items > 0) {
+        attention_reduce_kernel<HD><<<dim3(a.num_reduce_items, kRowsPerTile), HD, 0, a.stream>>>(
+            a.reduce_items, a.partial_o, a.partial_ml, a.seg_q_start, a.seg_q_len, a.out, a.num_heads, a.num_kv_heads,
+            a.scale_log2e);
+    }
+    return launch_status();
+}
+
+}  // namespace
+
+// Returns 0, a HIP error code, or -1 for sizes these kernels do not take.  `live_items`: null, or a
+// device int that says how many of the `num_items` items count (a captured graph's plan).
 WLLM_API int wllm_paged_attention_mfma(const void* qkv, const void* cache, const int* block_tables, const int* items,
-                                       int num_items, const int* reduce_items, int num_reduce_items,
-                                       const int* seg_q_start, const int* seg_q_len, const int* seg_ctx_len, void* out,
-                                       float* partial_o, float* partial_ml, int num_heads, int num_kv_heads,
-                                       int head_dim, int page_size, int max_pages, float scale, int window,
-                                       hipStream_t stream) {
+                                       const int* live_items, int num_items, const int* reduce_items,
+                                       int num_reduce_items, const int* seg_q_start, const int* seg_q_len,
+                                       const int* seg_ctx_len, void* out, float* partial_o, float* partial_ml,
+                                       int num_heads, int num_kv_heads, int head_dim, int page_size, int max_pages,
+                                       float scale, int window, hipStream_t stream) {
     if (head_dim % 32 != 0 || head_dim < 32 || head_dim > 256 || page_size % 4 != 0 || num_heads % num_kv_heads != 0)
         return -1;
-    const float scale_log2e = scale * 1.4426950408889634f;
-    const bool v16 = page_size % 8 == 0;
-#define LAUNCH(HD, V16)                                                                                              \
-    paged_attention_mfma_kernel<HD, V16><<<num_items, 256, 0, stream>>>(                                            \
-        static_cast<const bf16*>(qkv), static_cast<const bf16*>(cache), block_tables, items, seg_q_start, seg_q_len, \
-        seg_ctx_len, static_cast<bf16*>(out), partial_o, partial_ml, num_heads, num_kv_heads, page_size, max_pages,  \
-        scale_log2e, window)
-#define LAUNCH_R(HD)                                                                                                 \
-    if (num_reduce_items >= 64) {                                                                                    \
-        attention_reduce_wide_kernel<HD><<<dim3(num_reduce_items, kRowsPerTile / 4), HD, 0, stream>>>(               \
-            reduce_items, partial_o, partial_ml, seg_q_start, seg_q_len, static_cast<bf16*>(out), num_heads,         \
-            num_kv_heads, scale_log2e);                                                                              \
-    } else {                                                                                                         \
-        attention_reduce_kernel<HD><<<dim3(num_reduce_items, kRowsPerTile), HD, 0, stream>>>(                        \
-            reduce_items, partial_o, partial_ml, seg_q_start, seg_q_len, static_cast<bf16*>(out), num_heads,         \
-            num_kv_heads, scale_log2e);                                                                              \
-    }
-#define CASE(HD)                                   \
-    case HD:                                       \
-        if (num_items > 0) {                       \
-            if (v16) LAUNCH(HD, true);             \
-            else LAUNCH(HD, false);                \
-        }                                          \
-        if (num_reduce_items > 0) LAUNCH_R(HD);    \
-        break;
+    const AttentionArguments a = {static_cast<const bf16*>(qkv), static_cast<const bf16*>(cache), block_tables, items,
+                                  live_items, num_items, reduce_items, num_reduce_items, seg_q_start, seg_q_len,
+                                  seg_ctx_len, static_cast<bf16*>(out), partial_o, partial_ml, num_heads, num_kv_heads,
+                                  page_size, max_pages, scale * 1.4426950408889634f, window, stream};
     switch (head_dim) {
-        CASE(32)
-        CASE(64)
-        CASE(96)
-        CASE(128)
-        CASE(160)
-        CASE(192)
-        CASE(224)
-        CASE(256)
-        default:
-            return -1;
+        case 32: return launch_all<32>(a);
+        case 64: return launch_all<64>(a);
+        case 96: return launch_all<96>(a);
+        case 128: return launch_all<128>(a);
+        case 160: return launch_all<160>(a);
+        case 192: return launch_all<192>(a);
+        case 224: return launch_all<224>(a);
+        case 256: return launch_all<256>(a);
+        default: return -1;
     }
-#undef CASE
-#undef LAUNCH
-#undef LAUNCH_R
-    return launch_status();
 }

@@ -39,11 +39,16 @@ class PageView:
 
 
 class Workspace:
-    """Named scratch tensors that live across steps and grow on demand."""
+    """Named scratch tensors that live across steps and grow on demand, until `freeze`: a captured
+    graph holds their addresses, so afterwards a request for more than there is raises."""
 
     def __init__(self, device):
         self.device = device
         self._flat: dict = {}
+        self._frozen = False
+
+    def freeze(self) -> None:
+        self._frozen = True
 
     def get(self, name: str, shape: tuple, dtype: torch.dtype) -> torch.Tensor:
         count = 1
@@ -52,6 +57,9 @@ class Workspace:
         key = (name, dtype)
         flat = self._flat.get(key)
         if flat is None or flat.numel() < count:
+            if self._frozen:
+                raise RuntimeError(f"scratch tensor {name!r} would have to grow to {count} elements, "
+                                   "but a captured graph holds its address")
             flat = torch.empty(max(count, 1), dtype=dtype, device=self.device)
             self._flat[key] = flat
         return flat[:count].view(shape)

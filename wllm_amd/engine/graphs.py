@@ -4,7 +4,9 @@ A decode step (every request brings one token and wants its logits) launches a f
 small kernels; issued one by one from Python they cost more host time than GPU time (the
 reference counts about 880 launches of 8 microseconds in a 30 ms step,
 src/wllm/engine/cuda_graph_decoder.py:5-11, and captures one CUDA graph per batch-size
-bucket, :66-134).  Here one graph is captured per bucket too.  A graph owns everything whose
+bucket, :66-134).  Here a graph is captured per bucket and class of context lengths (its
+attention kernel's grid and its block tables are as large as its longest context needs, so
+short contexts get graphs of their own).  A graph owns everything whose
 address its kernels hold: a packed int32 buffer with all index arrays of the step (ids,
 positions, slots, block tables of fixed width, attention work items of fixed count), its
 scratch tensors and its logits.  A step fills the pinned host copy of the buffer, copies it
@@ -45,7 +47,7 @@ def capture(body):
 
 
 class DecodeGraph:
-    def __init__(self, runner, bucket: int, max_context: int):
+    def __init__(self, runner, bucket: int, max_context: int, workspace=None):
         self.runner = runner
         self.bucket = bucket
         self.max_context = max_context
@@ -66,7 +68,7 @@ class DecodeGraph:
         v = [self.dev[self._offsets[i]:self._offsets[i + 1]] for i in range(len(sizes))]
         g = self.num_groups
         self._feed_dst, self._feed_src = v[8 + 2 * g], v[9 + 2 * g]
-        self.workspace = Workspace(self.device)
+        self.workspace = workspace if workspace is not None else Workspace(self.device)
         self.ctx = StepContext(
             n=b, num_segments=b, dtype=model.dtype, device=self.device, workspace=self.workspace, cache=cache,
             schedule=model.plan.schedule, token_ids=v[0], positions=v[1], token_segment=v[2], seg_q_start=v[3],
@@ -143,5 +145,6 @@ class DecodeGraph:
             self.runner.model.forward(self.ctx)
             torch.cuda.synchronize()
             self.graph, self.logits = capture(lambda: self.runner.model.forward(self.ctx))
+            self.workspace.freeze()
         self.graph.replay()
         return self.logits[:len(entries)]

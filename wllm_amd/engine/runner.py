@@ -34,23 +34,33 @@ class ModelRunner:
         self.workspace = Workspace(self.device)
         self.steps_run = 0
         self.tokens_run = 0
-        self.graphs: dict = {}             # bucket -> DecodeGraph
+        self.graphs: dict = {}             # bucket -> {longest context -> DecodeGraph}
         self.graph_buckets: tuple = ()
+        self.graph_contexts: tuple = ()    # ascending; the last is graph_max_context
         self.graph_max_context = 0
         self.dummy_pages: list = []
         self.graph_steps = 0
 
-    def enable_graphs(self, buckets=(1, 2, 4, 8, 16, 32, 48, 64, 128, 256), max_context=None) -> None:
+    def enable_graphs(self, buckets=(1, 2, 4, 8, 16, 32, 48, 64, 128, 256), max_context=None, contexts=None) -> None:
         """Decode-only steps of up to max(buckets) requests replay a captured graph of the
         smallest bucket that holds them; the largest number of requests the cache admits, if it
         is below max(buckets), is a bucket too, so that a full batch of any size has its graph.
-        One page per group is set aside for padding rows."""
+        A bucket has a graph for each class of context lengths (the longest, a half of it, a
+        quarter, down to about a thousand tokens): a graph's attention runs as many workgroups
+        as its longest context needs, live or not, and its block tables are as wide.  Graphs
+        are captured when a step first needs them (`contexts` names other classes).  One page per
+        group is set aside for padding rows."""
         if self.graph_buckets:
             return
         if not self.model.graph_capturable():
             raise ValueError("a part of this model reads the step's arrays on the host; its steps cannot be captured")
         limit = min(self.model.plan.max_positions, min(g.pool.num_pages - 1 for g in self.cache.groups) * self.cache.page_size)
         self.graph_max_context = min(max_context or limit, limit)
+        if contexts is None:
+            contexts = [self.graph_max_context]
+            while contexts[-1] > 1024:
+                contexts.append(-(-contexts[-1] // (2 * self.cache.page_size)) * self.cache.page_size)
+        self.graph_contexts = tuple(sorted({c for c in contexts if c < self.graph_max_context} | {self.graph_max_context}))
         most = self.cache.max_requests
         self.graph_buckets = tuple(sorted({b for b in buckets if b <= most} | ({most} if most <= max(buckets) else set())))
         self.dummy_pages = [self.cache.set_aside_page(gi) for gi in range(len(self.cache.groups))]
@@ -58,16 +68,23 @@ class ModelRunner:
     def _graph_for(self, entries: list):
         if not self.graph_buckets or len(entries) > self.graph_buckets[-1]:
             return None
+        longest = 0
         for e in entries:
             if len(e.tokens) != 1 or list(e.want) != [0]:
                 return None
-            if self.cache.context_len(e.request) + 1 > self.graph_max_context:
-                return None
+            longest = max(longest, self.cache.context_len(e.request) + 1)
+        if longest > self.graph_max_context:
+            return None
         bucket = next(b for b in self.graph_buckets if b >= len(entries))
-        if bucket not in self.graphs:
+        context = next(c for c in self.graph_contexts if c >= longest)
+        of_bucket = self.graphs.setdefault(bucket, {})
+        if context not in of_bucket:
             from wllm_amd.engine.graphs import DecodeGraph
-            self.graphs[bucket] = DecodeGraph(self, bucket, self.graph_max_context)
-        return self.graphs[bucket]
+
+            # the graphs of a bucket run one at a time and need scratch tensors of the same shapes
+            shared = next(iter(of_bucket.values())).workspace if of_bucket else None
+            of_bucket[context] = DecodeGraph(self, bucket, context, workspace=shared)
+        return of_bucket[context]
 
     @classmethod
     def create(cls, model, *, num_pages: int, page_size: int, max_requests: int, **cache_options):

@@ -48,48 +48,59 @@ class AttentionPlan:
     prefill_items: Optional[torch.Tensor] = None  # int32 [num_prefill, 8]
     num_prefill: int = 0
     prefill_rows: int = 64
+    live_items: Optional[torch.Tensor] = None     # int32 [1] on the device: how many of `items` count (None: all)
 
 
 class StaticAttentionPlan(AttentionPlan):
-    """A plan of fixed shape for a captured graph: always `segments * kv_heads * fixed_splits`
+    """A plan of fixed shape for a captured graph: room for `segments * kv_heads * fixed_splits`
     work items in the same device tensors, whose contents `update` rewrites before each replay.
-    Partial slots are numbered over the live chunks only, so the partial buffers are as large
-    as the most keys the cache pool can hold needs, not as the fixed shape."""
+    The live items come first and their number lies in device memory behind them (`live_items`):
+    the kernel reads it, so a step costs what its live items cost.  Partial slots are numbered
+    over the live chunks only, so the partial buffers are as large as the most keys the cache
+    pool can hold needs, not as the fixed shape."""
 
     def __init__(self, segments: int, group: int, num_kv_heads: int, window: int, fixed_splits: int,
                  max_slots: int, head_dim: int, device):
-        n_i, n_r = segments * num_kv_heads * fixed_splits, segments * num_kv_heads
-        self._host = torch.empty((n_i + n_r) * ITEM_INTS, dtype=torch.int32, pin_memory=True)
-        self._dev = torch.empty_like(self._host, device=device)
-        self._args = (group, num_kv_heads, window, fixed_splits)
+        # a live item of a segment with several chunks holds a partial slot; a segment with one has one item
+        n_r = segments * num_kv_heads
+        n_i = min(n_r * fixed_splits, max_slots + n_r)
+        # the number of live items (and 7 unused), the reduce items, the items: a step copies the
+        # front of it, up to the last live item
+        self._host = torch.empty((1 + n_r + n_i) * ITEM_INTS, dtype=torch.int32, pin_memory=True)
+        self._dev = torch.zeros_like(self._host, device=device)
+        self._args = (group, num_kv_heads, window)
         self.max_slots = max_slots
-        super().__init__(self._dev[:n_i * ITEM_INTS].view(n_i, ITEM_INTS), self._dev[n_i * ITEM_INTS:].view(n_r, ITEM_INTS),
-                         n_i, n_r, max_slots,
+        a, b = ITEM_INTS, (1 + n_r) * ITEM_INTS
+        super().__init__(self._dev[b:].view(n_i, ITEM_INTS), self._dev[a:b].view(n_r, ITEM_INTS), n_i, n_r, max_slots,
                          torch.empty(max(1, max_slots) * ROWS_PER_TILE * head_dim, dtype=torch.float32, device=device),
                          torch.empty(max(1, max_slots) * ROWS_PER_TILE * 2, dtype=torch.float32, device=device))
+        self.live_items = self._dev[:1]
 
     def update(self, q_len: np.ndarray, ctx_len: np.ndarray) -> None:
-        group, nkv, window, fixed = self._args
-        items, reduces, slots, prefill, _ = build_work_items(q_len, ctx_len, group, nkv, window, fixed)
+        group, nkv, window = self._args
+        items, reduces, slots, prefill, _ = build_work_items(q_len, ctx_len, group, nkv, window)
         assert prefill.shape[0] == 0, "a captured decode graph holds no long segment"
         if slots > self.max_slots:
             raise ValueError(f"the step needs {slots} partial slots, the graph's plan has {self.max_slots}")
-        assert items.shape[0] == self.num_items and reduces.shape[0] == self.num_reduce
+        if items.shape[0] > self.num_items or reduces.shape[0] > self.num_reduce:
+            raise ValueError(f"the step needs {items.shape[0]} work items and {reduces.shape[0]} reduce items, "
+                             f"the graph's plan has room for {self.num_items} and {self.num_reduce}")
         buf = self._host.numpy()
-        buf[:items.size] = items.reshape(-1)
-        buf[items.size:] = reduces.reshape(-1)
-        self._dev.copy_(self._host, non_blocking=True)
+        buf[0] = items.shape[0]
+        # a graph runs a reduce item for every (segment, key/value head); those beyond the segments
+        # with several chunks stand for nothing
+        a, b = ITEM_INTS, (1 + self.num_reduce) * ITEM_INTS
+        buf[a:b].reshape(-1, ITEM_INTS)[reduces.shape[0]:, 0] = -1
+        buf[a:a + reduces.size] = reduces.reshape(-1)
+        buf[b:b + items.size] = items.reshape(-1)
+        used = b + items.size
+        self._dev[:used].copy_(self._host[:used], non_blocking=True)
 
 
 def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_heads: int, window: int,
-                     fixed_splits: int = 0, page_size: int = 16):
+                     page_size: int = 16):
     """Returns (items [n, 8], reduce_items [m, 8], partial slots, prefill items [p, 8], rows per
-    prefill item) as int32 arrays.
-
-    `fixed_splits` > 0 gives every short segment exactly that many items per key/value head
-    (items beyond the segment's keys are padding that the kernel skips), so that the number
-    of items depends on the number of segments only: the shape a captured graph needs.
-    """
+    prefill item) as int32 arrays."""
     q_len = np.asarray(q_len, dtype=np.int64)
     ctx_len = np.asarray(ctx_len, dtype=np.int64)
     rows = q_len * group
@@ -105,15 +116,13 @@ def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_
         c0 = lo // KEY_CHUNK
         c1 = (ctx_len[idx] - 1) // KEY_CHUNK
         ns = c1 - c0 + 1
-        width = int(fixed_splits) if fixed_splits > 0 else int(ns.max())
-        if fixed_splits > 0 and int(ns.max()) > fixed_splits:
-            raise ValueError(f"a segment needs {int(ns.max())} key chunks, the plan is fixed at {fixed_splits}")
+        width = int(ns.max())
         j = np.arange(width, dtype=np.int64)
         chunk = c0[:, None] + j[None, :]                       # [S, width]
         live = j[None, :] < ns[:, None]
         kb = np.maximum(lo[:, None], chunk * KEY_CHUNK)
         ke = np.minimum(ctx_len[idx][:, None], (chunk + 1) * KEY_CHUNK)
-        single = (ns == 1) & (fixed_splits <= 0)
+        single = ns == 1
         # partial slots: one per (segment, kv head, split) for segments that are split
         n_split_seg = np.where(single, 0, ns)
         seg_base = np.concatenate([[0], np.cumsum(n_split_seg * num_kv_heads)])[:-1]
@@ -127,10 +136,7 @@ def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_
         it[..., 5] = ke[:, None, :]
         slot = seg_base[:, None, None] + kv[None, :, None] * n_split_seg[:, None, None] + j[None, None, :]
         it[..., 6] = np.where(single[:, None, None], -1, slot)
-        if fixed_splits > 0:
-            keep = np.ones((S, num_kv_heads, width), dtype=bool)
-        else:
-            keep = np.broadcast_to(live[:, None, :], (S, num_kv_heads, width))
+        keep = np.broadcast_to(live[:, None, :], (S, num_kv_heads, width))
         items.append(it[keep].reshape(-1, ITEM_INTS))
         split_seg = ~single
         if split_seg.any():

@@ -45,7 +45,7 @@ _SIGNATURES = {
                                      c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                      c_float, c_int, c_void_p],
     "wllm_paged_attention_generic_chunk_keys": [],
-    "wllm_paged_attention_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
+    "wllm_paged_attention_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
                                   c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
                                   c_int, c_void_p],
     "wllm_paged_attention_prefill": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
@@ -167,11 +167,11 @@ class HipBackend:
         return dtype == torch.bfloat16 and head_dim % 32 == 0 and 32 <= head_dim <= 256 and page_size % 4 == 0
 
     def plan_paged_attention(self, host_q_len, host_ctx_len, num_heads, num_kv_heads, head_dim, page_size, window,
-                             dtype, device, fixed_splits: int = 0):
+                             dtype, device):
         if not self.mfma_attention_takes(dtype, head_dim, page_size):
             return None
         items, reduces, slots, prefill, prefill_rows = build_work_items(
-            host_q_len, host_ctx_len, num_heads // num_kv_heads, num_kv_heads, window, fixed_splits, page_size)
+            host_q_len, host_ctx_len, num_heads // num_kv_heads, num_kv_heads, window, page_size)
         flat = np.concatenate([items.reshape(-1), reduces.reshape(-1), prefill.reshape(-1)])
         dev = pack_int32([flat], device)[0]
         n_i, n_r, n_p = items.shape[0], reduces.shape[0], prefill.shape[0]
@@ -220,7 +220,8 @@ class HipBackend:
             if plan.num_items == 0 and plan.num_reduce == 0:
                 return
             self._check(self.lib.wllm_paged_attention_mfma(
-                _ptr(qkv), _ptr(cache), _ptr(block_tables), _ptr(plan.items), plan.num_items, _ptr(plan.reduce_items),
+                _ptr(qkv), _ptr(cache), _ptr(block_tables), _ptr(plan.items),
+                _ptr(plan.live_items), plan.num_items, _ptr(plan.reduce_items),
                 plan.num_reduce, _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out),
                 _ptr(plan.partial_o), _ptr(plan.partial_ml), num_heads, num_kv_heads, head_dim, page_size,
                 block_tables.shape[1], scale, window, self._stream()), "paged_attention (matrix cores)")
