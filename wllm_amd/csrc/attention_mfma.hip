@@ -337,6 +337,7 @@ attention_reduce_kernel(const int* __restrict__ reduce_items, const float* __res
     const size_t stride = static_cast<size_t>(item[5]) * kRowsPerTile;     // rows between two splits
     const int group = num_heads / num_kv_heads;
     const int r = blockIdx.y, d = threadIdx.x;
+    const int q_start = seg_q_start[seg];       // asked for with the length: the store at the end does not wait for it
     if (row0 + r >= seg_q_len[seg] * group) return;
     const float* ml = partial_ml + (static_cast<size_t>(first) * kRowsPerTile + r) * 2;
     const float* po = partial_o + (static_cast<size_t>(first) * kRowsPerTile + r) * HD + d;
@@ -372,7 +373,7 @@ attention_reduce_kernel(const int* __restrict__ reduce_items, const float* __res
     }
     const int row = row0 + r;
     const int tok = row / group, head = kvh * group + row % group;
-    out[(static_cast<size_t>(seg_q_start[seg] + tok) * num_heads + head) * HD + d] = from_float<bf16>(num / den);
+    out[(static_cast<size_t>(q_start + tok) * num_heads + head) * HD + d] = from_float<bf16>(num / den);
 }
 
 // The same sums for steps with many tiles to combine (the pieces of a long prompt): a thread takes
@@ -392,6 +393,7 @@ attention_reduce_wide_kernel(const int* __restrict__ reduce_items, const float* 
     const int group = num_heads / num_kv_heads;
     constexpr int kQuads = HD / 4;
     const int r = blockIdx.y * 4 + threadIdx.x / kQuads, d = (threadIdx.x % kQuads) * 4;
+    const int q_start = seg_q_start[seg];
     if (row0 + r >= seg_q_len[seg] * group) return;
     const float* ml = partial_ml + (static_cast<size_t>(first) * kRowsPerTile + r) * 2;
     const float* po = partial_o + (static_cast<size_t>(first) * kRowsPerTile + r) * HD + d;
@@ -430,7 +432,7 @@ attention_reduce_wide_kernel(const int* __restrict__ reduce_items, const float* 
     uint2 w;
     w.x = pack2_bf16(num[0] / den, num[1] / den);
     w.y = pack2_bf16(num[2] / den, num[3] / den);
-    *reinterpret_cast<uint2*>(out + (static_cast<size_t>(seg_q_start[seg] + tok) * num_heads + head) * HD + d) = w;
+    *reinterpret_cast<uint2*>(out + (static_cast<size_t>(q_start + tok) * num_heads + head) * HD + d) = w;
 }
 
 namespace {

@@ -130,8 +130,14 @@ __global__ void rms_norm_vec_kernel(float* __restrict__ x, const TD* __restrict_
     float* xr = x + static_cast<size_t>(irow) * hidden;
     const TD* dr = delta ? delta + static_cast<size_t>(irow) * hidden : nullptr;
     TO* o = out + static_cast<size_t>(orow) * hidden;
-    Quad<float> keep[kNormGroups];
+    Quad<float> keep[kNormGroups], w[kNormGroups];
     float ss = 0.f;
+    // the norm's weights are asked for with everything else, not after the sum of squares
+#pragma unroll
+    for (int e = 0; e < kNormGroups; ++e) {
+        const int i = (threadIdx.x + e * blockDim.x) * 4;
+        w[e] = i < hidden ? *reinterpret_cast<const Quad<float>*>(weight + i) : Quad<float>{{0.f, 0.f, 0.f, 0.f}};
+    }
 #pragma unroll
     for (int e = 0; e < kNormGroups; ++e) {
         const int i = (threadIdx.x + e * blockDim.x) * 4;
@@ -142,13 +148,14 @@ __global__ void rms_norm_vec_kernel(float* __restrict__ x, const TD* __restrict_
                 // the partial sums of a stack are added in stack order, then their sum to x
                 const int stack = (sizeof(TD) == sizeof(float) && splits > 1) ? splits : 1;
                 Quad<float> d = {{0.f, 0.f, 0.f, 0.f}};
-                for (int s0 = 0; s0 < stack; s0 += 8) {
-                    Quad<TD> q[8];       // eight loads in flight
+                constexpr int kInFlight = 16;
+                for (int s0 = 0; s0 < stack; s0 += kInFlight) {
+                    Quad<TD> q[kInFlight];       // loads in flight
 #pragma unroll
-                    for (int j = 0; j < 8; ++j)
+                    for (int j = 0; j < kInFlight; ++j)
                         q[j] = *reinterpret_cast<const Quad<TD>*>(dr + min(s0 + j, stack - 1) * split_stride + i);
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) {
+                    for (int j = 0; j < kInFlight; ++j) {
                         if (s0 + j >= stack) break;
 #pragma unroll
                         for (int k = 0; k < 4; ++k) d.v[k] = s0 + j == 0 ? to_float(q[j].v[k]) : d.v[k] + to_float(q[j].v[k]);
@@ -169,10 +176,9 @@ __global__ void rms_norm_vec_kernel(float* __restrict__ x, const TD* __restrict_
     for (int e = 0; e < kNormGroups; ++e) {
         const int i = (threadIdx.x + e * blockDim.x) * 4;
         if (i < hidden) {
-            const Quad<float> w = *reinterpret_cast<const Quad<float>*>(weight + i);
             Quad<TO> r;
 #pragma unroll
-            for (int k = 0; k < 4; ++k) r.v[k] = from_float<TO>(keep[e].v[k] * inv * (offset + w.v[k]));
+            for (int k = 0; k < 4; ++k) r.v[k] = from_float<TO>(keep[e].v[k] * inv * (offset + w[e].v[k]));
             *reinterpret_cast<Quad<TO>*>(o + i) = r;
         }
     }
