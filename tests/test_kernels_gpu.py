@@ -325,7 +325,9 @@ def test_paged_attention_finds_one_far_key(dtype):
                                    (200, 777, 64), (2, 16, 32), (16, 20, 1056), (16, 2048, 8192), (12, 100, 4128),
                                    (9, 3072, 24576), (11, 16500, 320),
                                    # more than 64 rows of an unsplit product (logits of many rows): groups of 64 rows in one launch
-                                   (65, 24600, 64), (130, 25001, 96), (256, 26000, 128), (200, 50000, 32)])
+                                   (65, 24600, 64), (130, 25001, 96), (256, 26000, 128), (200, 50000, 32),
+                                   # some hundred rows and a long K axis: the tiled product, its K axis in pieces
+                                   (65, 2048, 16384), (300, 96, 8192), (513, 200, 8192), (1024, 48, 16384), (130, 3072, 24576)])
 def test_linear(dtype, m, n, k):
     torch.manual_seed(4)
     for out_dtype in {dtype, torch.float32}:
@@ -367,7 +369,7 @@ def test_tile_weight_is_the_documented_permutation():
 
 
 @pytest.mark.parametrize("m,n,k", [(8, 2048, 16384), (5, 2560, 2048), (64, 1000, 1024), (1, 777, 512), (16, 1000, 8192),
-                                   (3, 3072, 24576), (40, 2048, 16384)])
+                                   (3, 3072, 24576), (40, 2048, 16384), (100, 2048, 16384), (512, 96, 8192), (1025, 96, 8192)])
 def test_linear_leaves_partial_sums_to_the_caller(m, n, k):
     torch.manual_seed(8)
     x = torch.randn(m, k, device=DEV).to(torch.bfloat16)
@@ -392,7 +394,9 @@ def test_linear_leaves_partial_sums_to_the_caller(m, n, k):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("act", ["gelu_tanh", "silu"])
 @pytest.mark.parametrize("m,inter,k", [(8, 16384, 2048), (3, 250, 96), (64, 777, 128), (100, 384, 96), (17, 112, 80),
-                                       (16, 1000, 4128), (1, 250, 96), (13, 2000, 3072), (16, 20, 32)])
+                                       (16, 1000, 4128), (1, 250, 96), (13, 2000, 3072), (16, 20, 32),
+                                       # some hundred rows: the tiled product with the activation in its registers
+                                       (65, 4000, 2048), (130, 250, 128), (256, 777, 320), (200, 64, 64)])
 def test_gated_linear(dtype, act, m, inter, k):
     torch.manual_seed(9)
 

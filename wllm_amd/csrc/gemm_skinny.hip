@@ -207,6 +207,16 @@ __global__ void split_sum_kernel(const float* __restrict__ partial, TO* __restri
     }
 }
 
+// out[i] = the sum in order of partial[p * total + i], p < splits.
+WLLM_API int wllm_split_sum(const float* partial, void* out, int out_bf16, long long total, int splits, hipStream_t stream) {
+    if (total < 1 || splits < 1) return -1;
+    const long long want = (total + 255) / 256;
+    const int blocks = static_cast<int>(want < 4096 ? want : 4096);
+    if (out_bf16) split_sum_kernel<bf16><<<blocks, 256, 0, stream>>>(partial, static_cast<bf16*>(out), total, splits);
+    else split_sum_kernel<float><<<blocks, 256, 0, stream>>>(partial, static_cast<float*>(out), total, splits);
+    return launch_status();
+}
+
 // Returns 0, a HIP error code, or -1 for sizes this kernel does not take.
 // `partial` must hold splits * M * N floats when splits > 1; with `out` null the partial sums
 // are the result and nothing adds them.
