@@ -53,8 +53,10 @@ union Pack16 {
 
 __device__ __forceinline__ uint16_t bf16_bits(float f) { return from_float<bf16>(f).bits; }
 
+// Three workgroups a compute unit (168 registers a lane) where the kernel fits them without spilling;
+// two for the head sizes and page sizes whose staging needs more.
 template <int HD, bool V16>
-__global__ void __launch_bounds__(256, 3)
+__global__ void __launch_bounds__(256, (HD <= 160 || (HD == 256 && V16)) ? 3 : 2)
 paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict__ cache,
                             const int* __restrict__ block_tables, const int* __restrict__ items,
                             const int* __restrict__ live_items, const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
