@@ -69,7 +69,7 @@ class EmulatedKernels:
         sumsq.copy_((residual.to(self.acc) ** 2).view(residual.shape[0], -1, 16).sum(-1).to(torch.float32))
 
     def qkv_rope_takes(self, rows, dtype, in_features, head_dim, rotary_dim):
-        return self.fused_qkv and rotary_dim == head_dim and rows <= 16
+        return self.fused_qkv and rotary_dim == head_dim and rows <= 32
 
     def qkv_rope(self, x, weight, tiles, qkv, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads,
                  head_dim, page_size):

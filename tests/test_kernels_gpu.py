@@ -464,11 +464,14 @@ def test_feed_tokens_writes_only_the_named_places():
 @pytest.mark.parametrize("tiled", [False, True])
 @pytest.mark.parametrize("m,k,nh,nkv,d,ps,with_bias,with_cache", [
     (8, 2048, 8, 1, 256, 16, False, True), (16, 96, 3, 1, 32, 4, True, True), (1, 320, 4, 2, 64, 8, False, True),
-    (5, 4128, 2, 2, 96, 12, True, True), (3, 64, 5, 5, 128, 16, False, False)])
+    (5, 4128, 2, 2, 96, 12, True, True), (3, 64, 5, 5, 128, 16, False, False),
+    # 17 to 32 tokens: two tiles of 16
+    (17, 2048, 8, 1, 256, 16, False, True), (29, 320, 4, 2, 64, 8, True, True), (32, 3072, 2, 2, 256, 16, False, True),
+    (20, 96, 3, 1, 32, 4, True, False)])
 def test_qkv_projection_rotation_and_cache_write_in_one_kernel(tiled, m, k, nh, nkv, d, ps, with_bias, with_cache):
     dtype = torch.bfloat16
     assert ops.qkv_rope_takes(m, dtype, k, d, d)
-    assert not ops.qkv_rope_takes(17, dtype, k, d, d) and not ops.qkv_rope_takes(m, torch.float32, k, d, d)
+    assert not ops.qkv_rope_takes(33, dtype, k, d, d) and not ops.qkv_rope_takes(m, torch.float32, k, d, d)
     assert not ops.qkv_rope_takes(m, dtype, k, d, d // 2), "heads rotated in part take the two kernels"
     width = (nh + 2 * nkv) * d
 

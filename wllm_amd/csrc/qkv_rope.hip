@@ -1,5 +1,5 @@
 // The query/key/value projection of a decode step, its bias, the rotation of queries and keys and
-// the write of keys and values into their pages, in one kernel: for at most 16 tokens, bfloat16,
+// the write of keys and values into their pages, in one kernel: for at most 32 tokens, bfloat16,
 // heads whose size is a multiple of 32 and that are rotated whole.
 //
 // out[m, :] = x[m, :] . w^T as in `gemm_skinny.hip` (weights as the A operand of
@@ -12,6 +12,9 @@
 // pair is turned in registers by position * inv_freq[j] (angle, sine, cosine in float32), written
 // to the row of queries, keys and values, and keys go to the cache as [page_size, HD], values
 // transposed as [HD, page_size].  Heads of values take the same path without the rotation.
+// 17 to 32 tokens are two tiles of 16: every fragment of the weights then feeds two products.  (Three
+// and four tiles were measured too: with fewer steps in flight to fit the registers they are no faster
+// than the product and the rotation as two kernels.)
 #include "common.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
@@ -23,78 +26,13 @@ union QFrag {
 };
 
 constexpr int kQkvWaves = 8;
-constexpr int kQkvInFlight = 8;     // steps of 32 keys whose loads a wavefront keeps in flight, per band
 
-template <bool TILED>
-__global__ void __launch_bounds__(kQkvWaves * 64)
-qkv_rope_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const float* __restrict__ bias,
-                const int* __restrict__ positions, const float* __restrict__ inv_freq, const int* __restrict__ slots,
-                bf16* __restrict__ qkv, bf16* __restrict__ cache, int M, int K, int num_heads, int num_kv_heads, int HD,
-                int page_size, long long num_pages) {
-    __shared__ float4_t red[(kQkvWaves - 1) * kWave * 2];
-    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-    const int i = lane % 16, g = lane / 16;
-    const int pairs = HD / 32;                          // pairs of bands in a head
-    const int head = blockIdx.x / pairs, p = blockIdx.x % pairs;
-    const int band_lo = head * (HD / 16) + p, band_hi = band_lo + pairs;
-    const int steps = K / 32;
-    const int per = (steps + kQkvWaves - 1) / kQkvWaves;
-    const int s0 = wave * per, s1 = min(steps, s0 + per);
-    constexpr int kStep = TILED ? 512 : 32;             // elements from one step of 32 keys to the next
-    const bf16* lo = TILED ? w + static_cast<size_t>(band_lo) * steps * 512 + lane * 8
-                           : w + (static_cast<size_t>(band_lo) * 16 + i) * K + 8 * g;
-    const bf16* hi = TILED ? w + static_cast<size_t>(band_hi) * steps * 512 + lane * 8
-                           : w + (static_cast<size_t>(band_hi) * 16 + i) * K + 8 * g;
-    const bf16* xp = x + static_cast<size_t>(min(i, M - 1)) * K + 8 * g;
-    const bool x_row = i < M;
-    // what the first wavefront needs after the sums, asked for now so that it has arrived by then
-    const int j0 = p * 16 + 4 * g, half = HD / 2;
-    const bool rotated = head < num_heads + num_kv_heads && inv_freq != nullptr;
-    float pos = 0.f;
-    float4 freq = make_float4(0.f, 0.f, 0.f, 0.f);
-    int slot = -1;
-    if (wave == 0 && x_row) {
-        if (rotated) {
-            pos = static_cast<float>(positions[i]);
-            freq = *reinterpret_cast<const float4*>(inv_freq + j0);
-        }
-        if (cache && head >= num_heads) slot = slots[i];
-    }
-    constexpr int U = kQkvInFlight;
-    QFrag cl[U], ch[U], cx[U];
-    auto load_step = [&](int u, int at) {
-        const bool ok = at < s1;
-        cl[u].u = ok ? *reinterpret_cast<const uint4*>(lo + static_cast<size_t>(at) * kStep) : make_uint4(0, 0, 0, 0);
-        ch[u].u = ok ? *reinterpret_cast<const uint4*>(hi + static_cast<size_t>(at) * kStep) : make_uint4(0, 0, 0, 0);
-        cx[u].u = ok && x_row ? *reinterpret_cast<const uint4*>(xp + static_cast<size_t>(at) * 32) : make_uint4(0, 0, 0, 0);
-    };
-#pragma unroll
-    for (int u = 0; u < U; ++u) load_step(u, s0 + u);
-    float4_t acc_lo = float4_t{0.f, 0.f, 0.f, 0.f}, acc_hi = float4_t{0.f, 0.f, 0.f, 0.f};
-    for (int s = s0; s < s1; s += U) {
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            acc_lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cl[u].v, cx[u].v, acc_lo, 0, 0, 0);
-            acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ch[u].v, cx[u].v, acc_hi, 0, 0, 0);
-            load_step(u, s + U + u);
-        }
-    }
-    if (wave > 0) {
-        red[((wave - 1) * kWave + lane) * 2] = acc_lo;
-        red[((wave - 1) * kWave + lane) * 2 + 1] = acc_hi;
-    }
-    __syncthreads();
-    if (wave > 0) return;
-#pragma unroll
-    for (int q = 0; q < kQkvWaves - 1; ++q) {
-        acc_lo += red[(q * kWave + lane) * 2];
-        acc_hi += red[(q * kWave + lane) * 2 + 1];
-    }
-    // lane (i, g): token m = i, elements j .. j + 3 of the head and their partners
-    const int m = i;
-    if (m >= M) return;
-    const int width = (num_heads + 2 * num_kv_heads) * HD;
-    const int col = head * HD + j0;
+// What the first wavefront does with one token's sums of a pair of bands: bias, the rotation of the
+// pair (element j of the head with j + HD/2), the row of queries, keys and values, and the cache.
+__device__ __forceinline__ void finish_row(float4_t acc_lo, float4_t acc_hi, const float* __restrict__ bias, int col, int half,
+                                           bool rotated, float pos, const float* fr, bf16* __restrict__ qkv, int m, int width,
+                                           bf16* __restrict__ cache, int head, int num_heads, int num_kv_heads, int slot,
+                                           int page_size, long long num_pages, size_t page_elems, int HD, int j0) {
     if (bias) {
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
@@ -103,7 +41,6 @@ qkv_rope_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const fl
         }
     }
     if (rotated) {
-        const float fr[4] = {freq.x, freq.y, freq.z, freq.w};
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             float s, c;
@@ -127,7 +64,6 @@ qkv_rope_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const fl
     const long long page = slot / page_size;
     const int off = slot % page_size;
     if (slot < 0 || page >= num_pages) return;
-    const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * HD;
     bf16* kpage = cache + page * page_elems;
     if (head < num_heads + num_kv_heads) {
         bf16* dst = kpage + (static_cast<size_t>(head - num_heads) * page_size + off) * HD + j0;
@@ -149,22 +85,128 @@ qkv_rope_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const fl
     }
 }
 
+template <bool TILED, int MT>
+__global__ void __launch_bounds__(kQkvWaves * 64)
+qkv_rope_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const float* __restrict__ bias,
+                const int* __restrict__ positions, const float* __restrict__ inv_freq, const int* __restrict__ slots,
+                bf16* __restrict__ qkv, bf16* __restrict__ cache, int M, int K, int num_heads, int num_kv_heads, int HD,
+                int page_size, long long num_pages) {
+    __shared__ float4_t red[(kQkvWaves - 1) * kWave * 2 * MT];
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int i = lane % 16, g = lane / 16;
+    const int pairs = HD / 32;                          // pairs of bands in a head
+    const int head = blockIdx.x / pairs, p = blockIdx.x % pairs;
+    const int band_lo = head * (HD / 16) + p, band_hi = band_lo + pairs;
+    const int steps = K / 32;
+    const int per = (steps + kQkvWaves - 1) / kQkvWaves;
+    const int s0 = wave * per, s1 = min(steps, s0 + per);
+    constexpr int kStep = TILED ? 512 : 32;             // elements from one step of 32 keys to the next
+    const bf16* lo = TILED ? w + static_cast<size_t>(band_lo) * steps * 512 + lane * 8
+                           : w + (static_cast<size_t>(band_lo) * 16 + i) * K + 8 * g;
+    const bf16* hi = TILED ? w + static_cast<size_t>(band_hi) * steps * 512 + lane * 8
+                           : w + (static_cast<size_t>(band_hi) * 16 + i) * K + 8 * g;
+    const bf16* xp[MT];
+    bool x_row[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        xp[t] = x + static_cast<size_t>(min(16 * t + i, M - 1)) * K + 8 * g;
+        x_row[t] = 16 * t + i < M;
+    }
+    // what the first wavefront needs after the sums, asked for now so that it has arrived by then
+    const int j0 = p * 16 + 4 * g, half = HD / 2;
+    const bool rotated = head < num_heads + num_kv_heads && inv_freq != nullptr;
+    float pos[MT];
+    float4 freq = make_float4(0.f, 0.f, 0.f, 0.f);
+    int slot[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        pos[t] = 0.f;
+        slot[t] = -1;
+        if (wave == 0 && x_row[t]) {
+            if (rotated) pos[t] = static_cast<float>(positions[16 * t + i]);
+            if (cache && head >= num_heads) slot[t] = slots[16 * t + i];
+        }
+    }
+    if (wave == 0 && rotated) freq = *reinterpret_cast<const float4*>(inv_freq + j0);
+    constexpr int U = 8;        // steps of 32 keys whose loads a wavefront keeps in flight, per band
+    QFrag cl[U], ch[U], cx[U][MT];
+    auto load_step = [&](int u, int at) {
+        const bool ok = at < s1;
+        cl[u].u = ok ? *reinterpret_cast<const uint4*>(lo + static_cast<size_t>(at) * kStep) : make_uint4(0, 0, 0, 0);
+        ch[u].u = ok ? *reinterpret_cast<const uint4*>(hi + static_cast<size_t>(at) * kStep) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+            cx[u][t].u = ok && x_row[t] ? *reinterpret_cast<const uint4*>(xp[t] + static_cast<size_t>(at) * 32) : make_uint4(0, 0, 0, 0);
+    };
+#pragma unroll
+    for (int u = 0; u < U; ++u) load_step(u, s0 + u);
+    float4_t acc_lo[MT], acc_hi[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        acc_lo[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+        acc_hi[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    for (int s = s0; s < s1; s += U) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                acc_lo[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cl[u].v, cx[u][t].v, acc_lo[t], 0, 0, 0);
+                acc_hi[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ch[u].v, cx[u][t].v, acc_hi[t], 0, 0, 0);
+            }
+            load_step(u, s + U + u);
+        }
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            red[(((wave - 1) * kWave + lane) * MT + t) * 2] = acc_lo[t];
+            red[(((wave - 1) * kWave + lane) * MT + t) * 2 + 1] = acc_hi[t];
+        }
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int q = 0; q < kQkvWaves - 1; ++q)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+            acc_lo[t] += red[((q * kWave + lane) * MT + t) * 2];
+            acc_hi[t] += red[((q * kWave + lane) * MT + t) * 2 + 1];
+        }
+    const int width = (num_heads + 2 * num_kv_heads) * HD;
+    const int col = head * HD + j0;
+    const float fr[4] = {freq.x, freq.y, freq.z, freq.w};
+    const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * HD;
+    // lane (i, g): token m = 16 t + i, elements j .. j + 3 of the head and their partners
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        const int m = 16 * t + i;
+        if (m >= M) continue;
+        finish_row(acc_lo[t], acc_hi[t], bias, col, half, rotated, pos[t], fr, qkv, m, width, cache, head, num_heads,
+                   num_kv_heads, slot[t], page_size, num_pages, page_elems, HD, j0);
+    }
+}
 // Returns 0, a HIP error code, or -1 for sizes this kernel does not take (the caller then runs the
 // product and the rotation as two kernels).  `w` is the stacked [q; k; v] weight, row by row or
 // (`tiled`) its tile-major copy.  inv_freq has HD/2 entries or is null (no rotation).
 WLLM_API int wllm_qkv_rope(const void* x, const void* w, int tiled, const float* bias, const int* positions,
                            const float* inv_freq, const int* slots, void* qkv, void* cache, long long num_pages, int M,
                            int K, int num_heads, int num_kv_heads, int head_dim, int page_size, hipStream_t stream) {
-    if (M < 1 || M > 16 || K < 32 || K % 32 != 0 || head_dim < 32 || head_dim % 32 != 0 || num_heads < 1 || num_kv_heads < 1 ||
+    if (M < 1 || M > 32 || K < 32 || K % 32 != 0 || head_dim < 32 || head_dim % 32 != 0 || num_heads < 1 || num_kv_heads < 1 ||
         page_size < 1)
         return -1;
     const int grid = (num_heads + 2 * num_kv_heads) * (head_dim / 32);
-#define LAUNCH(T)                                                                                                      \
-    qkv_rope_kernel<T><<<grid, kQkvWaves * 64, 0, stream>>>(                                                           \
+#define LAUNCH(T, MT)                                                                                                  \
+    qkv_rope_kernel<T, MT><<<grid, kQkvWaves * 64, 0, stream>>>(                                                       \
         static_cast<const bf16*>(x), static_cast<const bf16*>(w), bias, positions, inv_freq, slots, static_cast<bf16*>(qkv), \
         static_cast<bf16*>(cache), M, K, num_heads, num_kv_heads, head_dim, page_size, num_pages)
-    if (tiled) LAUNCH(true);
-    else LAUNCH(false);
+    if (tiled) {
+        if (M <= 16) LAUNCH(true, 1);
+        else LAUNCH(true, 2);
+    } else {
+        if (M <= 16) LAUNCH(false, 1);
+        else LAUNCH(false, 2);
+    }
 #undef LAUNCH
     return launch_status();
 }

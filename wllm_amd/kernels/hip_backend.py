@@ -149,9 +149,9 @@ class HipBackend:
 
     @staticmethod
     def qkv_rope_takes(rows: int, dtype, in_features: int, head_dim: int, rotary_dim: int) -> bool:
-        """The fused projection, rotation and cache write: bfloat16, at most 16 tokens, heads of a
+        """The fused projection, rotation and cache write: bfloat16, at most 32 tokens, heads of a
         multiple of 32 that are rotated whole."""
-        return (dtype == torch.bfloat16 and 1 <= rows <= 16 and in_features % 32 == 0 and head_dim % 32 == 0
+        return (dtype == torch.bfloat16 and 1 <= rows <= 32 and in_features % 32 == 0 and head_dim % 32 == 0
                 and rotary_dim == head_dim)
 
     def qkv_rope(self, x, weight, tiles, qkv, bias, positions, inv_freq, slots, cache, num_heads, num_kv_heads,
