@@ -70,14 +70,31 @@ template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float4_t v) {
 // their own that read the same weights.  The workgroups of a tile's row groups get indices that are 8
 // apart, so they are dispatched one after the other to the same XCD (workgroup index modulo 8) and the
 // later ones find the weights in that XCD's L2 instead of asking HBM for them again.
-template <int MT, int NT, typename TO, bool TILED>
+template <int MT, int NT, typename TO, bool TILED, int KB = 16 / NT, int CS = 0>
 __global__ void __launch_bounds__(256)
 gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* __restrict__ out,
-                   float* __restrict__ partial, int M, int N, int K, int k_per_split, int chunk, int row_groups) {
+                   float* __restrict__ partial, int M, int N, int K, int k_per_split, int chunk, int row_groups, int splits) {
     extern __shared__ uint4 xs[];                 // [MT*16][chunk/8 + 1]
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const int i = lane % 16, g = lane / 16;
     int tile_group = blockIdx.x;                  // which 64 * NT weight rows
+    int split = 0;                                // which piece of the K axis
+    if (splits > 1) {
+        // The workgroups of one piece of the K axis read the same part of x: they get indices that are
+        // equal modulo 8, so they run on one XCD and all but the first find that part in its L2.  (The
+        // XCDs' caches are separate: a part of x that all eight of them read crosses the fabric eight
+        // times, which at 64 rows and a long K axis is a quarter of what the weights take.)
+        const int xcd = blockIdx.x % 8, j = blockIdx.x / 8;
+        if (splits >= 8) {
+            const int per = splits / 8;           // splits is a power of two
+            split = xcd * per + j % per;
+            tile_group = j / per;
+        } else {
+            split = xcd % splits;
+            tile_group = xcd / splits + (8 / splits) * j;
+            if (tile_group * 64 * NT >= N) return;     // the grid is padded to whole rounds of 8
+        }
+    }
     if (row_groups > 1) {
         const int xcd = blockIdx.x % 8, j = blockIdx.x / 8;
         const int rg = j % row_groups;
@@ -87,7 +104,7 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* _
         M = min(64, M - rg * 64);
     }
     const int n0 = (tile_group * 4 + wave) * 16 * NT;
-    const int k_begin = blockIdx.y * k_per_split, k_end = min(K, k_begin + k_per_split);
+    const int k_begin = split * k_per_split, k_end = min(K, k_begin + k_per_split);
     const int stride = chunk / 8 + 1;             // in uint4; the odd stride spreads rows over the banks
     constexpr int kStep = TILED ? 512 : 32;       // elements from one step of 32 keys to the next
     const bf16* wp[NT];
@@ -109,7 +126,7 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* _
     // The weight stream: kBatch 16-byte loads per lane and tile are in flight, the first before x is
     // staged at all; a register is refilled with the step kBatch further on as soon as its products
     // have been issued.
-    constexpr int kBatch = 16 / NT;
+    constexpr int kBatch = KB;
     const bool live = n0 < N;
     const int steps = (k_end - k_begin) / 32;
     Frag cur[NT][kBatch];
@@ -123,27 +140,75 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* _
     // x is staged chunk by chunk; the loads of the next chunk are in flight during the products
     constexpr int kXRegs = 8;                     // 16-byte pieces of a chunk per thread (MT*16*chunk/8 <= 2048)
     uint4 xreg[kXRegs];
+    // A thread's pieces are (row, 8 keys) pairs of the whole chunk's shape, piece number threadIdx.x +
+    // 256 u; their places are worked out once, not per chunk (a division by a run-time number costs
+    // some forty instructions), and a shorter last chunk only leaves pieces out.
+    const int vecs_full = chunk / 8;
+    int x_col[kXRegs], x_row[kXRegs];
+    {
+        const int dq = 256 / vecs_full, dr = 256 % vecs_full;
+        int m = threadIdx.x / vecs_full, c = threadIdx.x % vecs_full;
+#pragma unroll
+        for (int u = 0; u < kXRegs; ++u) {
+            x_row[u] = m < MT * 16 ? m : -1;
+            x_col[u] = c;
+            m += dq;
+            c += dr;
+            if (c >= vecs_full) { c -= vecs_full; ++m; }
+        }
+    }
     auto fetch_x = [&](int kc) {
         const int vecs = min(chunk, k_end - kc) / 8;
 #pragma unroll
         for (int u = 0; u < kXRegs; ++u) {
-            const int idx = threadIdx.x + u * 256;
-            const int m = idx / vecs, c = idx % vecs;
-            xreg[u] = (idx < MT * 16 * vecs && m < M) ? *reinterpret_cast<const uint4*>(x + static_cast<size_t>(m) * K + kc + c * 8)
-                                                      : make_uint4(0, 0, 0, 0);
+            const int m = x_row[u], c = x_col[u];
+            xreg[u] = (m >= 0 && m < M && c < vecs) ? *reinterpret_cast<const uint4*>(x + static_cast<size_t>(m) * K + kc + c * 8)
+                                                    : make_uint4(0, 0, 0, 0);
         }
     };
     fetch_x(k_begin);
     int step = 0;
-    for (int kc = k_begin; kc < k_end; kc += chunk) {
+    if constexpr (CS > 0) {
+        // chunk == 32 * CS and the weights' loads run KB / CS chunks of x ahead: a register's step is
+        // fixed by its place among the KB steps, so the chunks of a batch are unrolled
+        for (int kb = k_begin; kb < k_end; kb += 32 * KB) {
+#pragma unroll
+            for (int sc = 0; sc < KB / CS; ++sc) {
+                const int kc = kb + sc * 32 * CS;
+                if (kc >= k_end) break;
+                const int len = min(32 * CS, k_end - kc);
+                const int vecs = len / 8;
+                __syncthreads();
+#pragma unroll
+                for (int u = 0; u < kXRegs; ++u)
+                    if (x_row[u] >= 0 && x_col[u] < vecs) xs[x_row[u] * stride + x_col[u]] = xreg[u];
+                __syncthreads();
+                if (kc + 32 * CS < k_end) fetch_x(kc + 32 * CS);
+#pragma unroll
+                for (int u = 0; u < CS; ++u) {
+                    if (32 * u < len) {
+                        Frag b[MT];
+#pragma unroll
+                        for (int t = 0; t < MT; ++t) b[t].u = xs[(t * 16 + i) * stride + 4 * u + g];
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                            for (int t = 0; t < MT; ++t)
+                                acc[nt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[nt][sc * CS + u].v, b[t].v, acc[nt][t], 0, 0, 0);
+                        load_step(sc * CS + u, step + sc * CS + u + KB);
+                    }
+                }
+            }
+            step += KB;
+        }
+    }
+    for (int kc = k_begin; CS == 0 && kc < k_end; kc += chunk) {
         const int len = min(chunk, k_end - kc);   // a multiple of 32 * kBatch, except the last
         const int vecs = len / 8;
         __syncthreads();
 #pragma unroll
-        for (int u = 0; u < kXRegs; ++u) {
-            const int idx = threadIdx.x + u * 256;
-            if (idx < MT * 16 * vecs) xs[(idx / vecs) * stride + idx % vecs] = xreg[u];
-        }
+        for (int u = 0; u < kXRegs; ++u)
+            if (x_row[u] >= 0 && x_col[u] < vecs) xs[x_row[u] * stride + x_col[u]] = xreg[u];
         __syncthreads();
         if (kc + chunk < k_end) fetch_x(kc + chunk);
         for (int k = 0; k < len; k += 32 * kBatch) {
@@ -174,7 +239,7 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* _
         for (int t = 0; t < MT; ++t) {
             const int m = t * 16 + i;
             if (m >= M) continue;
-            if (gridDim.y == 1) {
+            if (splits == 1) {
                 TO* o = out + static_cast<size_t>(m) * N + n;
                 if (n + 3 < N && (N % 4 == 0)) {
                     store4<TO>(o, acc[nt][t]);
@@ -184,7 +249,7 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* _
                         if (n + v < N) o[v] = from_float<TO>(acc[nt][t][v]);
                 }
             } else {
-                float* o = partial + (static_cast<size_t>(blockIdx.y) * M + m) * N + n;
+                float* o = partial + (static_cast<size_t>(split) * M + m) * N + n;
                 if (n + 3 < N && (N % 4 == 0)) {
                     *reinterpret_cast<float4_t*>(o) = acc[nt][t];
                 } else {
@@ -250,13 +315,20 @@ WLLM_API int wllm_gemm_skinny(const void* x, const void* w, int tiled, void* out
     // with row groups the tile groups are padded to a multiple of 8, one stripe per XCD (tile groups beyond
     // the last hold no live weight rows and write nothing)
     const int tile_groups = (N + 64 * nt - 1) / (64 * nt);
-    const long long blocks = row_groups > 1 ? static_cast<long long>((tile_groups + 7) / 8 * 8) * row_groups : tile_groups;
+    long long blocks = row_groups > 1 ? static_cast<long long>((tile_groups + 7) / 8 * 8) * row_groups : tile_groups;
+    if (splits > 1) {
+        // one index for pieces of K and tile groups, the pieces spread over the XCDs (see the kernel)
+        if ((splits & (splits - 1)) != 0) return -1;
+        const int q = splits >= 8 ? 1 : 8 / splits;
+        blocks = splits >= 8 ? static_cast<long long>(splits) * tile_groups
+                             : static_cast<long long>((tile_groups + q - 1) / q) * 8;
+    }
     if (blocks > 0x7fffffffLL) return -1;
-    const dim3 grid(static_cast<unsigned>(blocks), splits);
+    const dim3 grid(static_cast<unsigned>(blocks));
 #define LAUNCH_T(MT, NT, TO, T)                                                                                  \
     gemm_skinny_kernel<MT, NT, TO, T><<<grid, 256, smem, stream>>>(static_cast<const bf16*>(x), static_cast<const bf16*>(w), \
                                                                    static_cast<TO*>(out), partial, M, N, K, k_per_split, chunk, \
-                                                                   row_groups)
+                                                                   row_groups, splits)
 #define LAUNCH(MT, NT, TO)                  \
     if (tiled) LAUNCH_T(MT, NT, TO, true);  \
     else LAUNCH_T(MT, NT, TO, false)
@@ -318,8 +390,8 @@ struct NormOnLoad {
     float eps, offset;
 };
 
-template <int MT, int ACT, bool TILED, int TPW, bool NORM, int XR>
-__global__ void __launch_bounds__(TPW * 128, MT == 1 ? (NORM && XR > 2 ? 3 : 4) : (MT == 2 ? 3 : 2))
+template <int MT, int ACT, bool TILED, int TPW, bool NORM, int XR, int KB = 8>
+__global__ void __launch_bounds__(TPW * 128, KB > 8 ? 1 : (MT == 1 ? (NORM && XR > 2 ? 3 : 4) : (MT == 2 ? 3 : 2)))
 gemm_skinny_gated_kernel(const bf16* __restrict__ x, NormOnLoad norm, const bf16* __restrict__ w, bf16* __restrict__ out,
                          int M, int inter, int K, int chunk) {
     extern __shared__ uint4 xs[];                 // two halves of [MT*16][chunk/8 + 1]
@@ -349,7 +421,7 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, NormOnLoad norm, const bf16
     // The weight stream: kBatch 16-byte loads per lane and stream are in flight; a register is
     // refilled with the step kBatch further on as soon as its product has been issued, so the loads
     // in flight take 16 registers a stream and not twice that, and two workgroups fit a compute unit.
-    constexpr int kBatch = 8;       // per stream; two streams
+    constexpr int kBatch = KB;      // per stream; two streams
     const bool live = n0 < inter;
     const int steps = half_k / 32;
     Frag curg[kBatch], curu[kBatch];
@@ -382,6 +454,22 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, NormOnLoad norm, const bf16
     constexpr int kXRegs = NORM ? XR : (MT == 1 ? 4 : 8);       // pieces of a chunk per thread
     uint4 xreg[NORM ? 1 : kXRegs];
     float4 xraw[NORM ? kXRegs : 1][2], wraw[2];
+    // a thread's pieces of a chunk as (row, 8 keys) pairs of the whole chunk's shape, worked out once: a
+    // division by a run-time number per piece and chunk would cost more than the products
+    int x_col[NORM ? 1 : kXRegs], x_row[NORM ? 1 : kXRegs];
+    if (!NORM) {
+        const int vecs_full = chunk / 8;
+        const int dq = kHalfThreads / vecs_full, dr = kHalfThreads % vecs_full;
+        int m = tid_half / vecs_full, c = tid_half % vecs_full;
+#pragma unroll
+        for (int u = 0; u < (NORM ? 1 : kXRegs); ++u) {
+            x_row[u] = m < MT * 16 ? m : -1;
+            x_col[u] = c;
+            m += dq;
+            c += dr;
+            if (c >= vecs_full) { c -= vecs_full; ++m; }
+        }
+    }
     auto fetch_x = [&](int kc) {
         if (NORM) {
             // chunks of 256 keys: a thread's pieces are rows tid_half / 32 + (kHalfThreads / 32) * u at the
@@ -402,9 +490,8 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, NormOnLoad norm, const bf16
         const int vecs = min(chunk, half_k - kc) / 8;
 #pragma unroll
         for (int u = 0; u < (NORM ? 1 : kXRegs); ++u) {
-            const int idx = tid_half + u * kHalfThreads;
-            const int m = idx / vecs, c = idx % vecs;
-            xreg[u] = (idx < MT * 16 * vecs && m < M)
+            const int m = x_row[u], c = x_col[u];
+            xreg[u] = (m >= 0 && m < M && c < vecs)
                           ? *reinterpret_cast<const uint4*>(x + static_cast<size_t>(m) * K + k_begin + kc + c * 8)
                           : make_uint4(0, 0, 0, 0);
         }
@@ -428,13 +515,40 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, NormOnLoad norm, const bf16
             return;
         }
 #pragma unroll
-        for (int u = 0; u < (NORM ? 1 : kXRegs); ++u) {
-            const int idx = tid_half + u * kHalfThreads;
-            if (idx < MT * 16 * vecs) xh[(idx / vecs) * stride + idx % vecs] = xreg[u];
-        }
+        for (int u = 0; u < (NORM ? 1 : kXRegs); ++u)
+            if (x_row[u] >= 0 && x_col[u] < vecs) xh[x_row[u] * stride + x_col[u]] = xreg[u];
     };
     fetch_x(0);
-    for (int kc = 0; kc < half_k; kc += chunk) {
+    if constexpr (KB > 8) {
+        // chunks of 256 keys (8 steps), the weights' loads KB / 8 chunks ahead
+        for (int kb = 0; kb < half_k; kb += 32 * KB) {
+#pragma unroll
+            for (int sc = 0; sc < KB / 8; ++sc) {
+                const int kc = kb + sc * 256;
+                if (kc >= half_k) break;
+                const int len = min(256, half_k - kc);
+                __syncthreads();
+                stage_x(len / 8);
+                __syncthreads();
+                if (kc + 256 < half_k) fetch_x(kc + 256);
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    if (32 * u < len) {
+#pragma unroll
+                        for (int t = 0; t < MT; ++t) {
+                            Frag b;
+                            b.u = xh[(t * 16 + i) * stride + 4 * u + g];
+                            accg[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(curg[sc * 8 + u].v, b.v, accg[t], 0, 0, 0);
+                            accu[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(curu[sc * 8 + u].v, b.v, accu[t], 0, 0, 0);
+                        }
+                        load_step(sc * 8 + u, step + sc * 8 + u + KB);
+                    }
+                }
+            }
+            step += KB;
+        }
+    }
+    for (int kc = 0; KB == 8 && kc < half_k; kc += chunk) {
         const int len = min(chunk, half_k - kc);      // a multiple of 32 * kBatch, except the last
         __syncthreads();
         stage_x(len / 8);
@@ -510,16 +624,16 @@ static int gated_launch(const void* x, NormOnLoad norm, bool with_norm, const vo
     if (smem > 160 * 1024 - 4096 || mt * 16 * (chunk / 8) > tpw * 64 * x_regs || (chunk % 256 != 0 && chunk < K / 2))
         return -1;
     const dim3 grid((inter + 16 * tpw - 1) / (16 * tpw));
-#define LAUNCH_K(MT, A, T, TPW, NORM, XR)                                                                            \
+#define LAUNCH_K(MT, A, T, TPW, NORM, XR, ...)                                                                            \
     do {                                                                                                              \
         static bool roomy = false;     /* more than 64 KiB of shared memory must be asked for once */                \
         if (smem > 65536 && !roomy) {                                                                                 \
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_gated_kernel<MT, A, T, TPW, NORM, XR>), \
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_gated_kernel<MT, A, T, TPW, NORM, XR, ##__VA_ARGS__>), \
                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 4096) != hipSuccess)    \
                 return launch_status();                                                                               \
             roomy = true;                                                                                             \
         }                                                                                                             \
-        gemm_skinny_gated_kernel<MT, A, T, TPW, NORM, XR><<<grid, TPW * 128, smem, stream>>>(                        \
+        gemm_skinny_gated_kernel<MT, A, T, TPW, NORM, XR, ##__VA_ARGS__><<<grid, TPW * 128, smem, stream>>>(                        \
             static_cast<const bf16*>(x), norm, static_cast<const bf16*>(w), static_cast<bf16*>(out), M, inter, K, chunk); \
     } while (0)
 #define LAUNCH_T(MT, A, T, TPW) LAUNCH_K(MT, A, T, TPW, false, 4)
@@ -541,6 +655,10 @@ static int gated_launch(const void* x, NormOnLoad norm, bool with_norm, const vo
         case 3: LAUNCH(3, A); break; \
         default: LAUNCH(4, A); break; \
     }
+    static const int x_kb = getenv("WLLM_X_GATED_KB") ? atoi(getenv("WLLM_X_GATED_KB")) : 0;     // EXPERIMENT
+    if (x_kb && !with_norm && mt == 4 && tiled && activation == 0 && chunk == 256) {
+        LAUNCH_K(4, 0, true, 4, false, 4, 16);
+    } else
     if (with_norm) {
         if (activation == 0) { LAUNCH_N(0) } else { LAUNCH_N(1) }
     } else {
