@@ -164,15 +164,15 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
         const bf16* vbase0 = cache + static_cast<size_t>(table[vpage0]) * page_elems + v_off + vslot0;
         const bf16* vbase1 = cache + static_cast<size_t>(V16 ? 0 : table[vpage1]) * page_elems + v_off + vslot1;
 #pragma unroll
-        for (int j = 0; j < DT; ++j) kraw[j] = *reinterpret_cast<const uint4_t*>(kpiece[j]);
+        for (int j = 0; j < DT; ++j) kraw[j] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(kpiece[j]));
 #pragma unroll
         for (int t = 0; t < DT; ++t) {
             const size_t drow = static_cast<size_t>(t * 16 + i) * page_size;
             if (V16) {
-                va_[t].u = *reinterpret_cast<const uint4*>(vbase0 + drow);
+                va_[t].u = load_streamed(vbase0 + drow);
             } else {
-                va_[t].half[0] = *reinterpret_cast<const uint2*>(vbase0 + drow);
-                va_[t].half[1] = *reinterpret_cast<const uint2*>(vbase1 + drow);
+                va_[t].half[0] = load_streamed8(vbase0 + drow);
+                va_[t].half[1] = load_streamed8(vbase1 + drow);
             }
         }
         const bool edge = kbase < seg_lo || kbase + kKeysPerBlock > ctx;

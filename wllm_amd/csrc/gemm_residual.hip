@@ -39,7 +39,7 @@ gemm_residual_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, flo
     RFrag cw[U], cx[U];
     auto load_step = [&](int u, int at) {
         const bool ok = at < s1;
-        cw[u].u = ok ? *reinterpret_cast<const uint4*>(wp + static_cast<size_t>(at) * kStep) : make_uint4(0, 0, 0, 0);
+        cw[u].u = ok ? load_streamed(wp + static_cast<size_t>(at) * kStep) : make_uint4(0, 0, 0, 0);
         cx[u].u = ok && x_row ? *reinterpret_cast<const uint4*>(xp + static_cast<size_t>(at) * 32) : make_uint4(0, 0, 0, 0);
     };
 #pragma unroll

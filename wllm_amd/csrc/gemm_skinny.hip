@@ -133,7 +133,9 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* _
     auto load_step = [&](int u, int at) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
-            cur[nt][u].u = (live && at < steps) ? *reinterpret_cast<const uint4*>(wp[nt] + at * kStep) : make_uint4(0, 0, 0, 0);
+            cur[nt][u].u = (live && at < steps) ? (row_groups > 1 ? *reinterpret_cast<const uint4*>(wp[nt] + at * kStep)
+                                                                  : load_streamed(wp[nt] + at * kStep))
+                                                : make_uint4(0, 0, 0, 0);
     };
 #pragma unroll
     for (int u = 0; u < kBatch; ++u) load_step(u, u);
@@ -427,8 +429,8 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, NormOnLoad norm, const bf16
     Frag curg[kBatch], curu[kBatch];
     auto load_step = [&](int u, int at) {
         const bool ok = live && at < steps;
-        curg[u].u = ok ? *reinterpret_cast<const uint4*>(gp + at * kStep) : make_uint4(0, 0, 0, 0);
-        curu[u].u = ok ? *reinterpret_cast<const uint4*>(up + at * kStep) : make_uint4(0, 0, 0, 0);
+        curg[u].u = ok ? load_streamed(gp + at * kStep) : make_uint4(0, 0, 0, 0);
+        curu[u].u = ok ? load_streamed(up + at * kStep) : make_uint4(0, 0, 0, 0);
     };
 #pragma unroll
     for (int u = 0; u < kBatch; ++u) load_step(u, u);

@@ -132,8 +132,8 @@ qkv_rope_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, const fl
     QFrag cl[U], ch[U], cx[U][MT];
     auto load_step = [&](int u, int at) {
         const bool ok = at < s1;
-        cl[u].u = ok ? *reinterpret_cast<const uint4*>(lo + static_cast<size_t>(at) * kStep) : make_uint4(0, 0, 0, 0);
-        ch[u].u = ok ? *reinterpret_cast<const uint4*>(hi + static_cast<size_t>(at) * kStep) : make_uint4(0, 0, 0, 0);
+        cl[u].u = ok ? load_streamed(lo + static_cast<size_t>(at) * kStep) : make_uint4(0, 0, 0, 0);
+        ch[u].u = ok ? load_streamed(hi + static_cast<size_t>(at) * kStep) : make_uint4(0, 0, 0, 0);
 #pragma unroll
         for (int t = 0; t < MT; ++t)
             cx[u][t].u = ok && x_row[t] ? *reinterpret_cast<const uint4*>(xp[t] + static_cast<size_t>(at) * 32) : make_uint4(0, 0, 0, 0);
