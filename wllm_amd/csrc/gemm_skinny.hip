@@ -70,7 +70,7 @@ template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float4_t v) {
 // their own that read the same weights.  The workgroups of a tile's row groups get indices that are 8
 // apart, so they are dispatched one after the other to the same XCD (workgroup index modulo 8) and the
 // later ones find the weights in that XCD's L2 instead of asking HBM for them again.
-template <int MT, int NT, typename TO, bool TILED, int KB = 16 / NT, int CS = 0>
+template <int MT, int NT, typename TO, bool TILED>
 __global__ void __launch_bounds__(256)
 gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* __restrict__ out,
                    float* __restrict__ partial, int M, int N, int K, int k_per_split, int chunk, int row_groups, int splits) {
@@ -126,7 +126,7 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* _
     // The weight stream: kBatch 16-byte loads per lane and tile are in flight, the first before x is
     // staged at all; a register is refilled with the step kBatch further on as soon as its products
     // have been issued.
-    constexpr int kBatch = KB;
+    constexpr int kBatch = 16 / NT;
     const bool live = n0 < N;
     const int steps = (k_end - k_begin) / 32;
     Frag cur[NT][kBatch];
@@ -170,41 +170,7 @@ gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, TO* _
     };
     fetch_x(k_begin);
     int step = 0;
-    if constexpr (CS > 0) {
-        // chunk == 32 * CS and the weights' loads run KB / CS chunks of x ahead: a register's step is
-        // fixed by its place among the KB steps, so the chunks of a batch are unrolled
-        for (int kb = k_begin; kb < k_end; kb += 32 * KB) {
-#pragma unroll
-            for (int sc = 0; sc < KB / CS; ++sc) {
-                const int kc = kb + sc * 32 * CS;
-                if (kc >= k_end) break;
-                const int len = min(32 * CS, k_end - kc);
-                const int vecs = len / 8;
-                __syncthreads();
-#pragma unroll
-                for (int u = 0; u < kXRegs; ++u)
-                    if (x_row[u] >= 0 && x_col[u] < vecs) xs[x_row[u] * stride + x_col[u]] = xreg[u];
-                __syncthreads();
-                if (kc + 32 * CS < k_end) fetch_x(kc + 32 * CS);
-#pragma unroll
-                for (int u = 0; u < CS; ++u) {
-                    if (32 * u < len) {
-                        Frag b[MT];
-#pragma unroll
-                        for (int t = 0; t < MT; ++t) b[t].u = xs[(t * 16 + i) * stride + 4 * u + g];
-#pragma unroll
-                        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                            for (int t = 0; t < MT; ++t)
-                                acc[nt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[nt][sc * CS + u].v, b[t].v, acc[nt][t], 0, 0, 0);
-                        load_step(sc * CS + u, step + sc * CS + u + KB);
-                    }
-                }
-            }
-            step += KB;
-        }
-    }
-    for (int kc = k_begin; CS == 0 && kc < k_end; kc += chunk) {
+    for (int kc = k_begin; kc < k_end; kc += chunk) {
         const int len = min(chunk, k_end - kc);   // a multiple of 32 * kBatch, except the last
         const int vecs = len / 8;
         __syncthreads();
@@ -392,8 +358,8 @@ struct NormOnLoad {
     float eps, offset;
 };
 
-template <int MT, int ACT, bool TILED, int TPW, bool NORM, int XR, int KB = 8>
-__global__ void __launch_bounds__(TPW * 128, KB > 8 ? 1 : (MT == 1 ? (NORM && XR > 2 ? 3 : 4) : (MT == 2 ? 3 : 2)))
+template <int MT, int ACT, bool TILED, int TPW, bool NORM, int XR>
+__global__ void __launch_bounds__(TPW * 128, MT == 1 ? (NORM && XR > 2 ? 3 : 4) : (MT == 2 ? 3 : 2))
 gemm_skinny_gated_kernel(const bf16* __restrict__ x, NormOnLoad norm, const bf16* __restrict__ w, bf16* __restrict__ out,
                          int M, int inter, int K, int chunk) {
     extern __shared__ uint4 xs[];                 // two halves of [MT*16][chunk/8 + 1]
@@ -423,7 +389,7 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, NormOnLoad norm, const bf16
     // The weight stream: kBatch 16-byte loads per lane and stream are in flight; a register is
     // refilled with the step kBatch further on as soon as its product has been issued, so the loads
     // in flight take 16 registers a stream and not twice that, and two workgroups fit a compute unit.
-    constexpr int kBatch = KB;      // per stream; two streams
+    constexpr int kBatch = 8;       // per stream; two streams
     const bool live = n0 < inter;
     const int steps = half_k / 32;
     Frag curg[kBatch], curu[kBatch];
@@ -521,36 +487,7 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, NormOnLoad norm, const bf16
             if (x_row[u] >= 0 && x_col[u] < vecs) xh[x_row[u] * stride + x_col[u]] = xreg[u];
     };
     fetch_x(0);
-    if constexpr (KB > 8) {
-        // chunks of 256 keys (8 steps), the weights' loads KB / 8 chunks ahead
-        for (int kb = 0; kb < half_k; kb += 32 * KB) {
-#pragma unroll
-            for (int sc = 0; sc < KB / 8; ++sc) {
-                const int kc = kb + sc * 256;
-                if (kc >= half_k) break;
-                const int len = min(256, half_k - kc);
-                __syncthreads();
-                stage_x(len / 8);
-                __syncthreads();
-                if (kc + 256 < half_k) fetch_x(kc + 256);
-#pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    if (32 * u < len) {
-#pragma unroll
-                        for (int t = 0; t < MT; ++t) {
-                            Frag b;
-                            b.u = xh[(t * 16 + i) * stride + 4 * u + g];
-                            accg[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(curg[sc * 8 + u].v, b.v, accg[t], 0, 0, 0);
-                            accu[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(curu[sc * 8 + u].v, b.v, accu[t], 0, 0, 0);
-                        }
-                        load_step(sc * 8 + u, step + sc * 8 + u + KB);
-                    }
-                }
-            }
-            step += KB;
-        }
-    }
-    for (int kc = 0; KB == 8 && kc < half_k; kc += chunk) {
+    for (int kc = 0; kc < half_k; kc += chunk) {
         const int len = min(chunk, half_k - kc);      // a multiple of 32 * kBatch, except the last
         __syncthreads();
         stage_x(len / 8);
@@ -626,16 +563,16 @@ static int gated_launch(const void* x, NormOnLoad norm, bool with_norm, const vo
     if (smem > 160 * 1024 - 4096 || mt * 16 * (chunk / 8) > tpw * 64 * x_regs || (chunk % 256 != 0 && chunk < K / 2))
         return -1;
     const dim3 grid((inter + 16 * tpw - 1) / (16 * tpw));
-#define LAUNCH_K(MT, A, T, TPW, NORM, XR, ...)                                                                            \
+#define LAUNCH_K(MT, A, T, TPW, NORM, XR)                                                                            \
     do {                                                                                                              \
         static bool roomy = false;     /* more than 64 KiB of shared memory must be asked for once */                \
         if (smem > 65536 && !roomy) {                                                                                 \
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_gated_kernel<MT, A, T, TPW, NORM, XR, ##__VA_ARGS__>), \
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_skinny_gated_kernel<MT, A, T, TPW, NORM, XR>), \
                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 4096) != hipSuccess)    \
                 return launch_status();                                                                               \
             roomy = true;                                                                                             \
         }                                                                                                             \
-        gemm_skinny_gated_kernel<MT, A, T, TPW, NORM, XR, ##__VA_ARGS__><<<grid, TPW * 128, smem, stream>>>(                        \
+        gemm_skinny_gated_kernel<MT, A, T, TPW, NORM, XR><<<grid, TPW * 128, smem, stream>>>(                        \
             static_cast<const bf16*>(x), norm, static_cast<const bf16*>(w), static_cast<bf16*>(out), M, inter, K, chunk); \
     } while (0)
 #define LAUNCH_T(MT, A, T, TPW) LAUNCH_K(MT, A, T, TPW, false, 4)
@@ -657,10 +594,6 @@ static int gated_launch(const void* x, NormOnLoad norm, bool with_norm, const vo
         case 3: LAUNCH(3, A); break; \
         default: LAUNCH(4, A); break; \
     }
-    static const int x_kb = getenv("WLLM_X_GATED_KB") ? atoi(getenv("WLLM_X_GATED_KB")) : 0;     // EXPERIMENT
-    if (x_kb && !with_norm && mt == 4 && tiled && activation == 0 && chunk == 256) {
-        LAUNCH_K(4, 0, true, 4, false, 4, 16);
-    } else
     if (with_norm) {
         if (activation == 0) { LAUNCH_N(0) } else { LAUNCH_N(1) }
     } else {
