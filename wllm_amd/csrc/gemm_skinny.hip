@@ -339,9 +339,12 @@ __device__ __forceinline__ float act_gelu_tanh(float z) {
 __device__ __forceinline__ float act_silu(float z) { return z / (1.f + expf(-z)); }
 
 // A workgroup is TPW tiles of 16 gate rows (with their up rows) times 2 halves of the K axis; the
-// halves are added through shared memory in a fixed order before the activation.  With few rows of
-// x (MT <= 2) the kernel needs few registers, a workgroup is 2 tiles (4 wavefronts), and four
-// workgroups share a compute unit: 16 wavefronts with 16 loads each in flight.
+// halves are added through shared memory in a fixed order before the activation.  A workgroup is 2
+// tiles (4 wavefronts); with few rows of x (MT <= 2) the kernel needs few registers and four
+// workgroups share a compute unit, 16 wavefronts with 16 loads each in flight, with three or four
+// tiles of rows two workgroups do.  (Workgroups of 4 tiles, which stage x half as often, are slower
+// at 48 and 64 rows, 34 against 30 and 38 against 35 us at the 2B sizes: a barrier then holds eight
+// wavefronts to the slowest one's loads.)
 //
 // NORM (at most 16 rows, chunks of 256 keys): x is not given; the kernel reads the float32 residual
 // stream and applies the RMS norm as it stages a chunk: x = residual * rsqrt(mean square + eps) *
@@ -419,7 +422,7 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, NormOnLoad norm, const bf16
         }
     }
     // x is staged chunk by chunk (per half of K); the next chunk's loads are in flight during the products
-    constexpr int kXRegs = NORM ? XR : (MT == 1 ? 4 : 8);       // pieces of a chunk per thread
+    constexpr int kXRegs = NORM ? XR : (MT == 1 ? 4 : (MT >= 3 && TPW == 2 ? 16 : 8));       // pieces of a chunk per thread
     uint4 xreg[NORM ? 1 : kXRegs];
     float4 xraw[NORM ? kXRegs : 1][2], wraw[2];
     // a thread's pieces of a chunk as (row, 8 keys) pairs of the whole chunk's shape, worked out once: a
@@ -553,13 +556,13 @@ static int gated_launch(const void* x, NormOnLoad norm, bool with_norm, const vo
     if (chunk > K / 2) chunk = K / 2;
     // the norm on load: at most 16 rows, whole chunks of 256 keys
     if (with_norm && (mt != 1 || chunk != 256 || (K / 2) % 256 != 0)) return -1;
-    const int tpw = mt <= 2 ? 2 : 4;                 // tiles of 16 gate rows per workgroup
+    const int tpw = 2;                               // tiles of 16 gate rows per workgroup
     size_t smem = static_cast<size_t>(2) * mt * 16 * (chunk / 8 + 1) * sizeof(uint4);
     const size_t red = static_cast<size_t>(tpw) * kWave * mt * 8 * sizeof(float);
     if (red > smem) smem = red;
     // the pieces of x a thread stages (4 up to 16 rows, else 8); a chunk that is not the last must be
     // whole batches of 8 steps, because a register's step is fixed by its place
-    const int x_regs = mt == 1 ? 4 : 8;
+    const int x_regs = mt == 1 ? 4 : (mt >= 3 && tpw == 2 ? 16 : 8);
     if (smem > 160 * 1024 - 4096 || mt * 16 * (chunk / 8) > tpw * 64 * x_regs || (chunk % 256 != 0 && chunk < K / 2))
         return -1;
     const dim3 grid((inter + 16 * tpw - 1) / (16 * tpw));
@@ -576,9 +579,9 @@ static int gated_launch(const void* x, NormOnLoad norm, bool with_norm, const vo
             static_cast<const bf16*>(x), norm, static_cast<const bf16*>(w), static_cast<bf16*>(out), M, inter, K, chunk); \
     } while (0)
 #define LAUNCH_T(MT, A, T, TPW) LAUNCH_K(MT, A, T, TPW, false, 4)
-#define LAUNCH(MT, A)                                        \
-    if (tiled) LAUNCH_T(MT, A, true, (MT <= 2 ? 2 : 4));      \
-    else LAUNCH_T(MT, A, false, (MT <= 2 ? 2 : 4))
+#define LAUNCH(MT, A)                        \
+    if (tiled) LAUNCH_T(MT, A, true, 2);      \
+    else LAUNCH_T(MT, A, false, 2)
 #define LAUNCH_N(A)                                           \
     if (tiled) {                                              \
         if (M <= 8) LAUNCH_K(1, A, true, 2, true, 2);         \
