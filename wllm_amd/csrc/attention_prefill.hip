@@ -321,7 +321,10 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
 }
 
 // ---- the same kernel with the tiles moved into shared memory by the memory pipeline itself -------
-// For head sizes 64, 128 and 256 and pages of a multiple of 8 keys.  A lane's 16-byte load goes
+// For head sizes 64, 128 and 256 and pages of 8, 16, 32, ... keys (a power of two, so that a key's
+// place is a shift and a mask and most of a load's address is fixed for a lane: with divisions and a
+// table look-up per load the address arithmetic was a third of the kernel's time; other page sizes
+// take the kernel above).  A lane's 16-byte load goes
 // straight to shared memory (lane l of a wavefront to base + 16 l), so staging costs no registers,
 // no writes to shared memory and no second barrier; two tiles of keys and values are held, and
 // the loads of block b+1 run while block b is multiplied.  Since a lane chooses its address, the
@@ -348,6 +351,17 @@ __device__ __forceinline__ void load_to_shared(const void* src, void* dst) {
     uint32_t saved_m0;
     asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
                  : "=&s"(saved_m0) : "v"(src), "s"(lds_address) : "memory");
+}
+
+// The same with the destination as a shared-memory address that is the same in all lanes (a scalar).
+__device__ __forceinline__ void load_to_shared_at(const void* src, uint32_t lds_address) {
+    uint32_t saved_m0;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
+                 : "=&s"(saved_m0) : "v"(src), "s"(__builtin_amdgcn_readfirstlane(lds_address)) : "memory");
+}
+__device__ __forceinline__ uint32_t shared_address(const void* p) {
+    return __builtin_amdgcn_readfirstlane(
+        static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const void*)p)));
 }
 
 template <int HD>
@@ -429,64 +443,76 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
 #pragma unroll
     for (int t = 0; t < DT; ++t) acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-    const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
-    auto page_of = [&](int key, int& slot) -> int {
-        if (page_shift >= 0) {
-            slot = key & (page_size - 1);
-            return table_s[(key >> page_shift) - page_base];
-        }
-        slot = key % page_size;
-        return table_s[key / page_size - page_base];
-    };
-    // this lane's part of the loads of one block.  Keys: wavefront load q of the tile carries the chunks
-    // 64 q .. 64 q + 63 of the tile in shared-memory order; values likewise.
-    int k_row[(kKeyInstr + kPrefillWaves - 1) / kPrefillWaves], k_chunk[(kKeyInstr + kPrefillWaves - 1) / kPrefillWaves];
+    // ---- the loads of a block.  The page size is a power of two here and a block begins at a multiple
+    //      of 32 keys, so the place of a lane's key kbase + rel splits into a part all lanes share and the
+    //      lane's own, which is worked out once: page (kbase >> shift) + (rel >> shift) of the request,
+    //      slot (kbase & mask) + (rel & mask).  Per block and load that leaves one look-up in the table
+    //      and one multiply-add for the address.  A page index beyond the request's last page (the keys
+    //      after the end of the last block) is clamped: whatever lies there is masked and cleared. ----
+    const int shift = __builtin_ctz(page_size), mask = page_size - 1;
+    static_assert(kKeyInstr % kPrefillWaves == 0 && kValInstr % kPrefillWaves == 0, "whole loads per wavefront");
+    constexpr int KU = kKeyInstr / kPrefillWaves, VU = kValInstr / kPrefillWaves;
+    const uint32_t page_bytes = static_cast<uint32_t>(page_elems * 2);
+    // keys: wavefront load q = wave + 4 u of the tile carries the chunks 64 q .. 64 q + 63 of the tile in
+    // shared-memory order
+    int k_page[KU];
+    const char* k_src[KU];
 #pragma unroll
-    for (int u = 0; u < (kKeyInstr + kPrefillWaves - 1) / kPrefillWaves; ++u) {
+    for (int u = 0; u < KU; ++u) {
         const int chunk_index = (wave + u * kPrefillWaves) * 64 + lane;       // position in the tile, in chunks
         const int r = chunk_index / CPR;                                      // row of the tile
-        k_chunk[u] = (chunk_index % CPR) ^ (r % 8);                           // the chunk of the key's row that lies there
-        k_row[u] = 8 * ((r % 16) / 4) + 4 * (r / 16) + r % 4;                 // the key of the block that row r holds
+        const int chunk = (chunk_index % CPR) ^ (r % 8);                      // the chunk of the key's row that lies there
+        const int rel = 8 * ((r % 16) / 4) + 4 * (r / 16) + r % 4;            // the key of the block that row r holds
+        k_page[u] = rel >> shift;
+        k_src[u] = reinterpret_cast<const char*>(cache + k_off + static_cast<size_t>(rel & mask) * HD + chunk * 8);
     }
-    const int v_q = (lane % 4) ^ ((lane / 8) % 4);                            // the chunk of 8 keys this lane moves, in every load
-    auto issue = [&](uint16_t* k_dst, uint16_t* v_dst, int kbase) {
+    // values: a lane moves the same chunk of 8 keys in every load, of the rows d = 16 q + lane / 4
+    const int v_rel = 8 * ((lane % 4) ^ ((lane / 8) % 4));
+    const int v_page = v_rel >> shift;
+    const char* v_src[VU];
 #pragma unroll
-        for (int u = 0; u < (kKeyInstr + kPrefillWaves - 1) / kPrefillWaves; ++u) {
-            const int q = wave + u * kPrefillWaves;
-            if (q < kKeyInstr) {
-                const int key = min(kbase + k_row[u], ctx - 1);
-                int slot;
-                const int page = page_of(key, slot);
-                const bf16* src = cache + static_cast<size_t>(page) * page_elems + k_off + static_cast<size_t>(slot) * HD + k_chunk[u] * 8;
-                load_to_shared(src, k_dst + q * 512);
-            }
-        }
-        {
-            const int key = min(kbase + 8 * v_q, (ctx - 1) & ~7);
-            int slot;
-            const int page = page_of(key, slot);
-            const bf16* src0 = cache + static_cast<size_t>(page) * page_elems + v_off + slot;
+    for (int u = 0; u < VU; ++u) {
+        const int d = (wave + u * kPrefillWaves) * 16 + lane / 4;
+        v_src[u] = reinterpret_cast<const char*>(cache + v_off + static_cast<size_t>(d) * page_size + (v_rel & mask));
+    }
+    const int table_last = blk_first < blk_end
+                               ? min(min(max_pages - 1, (min(blk_end * kBlockKeys, ctx) - 1) / page_size) - page_base + 1,
+                                     kMaxTablePages) - 1
+                               : 0;
+    // where this wavefront's loads land: tile + 1 KiB * (wave + 4 u)
+    const uint32_t k_lds[2] = {shared_address(k_s0) + wave * 1024u, shared_address(k_s1) + wave * 1024u};
+    const uint32_t v_lds[2] = {shared_address(v_s0) + wave * 1024u, shared_address(v_s1) + wave * 1024u};
+    auto issue = [&](int which, int kbase) {
+        const int pb = (kbase >> shift) - page_base;
+        const uint32_t k_slot_bytes = static_cast<uint32_t>(kbase & mask) * HD * 2, v_slot_bytes = static_cast<uint32_t>(kbase & mask) * 2;
+        int kp[KU];
 #pragma unroll
-            for (int u = 0; u < (kValInstr + kPrefillWaves - 1) / kPrefillWaves; ++u) {
-                const int q = wave + u * kPrefillWaves;
-                if (q < kValInstr) {
-                    const int d = q * 16 + lane / 4;
-                    load_to_shared(src0 + static_cast<size_t>(d) * page_size, v_dst + q * 512);
-                }
-            }
-        }
+        for (int u = 0; u < KU; ++u) kp[u] = table_s[min(pb + k_page[u], table_last)];
+        const int vp = table_s[min(pb + v_page, table_last)];
+#pragma unroll
+        for (int u = 0; u < KU; ++u)
+            load_to_shared_at(k_src[u] + (static_cast<uint64_t>(static_cast<uint32_t>(kp[u])) * page_bytes + k_slot_bytes),
+                              k_lds[which] + u * (kPrefillWaves * 1024u));
+        const uint64_t v_page_bytes = static_cast<uint64_t>(static_cast<uint32_t>(vp)) * page_bytes + v_slot_bytes;
+#pragma unroll
+        for (int u = 0; u < VU; ++u) load_to_shared_at(v_src[u] + v_page_bytes, v_lds[which] + u * (kPrefillWaves * 1024u));
     };
 
     __syncthreads();      // the block table is in shared memory
-    if (blk_first < blk_end) issue(k_s0, v_s0, blk_first * kBlockKeys);
+    if (blk_first < blk_end) issue(0, blk_first * kBlockKeys);
     // One block: its tiles are k_s and v_s, the next block's loads go to k_next and v_next.  The loop below
     // names the two pairs of tiles in turn, so every address in shared memory is a constant plus a lane's
     // fixed offset.
-    auto block = [&](int blk, const uint16_t* k_s, uint16_t* v_s, uint16_t* k_next, uint16_t* v_next) {
+    // a lane's fragment reads: every address is the tile, the lane's offset and a constant.  Chunk (4 c + g)
+    // ^ (i % 8) of a key row is 4 (c ^ bit 2 of i) + (g ^ (i % 4)): an offset for even c and one for odd c.
+    const int k_lane_even = (i * CPR + 4 * ((i >> 2) & 1) + (g ^ (i & 3))) * 8;
+    const int k_lane_odd = (i * CPR + 4 * (1 - ((i >> 2) & 1)) + (g ^ (i & 3))) * 8;
+    const int v_lane = (i * 4 + (g ^ ((i / 2) % 4))) * 8;
+    auto block = [&](int blk, const uint16_t* k_s, uint16_t* v_s, int next) {
         const int kbase = blk * kBlockKeys;
         __builtin_amdgcn_s_waitcnt(0);   // this lane's loads of the block have landed
         __syncthreads();                 // everyone's have, and everyone is done with the block before
-        if (blk + 1 < blk_end) issue(k_next, v_next, kbase + kBlockKeys);
+        if (blk + 1 < blk_end) issue(next, kbase + kBlockKeys);
         if (kbase + kBlockKeys > ctx || kbase < seg_lo) {
             // a block at the edge of the request: the values of keys that are not the request's are cleared
             if (tid < HD) {
@@ -506,7 +532,7 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
 #pragma unroll
             for (int c = 0; c < DC; ++c) {
                 PPack a;
-                a.u = *reinterpret_cast<const uint4*>(&k_s[((16 * t2 + i) * CPR + ((4 * c + g) ^ (i % 8))) * 8]);
+                a.u = *reinterpret_cast<const uint4*>(&k_s[((c & 1) ? k_lane_odd : k_lane_even) + (16 * t2 * CPR + 4 * (c & ~1)) * 8]);
                 sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qreg[c], sc, 0, 0, 0);
             }
 #pragma unroll
@@ -548,13 +574,13 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
 #pragma unroll
         for (int t = 0; t < DT; ++t) {
             PPack a;
-            a.u = *reinterpret_cast<const uint4*>(&v_s[((16 * t + i) * 4 + (g ^ ((i / 2) % 4))) * 8]);
+            a.u = *reinterpret_cast<const uint4*>(&v_s[v_lane + 16 * t * 4 * 8]);
             acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pv.v, acc[t], 0, 0, 0);
         }
     };
     for (int blk = blk_first; blk < blk_end; blk += 2) {
-        block(blk, k_s0, v_s0, k_s1, v_s1);
-        if (blk + 1 < blk_end) block(blk + 1, k_s1, v_s1, k_s0, v_s0);
+        block(blk, k_s0, v_s0, 1);
+        if (blk + 1 < blk_end) block(blk + 1, k_s1, v_s1, 0);
     }
     float l = l_run;
     l += __shfl_xor(l, 16, kWave);
@@ -592,7 +618,7 @@ WLLM_API int wllm_paged_attention_prefill(const void* qkv, const void* cache, co
     if (rows_per_item != 64) return -1;
     if (num_items <= 0) return 0;
     const float scale_log2e = scale * 1.4426950408889634f;
-    if (page_size % 8 == 0 && (head_dim == 64 || head_dim == 128 || head_dim == 256)) {
+    if (page_size >= 8 && (page_size & (page_size - 1)) == 0 && (head_dim == 64 || head_dim == 128 || head_dim == 256)) {
 #define LAUNCH_DMA(HD)                                                                                              \
     paged_attention_prefill_dma_kernel<HD><<<num_items, kPrefillThreads, 0, stream>>>(                              \
         static_cast<const bf16*>(qkv), static_cast<const bf16*>(cache), block_tables, items, seg_q_start, seg_q_len, \

@@ -444,26 +444,29 @@ __global__ void gated_activation_kernel(const T* __restrict__ gate_up, T* __rest
     }
 }
 
-// bfloat16 rows whose halves are multiples of 8: eight values per 16-byte load
+// bfloat16 rows whose halves are multiples of 8: eight values per 16-byte load; a workgroup walks one
+// row (blockIdx.y and on), so no thread divides, and the product of the matrix kernel before it is
+// read once
 template <int ACT>
-__global__ void gated_activation_bf16x8_kernel(const bf16* __restrict__ gate_up, bf16* __restrict__ out,
-                                               long long total_vecs, int inter) {
+__global__ void __launch_bounds__(256)
+gated_activation_bf16x8_kernel(const bf16* __restrict__ gate_up, bf16* __restrict__ out, int rows, int inter) {
     const int vecs = inter / 8;
-    const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
-    for (long long i = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x; i < total_vecs; i += stride) {
-        const long long r = i / vecs;
-        const int c = static_cast<int>(i % vecs) * 8;
-        const uint4 g4 = *reinterpret_cast<const uint4*>(gate_up + r * 2 * inter + c);
-        const uint4 u4 = *reinterpret_cast<const uint4*>(gate_up + r * 2 * inter + inter + c);
-        const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
-        uint32_t ow[4];
+    for (int r = blockIdx.y; r < rows; r += gridDim.y) {
+        const bf16* src = gate_up + static_cast<size_t>(r) * 2 * inter;
+        bf16* dst = out + static_cast<size_t>(r) * inter;
+        for (int v = blockIdx.x * 256 + threadIdx.x; v < vecs; v += gridDim.x * 256) {
+            const uint4 g4 = load_streamed(src + v * 8);
+            const uint4 u4 = load_streamed(src + inter + v * 8);
+            const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
+            uint32_t ow[4];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const float g0 = __uint_as_float(gw[k] << 16), g1 = __uint_as_float(gw[k] & 0xffff0000u);
-            const float u0 = __uint_as_float(uw[k] << 16), u1 = __uint_as_float(uw[k] & 0xffff0000u);
-            ow[k] = pack2_bf16((ACT == 0 ? gelu_tanh(g0) : silu(g0)) * u0, (ACT == 0 ? gelu_tanh(g1) : silu(g1)) * u1);
+            for (int k = 0; k < 4; ++k) {
+                const float g0 = __uint_as_float(gw[k] << 16), g1 = __uint_as_float(gw[k] & 0xffff0000u);
+                const float u0 = __uint_as_float(uw[k] << 16), u1 = __uint_as_float(uw[k] & 0xffff0000u);
+                ow[k] = pack2_bf16((ACT == 0 ? gelu_tanh(g0) : silu(g0)) * u0, (ACT == 0 ? gelu_tanh(g1) : silu(g1)) * u1);
+            }
+            *reinterpret_cast<uint4*>(dst + v * 8) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
         }
-        *reinterpret_cast<uint4*>(out + r * inter + c) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
     }
 }
 
@@ -471,15 +474,14 @@ WLLM_API int wllm_gated_activation(const void* gate_up, void* out, int is_bf16, 
                                    hipStream_t stream) {
     const long long total = static_cast<long long>(n) * inter;
     if (is_bf16 && inter % 8 == 0) {
-        const long long total_vecs = total / 8;
-        long long vblocks = (total_vecs + 255) / 256;
-        if (vblocks > 65536) vblocks = 65536;
+        const int vecs = inter / 8;
+        const dim3 grid(vecs < 2048 ? (vecs + 255) / 256 : 8, n < 16384 ? n : 16384);
         if (activation == 0)
-            gated_activation_bf16x8_kernel<0><<<static_cast<int>(vblocks), 256, 0, stream>>>(
-                static_cast<const bf16*>(gate_up), static_cast<bf16*>(out), total_vecs, inter);
+            gated_activation_bf16x8_kernel<0><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(gate_up),
+                                                                        static_cast<bf16*>(out), n, inter);
         else
-            gated_activation_bf16x8_kernel<1><<<static_cast<int>(vblocks), 256, 0, stream>>>(
-                static_cast<const bf16*>(gate_up), static_cast<bf16*>(out), total_vecs, inter);
+            gated_activation_bf16x8_kernel<1><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(gate_up),
+                                                                        static_cast<bf16*>(out), n, inter);
         return launch_status();
     }
     long long blocks = (total + 255) / 256;
