@@ -216,8 +216,7 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
             sv[e] = s[t2][v];
             if (ok[e]) tile_max = fmaxf(tile_max, sv[e]);
         }
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
+        tile_max = max_across(max_across(tile_max, 16), 32);
         m_run = tile_max;
         const float mc = (tile_max == -INFINITY ? 0.f : tile_max) * scale_log2e;
         Pack16 pv;
@@ -230,8 +229,7 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
         pv.u = make_uint4(pack2_bf16(pe[0], pe[1]), pack2_bf16(pe[2], pe[3]), pack2_bf16(pe[4], pe[5]),
                           pack2_bf16(pe[6], pe[7]));
         // the row's sum over its four lanes
-        l_run += __shfl_xor(l_run, 16, kWave);
-        l_run += __shfl_xor(l_run, 32, kWave);
+        l_run = sum_across(sum_across(l_run, 16), 32);
         // ---- out^T = V^T . P^T ----
 #pragma unroll
         for (int t = 0; t < DT; ++t) {

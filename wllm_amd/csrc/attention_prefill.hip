@@ -256,8 +256,7 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
             }
             float tile_max = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
                                    fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
+            tile_max = max_across(max_across(tile_max, 16), 32);
             const float m_new = fmaxf(m_run[rt], tile_max);
             const float m_use = m_new == -INFINITY ? 0.f : m_new;
             const float mc = m_use * scale_log2e;
@@ -294,8 +293,7 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
 #pragma unroll
     for (int rt = 0; rt < RTW; ++rt) {
         float l = l_run[rt];
-        l += __shfl_xor(l, 16, kWave);
-        l += __shfl_xor(l, 32, kWave);
+        l = sum_across(sum_across(l, 16), 32);
         if (!row_valid[rt]) continue;
         if (partial_slot >= 0) {
             // one slot per tile of 16 rows: [16][HD] accumulators and [16][2] (maximum, sum)
@@ -548,8 +546,7 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
             }
         }
         float tile_max = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
+        tile_max = max_across(max_across(tile_max, 16), 32);
         const float m_new = fmaxf(m_run, tile_max);
         const float m_use = m_new == -INFINITY ? 0.f : m_new;
         const float mc = m_use * scale_log2e;
@@ -583,8 +580,7 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
         if (blk + 1 < blk_end) block(blk + 1, k_s1, v_s1, 0);
     }
     float l = l_run;
-    l += __shfl_xor(l, 16, kWave);
-    l += __shfl_xor(l, 32, kWave);
+    l = sum_across(sum_across(l, 16), 32);
     if (!row_valid) return;
     if (partial_slot >= 0) {
         const size_t slot = static_cast<size_t>(partial_slot) + wave;

@@ -33,15 +33,56 @@ __device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
     return *reinterpret_cast<const uint32_t*>(&r);
 }
 
+// The sum (maximum) of a lane's value and that of the lane 16 (32) further on or back, as `v op
+// __shfl_xor(v, 16)` gives it, bit for bit, but with one swap instruction of the vector unit (gfx950's
+// v_permlane16_swap / v_permlane32_swap) where a shuffle takes a trip through the LDS pipeline.
+__device__ __forceinline__ void swap_halves(float v, int distance, float& a, float& b) {
+    typedef unsigned uint2_t __attribute__((ext_vector_type(2)));
+    const uint2_t r = distance == 16 ? __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false)
+                                     : __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    a = __uint_as_float(r.x);
+    b = __uint_as_float(r.y);
+}
+__device__ __forceinline__ float sum_across(float v, int distance) {
+    float a, b;
+    swap_halves(v, distance, a, b);
+    return a + b;
+}
+__device__ __forceinline__ float max_across(float v, int distance) {
+    float a, b;
+    swap_halves(v, distance, a, b);
+    return fmaxf(a, b);
+}
+
+// The value of another lane of the same row of 16 through the vector unit's own lane permutation
+// (no trip through the LDS pipeline).  kCtrl: 0xB1 and 0x4E exchange the lanes 1 and 2 apart, 0x124 and
+// 0x128 turn a row by 4 and by 8 lanes; a turn by 8 is the lane 8 apart, and a turn by 4 is the lane 4
+// apart for values that are already the same 8 lanes apart, as they are in the butterflies below.
+template <int kCtrl>
+__device__ __forceinline__ float row_permuted(float v) {
+    return __uint_as_float(static_cast<uint32_t>(
+        __builtin_amdgcn_update_dpp(0, static_cast<int>(__float_as_uint(v)), kCtrl, 0xf, 0xf, false)));
+}
+
+// Butterflies over the 64 lanes, from the lanes 32 apart down to neighbours: the operands and their
+// order are those of `v op __shfl_xor(v, off)` for off = 32 .. 1, so the results have the same bits.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    v = sum_across(v, 32);
+    v = sum_across(v, 16);
+    v += row_permuted<0x128>(v);
+    v += row_permuted<0x124>(v);
+    v += row_permuted<0x4E>(v);
+    v += row_permuted<0xB1>(v);
     return v;
 }
 
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    v = max_across(v, 32);
+    v = max_across(v, 16);
+    v = fmaxf(v, row_permuted<0x128>(v));
+    v = fmaxf(v, row_permuted<0x124>(v));
+    v = fmaxf(v, row_permuted<0x4E>(v));
+    v = fmaxf(v, row_permuted<0xB1>(v));
     return v;
 }
 

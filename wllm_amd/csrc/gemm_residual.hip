@@ -72,8 +72,7 @@ gemm_residual_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, flo
         sq = now[0] * now[0] + now[1] * now[1] + now[2] * now[2] + now[3] * now[3];
     }
     // the band's 16 columns of a row lie in the four lanes i, i + 16, i + 32, i + 48
-    sq += __shfl_xor(sq, 16, kWave);
-    sq += __shfl_xor(sq, 32, kWave);
+    sq = sum_across(sum_across(sq, 16), 32);
     if (x_row && g == 0) sumsq[static_cast<size_t>(i) * bands + band] = sq;
 }
 

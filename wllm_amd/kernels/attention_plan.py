@@ -175,7 +175,8 @@ def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_
             # whose boundaries are multiples of 32 counted from the block's first group of 32
             lo32 = lo // 32 * 32
             span = hi - lo32
-            ns = np.maximum(np.maximum(1, (span + chunk // 2) // chunk), -(-span // max_chunk))   # items per block
+            # no piece longer than `chunk`: the longest piece is what the last workgroups wait for
+            ns = np.maximum(np.maximum(1, -(-span // chunk)), -(-span // max_chunk))   # items per block
             piece = -(-span // (ns * 32)) * 32
             ns = -(-span // piece)
             n_items = int(ns.sum())
