@@ -18,9 +18,11 @@ def covered(q_len, ctx_len, group, nkv, window, page_size):
         assert slot not in slot_users, f"slot {slot} held by {slot_users[slot]} and {who}"
         slot_users[slot] = who
     for n, it in enumerate(items):
-        seg, kvh, row0, _, kb, ke, slot, _ = (int(v) for v in it)
+        seg, kvh, new_tokens, first_token, kb, ke, slot, context = (int(v) for v in it)
         rows = q_len[seg] * group
-        assert rows <= 16 and row0 == 0
+        assert rows <= 16
+        # the item carries the segment's lengths and the place of its first token in the step
+        assert new_tokens == q_len[seg] and context == ctx_len[seg] and first_token == sum(q_len[:seg])
         # the kernel gives each of its four wavefronts one block of 32 keys of an aligned group of 128
         assert kb < ke and kb // 128 == (ke - 1) // 128, (kb, ke)
         first_pos = ctx_len[seg] - q_len[seg]

@@ -82,16 +82,17 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
     // a captured graph launches as many workgroups as its plan has room for items; the live ones come first
     if (live_items != nullptr && static_cast<int>(blockIdx.x) >= live_items[0]) return;
     const int* item = items + static_cast<size_t>(blockIdx.x) * kItemInts;
-    const int seg = item[0], kvh = item[1], row_begin = item[2];
-    const int key_begin = item[4], key_end = item[5], partial_slot = item[6];
+    // the item brings the segment's lengths with it: no second trip to memory for them
+    const int seg = item[0], kvh = item[1], q_len = item[2], q_start = item[3];
+    const int key_begin = item[4], key_end = item[5], partial_slot = item[6], ctx = item[7];
+    constexpr int row_begin = 0;      // a short segment is one tile of rows
     if (seg < 0) return;    // padding item
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int i = lane % 16, g = lane / 16;
 
-    // ---- The request's lengths and this lane's queries are asked for first: they arrive while the
-    //      addresses of the keys and values are worked out. ----
-    const int q_start = seg_q_start[seg], q_len = seg_q_len[seg], ctx = seg_ctx_len[seg];
+    // ---- This lane's queries are asked for first: they arrive while the addresses of the keys and
+    //      values are worked out. ----
     const int group = num_heads / num_kv_heads;
     const int width = (num_heads + 2 * num_kv_heads) * HD;
     const int total_rows = q_len * group;

@@ -7,8 +7,10 @@ partial results combined by a second kernel; chunk boundaries are multiples of t
 counted from key 0, so they depend on the key index only.  Longer segments are cut into
 workgroups of four tiles of 16 rows (prefill items).
 
-A work item is 8 int32: segment, key/value head, first row, 1 (reserved), first key,
-end key, partial slot (-1: the workgroup writes the final result), unused.  A partial slot holds
+A work item is 8 int32: segment, key/value head, the segment's number of new tokens, the place of
+its first token among the step's tokens, first key, end key, partial slot (-1: the workgroup writes
+the final result), the segment's context length: what the kernel needs of the segment comes with
+the item, in the one read it begins with, and not from the segments' arrays in a second trip to memory.  A partial slot holds
 one tile of 16 rows.  A reduce item is 8 int32: segment, key/value head, first partial slot, number
 of splits, first row of the tile, slots between two splits, 2 unused.  A prefill item (long
 segments, 64 rows each, for the kernel that stages keys and values through shared memory) is
@@ -104,6 +106,7 @@ def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_
     q_len = np.asarray(q_len, dtype=np.int64)
     ctx_len = np.asarray(ctx_len, dtype=np.int64)
     rows = q_len * group
+    q_start = np.cumsum(q_len) - q_len
     short = rows <= ROWS_PER_TILE
     items, reduces = [], []
     slots = 0
@@ -130,10 +133,11 @@ def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_
         it = np.zeros((S, num_kv_heads, width, ITEM_INTS), dtype=np.int32)
         it[..., 0] = np.where(live, idx[:, None], -1)[:, None, :]
         it[..., 1] = kv[None, :, None]
-        it[..., 2] = 0
-        it[..., 3] = 1
+        it[..., 2] = q_len[idx][:, None, None]
+        it[..., 3] = q_start[idx][:, None, None]
         it[..., 4] = kb[:, None, :]
         it[..., 5] = ke[:, None, :]
+        it[..., 7] = ctx_len[idx][:, None, None]
         slot = seg_base[:, None, None] + kv[None, :, None] * n_split_seg[:, None, None] + j[None, None, :]
         it[..., 6] = np.where(single[:, None, None], -1, slot)
         keep = np.broadcast_to(live[:, None, :], (S, num_kv_heads, width))
