@@ -228,6 +228,10 @@ MFMA_SHAPES = ATTENTION_SHAPES + [
     (3, 1, 224, 16, [(1, 400), (6, 6), (7, 20)], 0),                               # group of 3: rows straddle tokens
     (4, 2, 64, 12, [(1, 300), (2, 77), (1, 5), (1, 128), (1, 129)], 0),            # pages that do not divide 128 keys
     (8, 2, 64, 20, [(1, 500), (3, 90), (1, 260)], 70),                             # the same with a window
+    (8, 2, 64, 24, [(40, 300), (1, 100)], 0),          # prompt portions with pages of a multiple of 8 that is no power of two
+    (4, 1, 128, 40, [(70, 70), (33, 200)], 60),
+    (8, 1, 256, 32, [(100, 1000)], 0),                 # ... and of a power of two other than 16
+    (4, 4, 128, 8, [(64, 64), (20, 500)], 100),
 ]
 
 
