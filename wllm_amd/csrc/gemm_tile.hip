@@ -11,8 +11,8 @@
 //
 // The K axis is walked in stages of 64 keys.  A stage's tiles of x and w (16 KB each) go from
 // memory straight into shared memory (global_load_lds_dwordx4: a wavefront's 64 lanes bring 8 rows
-// of 8 chunks of 16 bytes, lane l's chunk to base + 16 l), two stages in turn, the next one's loads
-// in flight during this one's products.  Chunk c of row r lies at place c ^ (r % 8) of its row, so
+// of 8 chunks of 16 bytes, lane l's chunk to base + 16 l), two stages in turn (four where a compute
+// unit has one workgroup), the next ones' loads in flight during this one's products.  Chunk c of row r lies at place c ^ (r % 8) of its row, so
 // that the 16 lanes of a fragment read meet 8 different places in each of two passes and no bank
 // twice.  A lane's eight source offsets never change; the stage's 128 bytes go into the scalar base.
 //
@@ -57,14 +57,20 @@ static __device__ __forceinline__ float tile_silu(float z) { return z / (1.f + e
 // GATED: 0 plain, 1 gelu_tanh, 2 silu.  N is the number of rows of w (plain) or of gate rows (gated).
 // (Tiles of 256 rows of x with eight wavefronts were no faster: the rate is set by the reads of
 // fragments from shared memory, which take as long as the products they feed.)
-template <int GATED>
-__global__ void __launch_bounds__(256, 2)
+// STAGES: how many stages' tiles shared memory holds.  Two, and two workgroups a compute unit, as
+// a rule; four, one workgroup a compute unit and three stages (96 KB) on their way, where the launch has
+// no more workgroups than the machine has compute units (a step of at most 128 rows, a down projection
+// of 256): the tiles of w then come from HBM, and the rate is set by how much a compute unit has in
+// flight (the gated product of 128 rows: 53 to 29 us).
+template <int GATED, int STAGES>
+__global__ void __launch_bounds__(256, STAGES == 2 ? 2 : 1)
 gemm_tile_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, bf16* __restrict__ out,
                  float* __restrict__ partial, int M, int N, int K, int m_tiles, int k_per_split) {
     constexpr int kXRows = kTileRows, kWaves = 4;
     constexpr int kWBytes = kTileRows * kRowBytes, kXBytes = kXRows * kRowBytes;
     constexpr int kLoads = (kTileRows + kXRows) / 8 / kWaves;      // loads a wavefront and stage: 8 rows each
-    __shared__ __align__(16) unsigned char tiles_s[2][kWBytes + kXBytes];      // [stage][w rows, x rows]
+    constexpr int kStageBytes = kWBytes + kXBytes;
+    extern __shared__ __align__(16) unsigned char tiles_s[];       // [STAGES][w rows, x rows]
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int i = lane % 16, g = lane / 16;
@@ -105,7 +111,7 @@ gemm_tile_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, bf16* _
 #pragma unroll
         for (int u = 0; u < kLoads; ++u) {
             const int q = wave + kWaves * u;        // the same for all lanes
-            load_to_shared(q < kTileRows / 8 ? wb : xb, offset[u], tiles_s[stage] + q * 1024);
+            load_to_shared(q < kTileRows / 8 ? wb : xb, offset[u], tiles_s + stage * kStageBytes + q * 1024);
         }
     };
 
@@ -123,14 +129,21 @@ gemm_tile_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, bf16* _
         w_row_s[a] = GATED ? (a < 2 ? wn * 32 + 16 * a + i : 64 + wn * 32 + 16 * (a - 2) + i) : wn * 64 + 16 * a + i;
         x_row_s[a] = wm * 64 + 16 * a + i;
     }
-    if (stages > 0) issue(0, 0);
+#pragma unroll
+    for (int p = 0; p < STAGES - 1; ++p)
+        if (p < stages) issue(p, p);
     for (int s = 0; s < stages; ++s) {
-        const int stage = s % 2;
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // this lane's loads of the stage have landed
-        __syncthreads();                                     // everyone's have, and everyone is done with the other stage
-        if (s + 1 < stages) issue(stage ^ 1, s + 1);
-        const unsigned char* ws = tiles_s[stage];
-        const unsigned char* xs = tiles_s[stage] + kWBytes;
+        const int stage = s % STAGES;
+        // This lane's loads of the stage have landed: loads come back in the order they went out, so
+        // only those of the stages after it may still be on their way (STAGES - 2 of them at most).
+        const int later = min(STAGES - 2, stages - 1 - s);
+        if (later >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoads) : "memory");
+        else if (later == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoads) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();                                     // everyone's have, and everyone is done with the stage before
+        if (s + STAGES - 1 < stages) issue((s + STAGES - 1) % STAGES, s + STAGES - 1);
+        const unsigned char* ws = tiles_s + stage * kStageBytes;
+        const unsigned char* xs = ws + kWBytes;
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
             const int place = ((ks * 4 + g) ^ (i % 8)) * 16;
@@ -231,8 +244,35 @@ WLLM_API int wllm_gemm_tile(const void* x, const void* w, void* out, float* part
     const bf16* wp = static_cast<const bf16*>(w);
     bf16* op = static_cast<bf16*>(out);
     const int per = K / splits;
-    if (activation == 0) gemm_tile_kernel<0><<<grid, 256, 0, stream>>>(xp, wp, op, partial, M, N, K, m_tiles, per);
-    else if (activation == 1) gemm_tile_kernel<1><<<grid, 256, 0, stream>>>(xp, wp, op, partial, M, N, K, m_tiles, per);
-    else gemm_tile_kernel<2><<<grid, 256, 0, stream>>>(xp, wp, op, partial, M, N, K, m_tiles, per);
+    constexpr int kStageBytes = 2 * kTileRows * kRowBytes;
+#define LAUNCH(GATED, STAGES)                                                                                      \
+    do {                                                                                                            \
+        static bool roomy = false;     /* more than 64 KiB of shared memory must be asked for once */              \
+        if (STAGES * kStageBytes > 65536 && !roomy) {                                                               \
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<GATED, STAGES>),                \
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, STAGES * kStageBytes) != hipSuccess) \
+                return launch_status();                                                                             \
+            roomy = true;                                                                                           \
+        }                                                                                                           \
+        gemm_tile_kernel<GATED, STAGES><<<grid, 256, STAGES * kStageBytes, stream>>>(xp, wp, op, partial, M, N, K,  \
+                                                                                     m_tiles, per);                 \
+    } while (0)
+    // at most a workgroup a compute unit: nothing is lost by holding one, and it can have more on its way
+    static int compute_units = 0;
+    if (compute_units == 0) {
+        int device = 0;
+        if (hipGetDevice(&device) != hipSuccess ||
+            hipDeviceGetAttribute(&compute_units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess)
+            return launch_status();
+    }
+    const bool deep = static_cast<long long>(n_tiles) * m_tiles * splits <= compute_units;
+#define BY_STAGES(GATED)                \
+    if (deep) LAUNCH(GATED, 4);         \
+    else LAUNCH(GATED, 2)
+    if (activation == 0) { BY_STAGES(0); }
+    else if (activation == 1) { BY_STAGES(1); }
+    else { BY_STAGES(2); }
+#undef BY_STAGES
+#undef LAUNCH
     return launch_status();
 }
