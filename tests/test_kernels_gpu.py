@@ -373,7 +373,8 @@ def test_tile_weight_is_the_documented_permutation():
 
 
 @pytest.mark.parametrize("m,n,k", [(8, 2048, 16384), (5, 2560, 2048), (64, 1000, 1024), (1, 777, 512), (16, 1000, 8192),
-                                   (3, 3072, 24576), (40, 2048, 16384), (100, 2048, 16384), (512, 96, 8192), (1025, 96, 8192)])
+                                   (3, 3072, 24576), (40, 2048, 16384), (100, 2048, 16384), (512, 96, 8192), (1025, 96, 8192),
+                                   (700, 2048, 16384), (1000, 3072, 24576)])
 def test_linear_leaves_partial_sums_to_the_caller(m, n, k):
     torch.manual_seed(8)
     x = torch.randn(m, k, device=DEV).to(torch.bfloat16)

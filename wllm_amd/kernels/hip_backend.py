@@ -294,25 +294,33 @@ class HipBackend:
     TILE_GATED_MAX_ROWS = 256
 
     @staticmethod
-    def tile_splits(n: int, k: int) -> int:
+    def tile_splits(n: int, k: int, rows: int = 128) -> int:
         """Over how many workgroups the tiled product splits the K axis: a function of the weight's
-        shape only, so that a row's sums do not depend on the step's other rows."""
+        shape up to 640 rows, so that a row's sums do not depend on the step's other rows there.
+        More rows fill the machine with fewer pieces, and every piece is a stack of partial sums to
+        write and to read: halved while the launch has more than 640 workgroups (the down projection
+        of 2,048 x 16,384 with the norm after it, 4 pieces against 8: 78 against 92 us at 1,024 rows,
+        70 against 80 at 896, 68 against 70 at 768, but 67 against 64 at 640; that of 3,072 x 24,576:
+        184 us with 2 pieces against 215 with 8 at 1,024 rows, 155 with 4 against 164 at 768)."""
         tiles = -(-n // 128)
         splits = 1
         while tiles * splits * 2 < 256 and k % (128 * splits) == 0 and k // (2 * splits) >= 512:
             splits *= 2
+        row_tiles = -(-rows // 128)
+        while splits > 2 and row_tiles > 5 and tiles * row_tiles * splits > 640:
+            splits //= 2
         return splits
 
     def tile_takes(self, dtype, rows: int, out_features: int, in_features: int) -> bool:
         return (dtype == torch.bfloat16 and 64 < rows <= self.TILE_MAX_ROWS and in_features >= self.TILE_LONG_K
-                and in_features % 64 == 0 and self.tile_splits(out_features, in_features) > 1
+                and in_features % 64 == 0 and self.tile_splits(out_features, in_features, rows) > 1
                 and max(rows, out_features) * in_features * 2 < 2 ** 32)
 
     def linear_splits(self, rows, out_features, in_features, dtype) -> int:
         if self.skinny_takes(dtype, rows, in_features):
             return self.skinny_split(out_features, in_features)
         if self.tile_takes(dtype, rows, out_features, in_features):
-            return self.tile_splits(out_features, in_features)
+            return self.tile_splits(out_features, in_features, rows)
         return 1
 
     def tile_weight(self, weight, tiles) -> None:
@@ -345,7 +353,7 @@ class HipBackend:
             if self.tile_takes(x.dtype, m, weight.shape[0], k):
                 # some hundred rows and a long K axis: the tiled product, its K axis in pieces whose
                 # sums the caller adds, or a kernel here in their order
-                n, splits = weight.shape[0], self.tile_splits(weight.shape[0], k)
+                n, splits = weight.shape[0], self.tile_splits(weight.shape[0], k, m)
                 stack = out if out.dim() == 3 else torch.empty((splits, m, n), dtype=torch.float32, device=x.device)
                 self._check(self.lib.wllm_gemm_tile(_ptr(x), _ptr(weight), None, _ptr(stack), m, n, k, splits, 0,
                                                     self._stream()), "linear (tiles, partial sums)")
