@@ -79,12 +79,15 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
     __shared__ __align__(16) unsigned char shared_raw[4 * kPartBytes];
     __shared__ float row_max_s[4][kRowsPerTile], row_sum_s[4][kRowsPerTile];
 
-    // a captured graph launches as many workgroups as its plan has room for items; the live ones come first
-    if (live_items != nullptr && static_cast<int>(blockIdx.x) >= live_items[0]) return;
+    // A captured graph launches as many workgroups as its plan has room for items; the live ones come
+    // first.  The item is asked for together with their number, not after it (there is an item, live
+    // or stale, for every workgroup of the launch), and brings the segment's lengths with it: one trip
+    // to memory for all of them.
     const int* item = items + static_cast<size_t>(blockIdx.x) * kItemInts;
-    // the item brings the segment's lengths with it: no second trip to memory for them
     const int seg = item[0], kvh = item[1], q_len = item[2], q_start = item[3];
     const int key_begin = item[4], key_end = item[5], partial_slot = item[6], ctx = item[7];
+    const int live = live_items != nullptr ? live_items[0] : 0x7fffffff;
+    if (static_cast<int>(blockIdx.x) >= live) return;
     constexpr int row_begin = 0;      // a short segment is one tile of rows
     if (seg < 0) return;    // padding item
     const int lane = threadIdx.x % kWave;
