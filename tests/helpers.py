@@ -9,7 +9,8 @@ from wllm_amd.parts import write_random_model_folder
 
 # Two tiny configurations that differ in every size and option, a third with
 # biases and an untied head, a fourth whose head size and page size are the
-# ones the matrix-core attention kernels take, and a fifth without grouped heads.
+# ones the matrix-core attention kernels take, a fifth without grouped heads, a sixth with more
+# query heads a key/value head than a tile of rows holds, and a seventh with pages of 6 tokens.
 TINY = {
     "A": dict(config=GemmaConfig(vocab_size=512, hidden_size=64, intermediate_size=256, num_hidden_layers=2,
                                  num_attention_heads=4, num_key_value_heads=1, head_dim=32, rms_norm_eps=1e-6,
@@ -34,6 +35,16 @@ TINY = {
                                  num_attention_heads=5, num_key_value_heads=5, head_dim=32, rms_norm_eps=1e-6,
                                  rope_theta=10000.0, max_position_embeddings=256, tie_word_embeddings=True),
               seed=55, std=0.04, norm_std=0.1, page_size=8),
+    # 32 query heads on one key/value head: a decoded token's rows fill two tiles of 16
+    "W": dict(config=GemmaConfig(vocab_size=640, hidden_size=64, intermediate_size=160, num_hidden_layers=2,
+                                 num_attention_heads=32, num_key_value_heads=1, head_dim=32, rms_norm_eps=1e-6,
+                                 rope_theta=10000.0, max_position_embeddings=256, tie_word_embeddings=True),
+              seed=66, std=0.04, norm_std=0.1, page_size=8),
+    # pages of 6 tokens (no multiple of 4), 20 query heads on two key/value heads
+    "P": dict(config=GemmaConfig(vocab_size=450, hidden_size=72, intermediate_size=200, num_hidden_layers=2,
+                                 num_attention_heads=20, num_key_value_heads=2, head_dim=32, rms_norm_eps=1e-5,
+                                 rope_theta=3000.0, max_position_embeddings=256, tie_word_embeddings=True),
+              seed=77, std=0.04, norm_std=0.1, page_size=6),
 }
 
 
@@ -41,7 +52,7 @@ TINY = {
 # this small the tied head's logit of a token for itself beats everything the context adds.  Tests
 # that compare generated tokens use these instead: the same sizes with weights large enough that
 # the context decides, so that a wrong key, page or position changes the tokens.
-VARIED = {"AV": dict(TINY["A"], std=0.3), "MV": dict(TINY["M"], std=0.3)}
+VARIED = {"AV": dict(TINY["A"], std=0.3), "MV": dict(TINY["M"], std=0.3), "WV": dict(TINY["W"], std=0.3)}
 
 
 def assert_varied(tokens: list, least: int = 4) -> None:
@@ -61,6 +72,9 @@ def degenerate_folder(src: str, out: str, kind: str) -> str:
         layer adds nothing: logits = final_norm(E[ids] * sqrt(H)) @ head^T;
     "one_feed_forward": as above, but layer 0's down_proj and post-attention norm weight are kept:
         logits = final_norm(x + mlp(norm(x))) @ head^T with x = E[ids] * sqrt(H);
+    "one_attention": every down_proj zero, every o_proj but layer 0's zero, the norm weights of the other
+        layers zero (layer 0 keeps both of its own, so that taking the wrong one shows):
+        logits = final_norm(x + attention(input_norm(x))) @ head^T;
     "bias_only_queries_and_keys": q_proj and k_proj weights zero (the folder must have biases): queries
         and keys are the rotated biases."""
     import os
@@ -74,6 +88,12 @@ def degenerate_folder(src: str, out: str, kind: str) -> str:
             if n.endswith("o_proj.weight") or (n.endswith("down_proj.weight") and not keep):
                 t.zero_()
             if n.endswith("input_layernorm.weight") or (n.endswith("post_attention_layernorm.weight") and not keep):
+                t.zero_()
+        elif kind == "one_attention":
+            first = ".layers.0." in n
+            if n.endswith("down_proj.weight") or (n.endswith("o_proj.weight") and not first):
+                t.zero_()
+            if n.endswith(("input_layernorm.weight", "post_attention_layernorm.weight")) and not first:
                 t.zero_()
         elif kind == "bias_only_queries_and_keys":
             if n.endswith(("q_proj.weight", "k_proj.weight")):

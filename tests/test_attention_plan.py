@@ -18,9 +18,12 @@ def covered(q_len, ctx_len, group, nkv, window, page_size):
         assert slot not in slot_users, f"slot {slot} held by {slot_users[slot]} and {who}"
         slot_users[slot] = who
     for n, it in enumerate(items):
-        seg, kvh, new_tokens, first_token, kb, ke, slot, context = (int(v) for v in it)
+        seg, head_and_row, new_tokens, first_token, kb, ke, slot, context = (int(v) for v in it)
+        kvh, row0 = head_and_row & 0xffff, head_and_row >> 16
         rows = q_len[seg] * group
-        assert rows <= 16
+        # short: at most 16 rows, or one token whose group of heads fills several tiles of 16
+        assert rows <= 16 or q_len[seg] == 1
+        assert row0 % 16 == 0 and row0 < rows
         # the item carries the segment's lengths and the place of its first token in the step
         assert new_tokens == q_len[seg] and context == ctx_len[seg] and first_token == sum(q_len[:seg])
         # the kernel gives each of its four wavefronts one block of 32 keys of an aligned group of 128
@@ -29,12 +32,12 @@ def covered(q_len, ctx_len, group, nkv, window, page_size):
         assert kb >= (max(0, first_pos - window + 1) if window > 0 else 0) and ke <= ctx_len[seg]
         if slot >= 0:
             hold(slot, ("short", n))
-        for r in range(rows):
+        for r in range(row0, min(rows, row0 + 16)):
             cover.setdefault((seg, kvh, r), []).append((kb, ke, slot))
     for n, it in enumerate(prefill):
         seg, kvh, row0, kb, ke, slot = (int(v) for v in it[:6])
         rows = q_len[seg] * group
-        assert rows > 16 and row0 % prefill_rows == 0 and row0 < rows
+        assert rows > 16 and q_len[seg] > 1 and row0 % prefill_rows == 0 and row0 < rows
         first_pos = ctx_len[seg] - q_len[seg]
         last = min(rows - 1, row0 + prefill_rows - 1)
         b_hi = first_pos + last // group + 1
@@ -82,7 +85,7 @@ def test_every_pair_is_covered_once(seed, monkeypatch):
     monkeypatch.setattr(ap, "PREFILL_MIN_CHUNK", 128)
     monkeypatch.setattr(ap, "PREFILL_TARGET_ITEMS", int(rng.choice([1, 8, 64, 1024])))
     monkeypatch.setattr(ap, "PREFILL_TABLE_PAGES", int(rng.choice([34, 1024])))
-    group, nkv = int(rng.choice([1, 2, 3, 8])), int(rng.choice([1, 2, 3]))
+    group, nkv = int(rng.choice([1, 2, 3, 8, 17, 24, 32, 40])), int(rng.choice([1, 2, 3]))
     window = int(rng.choice([0, 0, 40, 300]))
     page_size = int(rng.choice([4, 12, 16, 64]))
     n = int(rng.integers(1, 5))
@@ -103,3 +106,15 @@ def test_a_whole_prompt_of_many_heads_is_not_split():
     _, reduces, slots, prefill = covered([300], [300], 1, 1, 0, 16)
     assert slots == 0 and reduces.shape[0] == 0
     assert (prefill[:, 5] == -1).all()
+
+
+def test_a_decoded_token_of_a_large_group_stays_short():
+    """More than 16 query heads a key/value head: the token's rows fill several tiles of 16, each with
+    its own work items, partial slots and reduce item; nothing goes to the kernel for prompt portions,
+    so a captured decode graph can hold it."""
+    items, reduces, slots, prefill = covered([1, 1, 1], [50, 300, 129], 40, 2, 0, 16)
+    assert prefill.shape[0] == 0
+    assert sorted(set(int(v) >> 16 for v in items[:, 1])) == [0, 16, 32]
+    # 1 + 3 + 2 chunks of keys, for 2 key/value heads and 3 tiles of rows
+    assert items.shape[0] == (1 + 3 + 2) * 2 * 3
+    assert reduces.shape[0] == 2 * 2 * 3 and slots == (3 + 2) * 2 * 3

@@ -17,7 +17,7 @@ from wllm_amd.kernels import ops
 from wllm_amd.parts import load_model
 
 LENGTHS = {"A": [40, 57, 72, 33, 90, 64], "B": [45, 97, 64, 130, 51, 80], "C": [37, 66, 49, 100, 41], "M": [70, 130, 48, 97, 33],
-           "S": [50, 33, 120, 64, 77]}
+           "S": [50, 33, 120, 64, 77], "W": [60, 140, 33, 90, 75], "P": [44, 150, 61, 36, 100]}
 FAMILIES = {"whole": trace_whole, "tail": trace_tail, "portions": trace_portions, "mixed": trace_mixed}
 
 

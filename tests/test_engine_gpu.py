@@ -13,7 +13,7 @@ from wllm_amd.parts import load_model
 pytestmark = pytest.mark.gpu
 
 LENGTHS = {"A": [40, 57, 72, 33, 90, 64], "B": [45, 97, 64, 130, 51, 80], "C": [37, 66, 49, 100, 41], "M": [70, 130, 48, 97, 33],
-           "S": [50, 33, 120, 64, 77]}
+           "S": [50, 33, 120, 64, 77], "W": [60, 140, 33, 90, 75], "P": [44, 150, 61, 36, 100]}
 FAMILIES = {"whole": trace_whole, "tail": trace_tail, "portions": trace_portions, "mixed": trace_mixed}
 # float32: the engine and the oracle differ by the order of float32 sums only.
 # bfloat16: activations between kernels are rounded to 8 bits of mantissa; logits of
@@ -108,10 +108,11 @@ def test_sharp_attention_over_hundreds_of_keys(model_folders, tmp_path_factory, 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name,kind", [("A", "no_contributions"), ("C", "no_contributions"), ("A", "one_feed_forward"),
-                                       ("B", "one_feed_forward"), ("C", "bias_only_queries_and_keys")])
+                                       ("B", "one_feed_forward"), ("C", "bias_only_queries_and_keys"),
+                                       ("A", "one_attention"), ("B", "one_attention"), ("C", "one_attention")])
 def test_models_whose_logits_a_formula_gives(model_folders, tmp_path, name, kind, dtype):
     """The folders that pin the plain implementation's wiring (layers that contribute nothing; one
-    feed-forward alone; queries and keys that are rotated biases), through the engine: whole prompts,
+    feed-forward alone; one attention alone; queries and keys that are rotated biases), through the engine: whole prompts,
     the last tokens one by one, and portions."""
     from helpers import degenerate_folder
     folder = degenerate_folder(model_folders[name], str(tmp_path / kind), kind)

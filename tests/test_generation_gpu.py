@@ -176,14 +176,18 @@ def test_trace_run_says_when_a_trace_holds_more_than_max_tokens(model_folders, t
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_captured_graphs_give_what_eager_steps_give(varied_folders, dtype):
+@pytest.mark.parametrize("name", ["MV", "WV"])
+def test_captured_graphs_give_what_eager_steps_give(varied_folders, name, dtype):
     """Decode steps replayed from captured graphs against the same steps run kernel by kernel:
     several replays with eager work (prompt portions of newly admitted requests) between them,
-    batches that grow and shrink through the buckets, every replay checked."""
-    folder = varied_folders["MV"]
+    batches that grow and shrink through the buckets, every replay checked.  "WV" has 32 query heads
+    on one key/value head: a decoded token's rows fill two tiles of the decode kernel, and the
+    contexts grow past one chunk of keys, so its graphs hold partial results of both tiles."""
+    folder = varied_folders[name]
     model = load_model(folder, dtype, "cuda")
-    prompts = [random_ids(40 + i, n, 1000) for i, n in enumerate([9, 33, 17, 70, 5, 41])]
-    news = [30, 12, 25, 8, 40, 18]
+    vocab = VARIED[name]["config"].vocab_size
+    prompts = [random_ids(40 + i, n, vocab) for i, n in enumerate([9, 33, 17, 120, 5, 41])]
+    news = [30, 12, 25, 28, 40, 18]
 
     def run(graphs):
         runner = ModelRunner.create(model, num_pages=40, page_size=16, max_requests=4)

@@ -1,6 +1,7 @@
 """Each kernel alone against the plain emulation of its contract, at sizes other than
 the engine's tests use: widths and vocabularies that are no power of two, odd head
-counts and groups, partial rotation, windows, page sizes from 4 to 32."""
+counts and groups (up to 40 query heads a key/value head), partial rotation, windows, pages of
+1 to 40 tokens."""
 import math
 
 import pytest
@@ -73,9 +74,15 @@ def test_rms_norm(dtype, hidden, n, mode):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nh,nkv,d,rot,ps,bias", [(3, 1, 40, 24, 8, True), (8, 1, 256, 256, 16, False),
-                                                 (6, 6, 24, 24, 4, False), (4, 2, 64, 32, 32, True)])
+                                                 (6, 6, 24, 24, 4, False), (4, 2, 64, 32, 32, True),
+                                                 # pages that are no multiple of 4 tokens (the transposed values
+                                                 # of a token are then 2 bytes at an odd multiple of 2 apart)
+                                                 (4, 1, 32, 32, 1, False), (3, 3, 24, 24, 3, True),
+                                                 (8, 2, 64, 64, 6, False), (2, 1, 256, 256, 10, False),
+                                                 (5, 1, 20, 12, 7, True)])
 def test_rope_and_cache_write(dtype, nh, nkv, d, rot, ps, bias):
-    n, pages = 29, 12
+    n = 29
+    pages = max(12, -(-n // ps) + 3)
     torch.manual_seed(2)
     width = (nh + 2 * nkv) * d
 
@@ -197,6 +204,17 @@ ATTENTION_SHAPES = [
     (6, 2, 20, 16, [(9, 30), (1, 200)], 0),
     (12, 1, 48, 16, [(1, 150), (20, 64)], 0),
     (4, 2, 64, 16, [(1, 100), (30, 70), (50, 50)], 17),
+    # pages that are no multiple of 4 tokens: 1, 3, 6, 10, 7
+    (4, 1, 32, 1, [(1, 37), (9, 9), (3, 140)], 0),
+    (6, 3, 24, 3, [(1, 131), (20, 47), (2, 260)], 0),
+    (8, 2, 64, 6, [(1, 300), (33, 90), (1, 1), (5, 129)], 0),
+    (2, 1, 256, 10, [(1, 257), (40, 40)], 0),
+    (6, 2, 40, 7, [(1, 200), (17, 64), (1, 128)], 50),
+    # more than 16 query heads a key/value head: 17, 24, 32 and 40
+    (17, 1, 64, 16, [(1, 300), (1, 5), (3, 40), (20, 20)], 0),
+    (24, 1, 32, 8, [(1, 129), (2, 70), (1, 1)], 0),
+    (32, 1, 128, 16, [(1, 700), (1, 128), (9, 200)], 0),
+    (80, 2, 32, 4, [(1, 260), (1, 33), (5, 5)], 90),
 ]
 
 
@@ -343,6 +361,23 @@ def test_linear(dtype, m, n, k):
             torch.manual_seed(4)
             g, r = both("linear", make, dtype)
             close(g[2], r[2], out_dtype, f"product to {out_dtype}, tiled {tiled}")
+
+
+def test_float32_logits_of_a_large_vocabulary_at_few_rows():
+    """7 to 16 rows, two segments of the K axis and 120,000 columns: more partial sums than the buffer
+    of split sums holds at once, so the rows run in groups; every group's rows have the bits they have
+    in a product of many rows."""
+    torch.manual_seed(15)
+    n, k = 120000, 3072
+    x = torch.randn(40, k, device=DEV)
+    w = torch.randn(n, k, device=DEV) / math.sqrt(k)
+    many = torch.zeros(40, n, device=DEV)
+    ops.linear(x, w, many)
+    close(many, x.double() @ w.double().T, torch.float32, "product of many rows")
+    for rows in (6, 7, 12, 16):
+        few = torch.full((rows, n), 9.0, device=DEV)
+        ops.linear(x[3:3 + rows].contiguous(), w, few)
+        assert torch.equal(few, many[3:3 + rows]), f"{rows} rows"
 
 
 @pytest.mark.parametrize("n,k", [(777, 250), (2048, 2048), (100, 4128), (33, 64), (2560, 16384)])

@@ -26,6 +26,18 @@ def test_norm_with_zero_weight_is_plain_normalisation():
     assert torch.allclose(P.rms_norm_one_plus_w(x, torch.zeros(48, dtype=torch.float64), 0.0), x)
 
 
+def test_eps_is_added_under_the_root():
+    """Rows of mean square 1 and eps 0.5: x / sqrt(1.5) (src/wllm/models/gemma.py:47-48, rsqrt(variance + eps)).
+    With eps added to the root instead the result is x / 1.5, a fifth smaller; with eps inside a mean over
+    squares that forgot to divide, or left out, it is x."""
+    x = torch.randn(4, 40, dtype=torch.float64)
+    x = x / x.pow(2).mean(-1, keepdim=True).sqrt()
+    y = P.rms_norm_one_plus_w(x, torch.zeros(40, dtype=torch.float64), 0.5)
+    assert torch.allclose(y, x / math.sqrt(1.5), rtol=1e-12, atol=0)
+    assert not torch.allclose(y, x / 1.5, rtol=0.1, atol=0)
+    assert not torch.allclose(y, x, rtol=0.1, atol=0)
+
+
 def test_norm_weight_is_an_offset_from_one():
     x = torch.randn(3, 16, dtype=torch.float64)
     w = torch.randn(16, dtype=torch.float64)
@@ -223,6 +235,63 @@ def test_one_feed_forward_is_added_to_the_stream_it_read_through_a_norm(model_fo
     unnormed = (torch.nn.functional.gelu(x @ w[p + "mlp.gate_proj.weight"].T, approximate="tanh")
                 * (x @ w[p + "mlp.up_proj.weight"].T)) @ w[p + "mlp.down_proj.weight"].T
     assert not torch.allclose(got, _hand_norm(x + unnormed, w["model.norm.weight"], eps) @ w["model.embed_tokens.weight"].T, atol=1e-3)
+
+
+def _hand_attention(h, w, p, cfg):
+    """Attention of one layer written out with the library's routines: projections, the rotation as the
+    complex product (x_j + i x_{j+d/2}) * exp(i * pos * theta^(-2j/d)), causal SDPA head by head."""
+    nh, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    T = h.shape[0]
+    angle = torch.arange(T, dtype=torch.float64)[:, None] * cfg["rope_theta"] ** (-torch.arange(0, d, 2, dtype=torch.float64) / d)
+    turn = torch.polar(torch.ones_like(angle), angle)[:, None, :]            # [T, 1, d/2]
+
+    def rotated(x, heads):
+        x = x.view(T, heads, d)
+        z = torch.complex(x[..., :d // 2], x[..., d // 2:]) * turn
+        return torch.cat((z.real, z.imag), -1)
+
+    q = h @ w[p + "self_attn.q_proj.weight"].T
+    k = h @ w[p + "self_attn.k_proj.weight"].T
+    v = h @ w[p + "self_attn.v_proj.weight"].T
+    if cfg["attention_bias"]:
+        q, k, v = (t + w[p + f"self_attn.{n}_proj.bias"] for t, n in ((q, "q"), (k, "k"), (v, "v")))
+    q, k, v = rotated(q, nh), rotated(k, nkv), v.view(T, nkv, d)
+    out = torch.empty(T, nh, d, dtype=torch.float64)
+    for head in range(nh):
+        kv = head // (nh // nkv)
+        out[:, head] = torch.nn.functional.scaled_dot_product_attention(q[None, :, head], k[None, :, kv], v[None, :, kv],
+                                                                        is_causal=True)[0]
+    return out.reshape(T, nh * d) @ w[p + "self_attn.o_proj.weight"].T
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_one_attention_reads_the_input_norm_and_is_added_to_the_stream_as_it_was(model_folders, tmp_path, name):
+    """Only layer 0's attention contributes: logits = norm_f(x + attn(norm_1(x))) @ head^T, x = E[ids] * sqrt(H)
+    (src/wllm/models/gemma.py:83-87): attention reads the stream through `input_layernorm` (not through the
+    layer's other norm, and not the raw stream), and its output is added to the stream as it was, which
+    nothing normalises before the next norm."""
+    from helpers import degenerate_folder
+    folder = degenerate_folder(model_folders[name], str(tmp_path / "attn"), "one_attention")
+    cfg = P.read_config(folder)
+    w = P.read_weights(folder, torch.float64)
+    ids = torch.randint(0, cfg["vocab_size"], (13,))
+    eps, p = cfg["rms_norm_eps"], "model.layers.0."
+    table = w["model.embed_tokens.weight"]
+    head = table if cfg["tie_word_embeddings"] else w["lm_head.weight"]
+    # the factor is a float32 number in the reference (src/wllm/models/llama.py:388-397), also under a wider model
+    x = table[ids] * float(torch.tensor(cfg["hidden_size"] ** 0.5, dtype=torch.float32))
+    final = lambda t: _hand_norm(t, w["model.norm.weight"], eps) @ head.T
+    h = _hand_norm(x, w[p + "input_layernorm.weight"], eps)
+    attn = _hand_attention(h, w, p, cfg)
+    assert attn.abs().max() > 1e-3 * x.abs().max(), "the attention matters in this test"
+    got = P.forward_logits(cfg, w, ids)
+    assert torch.allclose(got, final(x + attn), atol=1e-10)
+    # the plausible mistakes are far away: the other norm's weight, the raw stream, the sum on the
+    # normalised copy, the attention's output normalised
+    other = _hand_attention(_hand_norm(x, w[p + "post_attention_layernorm.weight"], eps), w, p, cfg)
+    raw = _hand_attention(x, w, p, cfg)
+    for wrong in (final(x + other), final(x + raw), final(h + attn), final(x + _hand_norm(attn, w[p + "input_layernorm.weight"], eps))):
+        assert not torch.allclose(got, wrong, atol=1e-3)
 
 
 def test_biases_are_added_before_the_rotation():

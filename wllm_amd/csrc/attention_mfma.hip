@@ -10,7 +10,8 @@
 // src/wllm/kernels/csrc/paged_attention.cu:44-45,185).
 //
 // Work items.  The host cuts every (segment, key/value head) into work items, one workgroup of 4
-// wavefronts each: the segment's one tile of 16 rows and a chunk of keys that lies within one
+// wavefronts each: a tile of 16 of the segment's rows (it has one, unless more than 16 query heads
+// share a key/value head) and a chunk of keys that lies within one
 // aligned group of 128 keys, cut to what the rows can need.  Each wavefront takes one of the
 // chunk's four blocks of 32 keys; its loads of keys and values wait for the item and the block
 // table only (the request's lengths and the queries are read while they are in flight), and the
@@ -84,11 +85,11 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
     // or stale, for every workgroup of the launch), and brings the segment's lengths with it: one trip
     // to memory for all of them.
     const int* item = items + static_cast<size_t>(blockIdx.x) * kItemInts;
-    const int seg = item[0], kvh = item[1], q_len = item[2], q_start = item[3];
+    const int seg = item[0], kvh = item[1] & 0xffff, q_len = item[2], q_start = item[3];
     const int key_begin = item[4], key_end = item[5], partial_slot = item[6], ctx = item[7];
     const int live = live_items != nullptr ? live_items[0] : 0x7fffffff;
     if (static_cast<int>(blockIdx.x) >= live) return;
-    constexpr int row_begin = 0;      // a short segment is one tile of rows
+    const int row_begin = item[1] >> 16;      // the tile's first row: 0 unless a token has more than 16 heads a group
     if (seg < 0) return;    // padding item
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -498,7 +499,8 @@ WLLM_API int wllm_paged_attention_mfma(const void* qkv, const void* cache, const
                                        const int* seg_ctx_len, void* out, float* partial_o, float* partial_ml,
                                        int num_heads, int num_kv_heads, int head_dim, int page_size, int max_pages,
                                        float scale, int window, hipStream_t stream) {
-    if (head_dim % 32 != 0 || head_dim < 32 || head_dim > 256 || page_size % 4 != 0 || num_heads % num_kv_heads != 0)
+    if (head_dim % 32 != 0 || head_dim < 32 || head_dim > 256 || page_size % 4 != 0 || num_heads % num_kv_heads != 0 ||
+        num_heads >= (1 << 16))       // an item holds a key/value head and a tile's first row in 16 bits each
         return -1;
     const AttentionArguments a = {static_cast<const bf16*>(qkv), static_cast<const bf16*>(cache), block_tables, items,
                                   live_items, num_items, reduce_items, num_reduce_items, seg_q_start, seg_q_len,

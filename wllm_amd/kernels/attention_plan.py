@@ -1,13 +1,15 @@
 """How a step's attention is cut into work items for the matrix-core kernel.
 
 For one request (segment) and one key/value head the query rows are the pairs (token, query
-head of the group): rows = q_len * group.  A segment of at most 16 rows (a decoded token) is one
-tile of rows whose keys are split over workgroups in fixed chunks of `KEY_CHUNK` keys, the
+head of the group): rows = q_len * group.  A segment of at most 16 rows, and a segment of one token
+whatever its group (a decoded token), is short: tiles of 16 rows (one, unless more than 16 query heads
+share a key/value head) whose keys are split over workgroups in fixed chunks of `KEY_CHUNK` keys, the
 partial results combined by a second kernel; chunk boundaries are multiples of the chunk size
 counted from key 0, so they depend on the key index only.  Longer segments are cut into
 workgroups of four tiles of 16 rows (prefill items).
 
-A work item is 8 int32: segment, key/value head, the segment's number of new tokens, the place of
+A work item is 8 int32: segment, key/value head in the low 16 bits with the tile's first row in the
+high 16, the segment's number of new tokens, the place of
 its first token among the step's tokens, first key, end key, partial slot (-1: the workgroup writes
 the final result), the segment's context length: what the kernel needs of the segment comes with
 the item, in the one read it begins with, and not from the segments' arrays in a second trip to memory.  A partial slot holds
@@ -64,7 +66,8 @@ class StaticAttentionPlan(AttentionPlan):
     def __init__(self, segments: int, group: int, num_kv_heads: int, window: int, fixed_splits: int,
                  max_slots: int, head_dim: int, device):
         # a live item of a segment with several chunks holds a partial slot; a segment with one has one item
-        n_r = segments * num_kv_heads
+        n_r = segments * num_kv_heads * row_tiles(1, group)
+        max_slots = min(max_slots, n_r * fixed_splits)
         n_i = min(n_r * fixed_splits, max_slots + n_r)
         # the number of live items (and 7 unused), the reduce items, the items: a step copies the
         # front of it, up to the last live item
@@ -81,7 +84,8 @@ class StaticAttentionPlan(AttentionPlan):
     def update(self, q_len: np.ndarray, ctx_len: np.ndarray) -> None:
         group, nkv, window = self._args
         items, reduces, slots, prefill, _ = build_work_items(q_len, ctx_len, group, nkv, window)
-        assert prefill.shape[0] == 0, "a captured decode graph holds no long segment"
+        if prefill.shape[0]:
+            raise ValueError("a captured decode graph holds segments of one token only")
         if slots > self.max_slots:
             raise ValueError(f"the step needs {slots} partial slots, the graph's plan has {self.max_slots}")
         if items.shape[0] > self.num_items or reduces.shape[0] > self.num_reduce:
@@ -99,6 +103,14 @@ class StaticAttentionPlan(AttentionPlan):
         self._dev[:used].copy_(self._host[:used], non_blocking=True)
 
 
+def row_tiles(q_len: int, group: int) -> int:
+    """Tiles of 16 rows of a short segment of `q_len` tokens."""
+    return -(-(q_len * group) // ROWS_PER_TILE)
+
+
+MAX_HEADS = 1 << 16     # an item packs the key/value head and the tile's first row into 16 bits each
+
+
 def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_heads: int, window: int,
                      page_size: int = 16):
     """Returns (items [n, 8], reduce_items [m, 8], partial slots, prefill items [p, 8], rows per
@@ -107,7 +119,9 @@ def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_
     ctx_len = np.asarray(ctx_len, dtype=np.int64)
     rows = q_len * group
     q_start = np.cumsum(q_len) - q_len
-    short = rows <= ROWS_PER_TILE
+    if group * num_kv_heads >= MAX_HEADS:
+        raise ValueError(f"{group * num_kv_heads} query heads: a work item has 16 bits for a head")
+    short = (rows <= ROWS_PER_TILE) | (q_len == 1)
     items, reduces = [], []
     slots = 0
     kv = np.arange(num_kv_heads, dtype=np.int64)
@@ -126,33 +140,40 @@ def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_
         kb = np.maximum(lo[:, None], chunk * KEY_CHUNK)
         ke = np.minimum(ctx_len[idx][:, None], (chunk + 1) * KEY_CHUNK)
         single = ns == 1
-        # partial slots: one per (segment, kv head, split) for segments that are split
+        # tiles of 16 rows a segment has (one, unless a token's group has more than 16 heads)
+        rt = -(-rows[idx] // ROWS_PER_TILE)
+        T = int(rt.max())
+        tile = np.arange(T, dtype=np.int64)
+        tile_live = tile[None, :] < rt[:, None]                 # [S, T]
+        # partial slots: one per (segment, kv head, tile, split) for segments that are split
         n_split_seg = np.where(single, 0, ns)
-        seg_base = np.concatenate([[0], np.cumsum(n_split_seg * num_kv_heads)])[:-1]
+        seg_base = np.concatenate([[0], np.cumsum(n_split_seg * num_kv_heads * rt)])[:-1]
         S = idx.size
-        it = np.zeros((S, num_kv_heads, width, ITEM_INTS), dtype=np.int32)
-        it[..., 0] = np.where(live, idx[:, None], -1)[:, None, :]
-        it[..., 1] = kv[None, :, None]
-        it[..., 2] = q_len[idx][:, None, None]
-        it[..., 3] = q_start[idx][:, None, None]
-        it[..., 4] = kb[:, None, :]
-        it[..., 5] = ke[:, None, :]
-        it[..., 7] = ctx_len[idx][:, None, None]
-        slot = seg_base[:, None, None] + kv[None, :, None] * n_split_seg[:, None, None] + j[None, None, :]
-        it[..., 6] = np.where(single[:, None, None], -1, slot)
-        keep = np.broadcast_to(live[:, None, :], (S, num_kv_heads, width))
+        it = np.zeros((S, num_kv_heads, T, width, ITEM_INTS), dtype=np.int32)
+        it[..., 0] = np.where(live, idx[:, None], -1)[:, None, None, :]
+        it[..., 1] = (kv[None, :, None] | (tile[None, None, :] * ROWS_PER_TILE << 16))[..., None]
+        it[..., 2] = q_len[idx][:, None, None, None]
+        it[..., 3] = q_start[idx][:, None, None, None]
+        it[..., 4] = kb[:, None, None, :]
+        it[..., 5] = ke[:, None, None, :]
+        it[..., 7] = ctx_len[idx][:, None, None, None]
+        first_slot = seg_base[:, None, None] + (kv[None, :, None] * rt[:, None, None] + tile[None, None, :]) \
+            * n_split_seg[:, None, None]                        # [S, kv, T]
+        it[..., 6] = np.where(single[:, None, None, None], -1, first_slot[..., None] + j[None, None, None, :])
+        keep = np.broadcast_to(live[:, None, None, :] & tile_live[:, None, :, None], (S, num_kv_heads, T, width))
         items.append(it[keep].reshape(-1, ITEM_INTS))
         split_seg = ~single
         if split_seg.any():
-            rs = np.zeros((S, num_kv_heads, ITEM_INTS), dtype=np.int32)
-            rs[..., 0] = idx[:, None]
-            rs[..., 1] = kv[None, :]
-            rs[..., 2] = seg_base[:, None] + kv[None, :] * n_split_seg[:, None]
-            rs[..., 3] = ns[:, None]
-            rs[..., 4] = 0
+            rs = np.zeros((S, num_kv_heads, T, ITEM_INTS), dtype=np.int32)
+            rs[..., 0] = idx[:, None, None]
+            rs[..., 1] = kv[None, :, None]
+            rs[..., 2] = first_slot
+            rs[..., 3] = ns[:, None, None]
+            rs[..., 4] = tile[None, None, :] * ROWS_PER_TILE
             rs[..., 5] = 1
-            reduces.append(rs[split_seg].reshape(-1, ITEM_INTS))
-        slots = int((n_split_seg * num_kv_heads).sum())
+            keep_r = np.broadcast_to((split_seg[:, None] & tile_live)[:, None, :], (S, num_kv_heads, T))
+            reduces.append(rs[keep_r].reshape(-1, ITEM_INTS))
+        slots = int((n_split_seg * num_kv_heads * rt).sum())
     # ---- long segments: workgroups of 64 or 128 rows of one key/value head ----
     prefill = []
     long_idx = np.nonzero(~short)[0]

@@ -188,11 +188,11 @@ class HipBackend:
         """A plan of fixed shape for a captured decode graph of `segments` requests of one token."""
         if not self.mfma_attention_takes(dtype, head_dim, page_size):
             return None
-        from wllm_amd.kernels.attention_plan import KEY_CHUNK, StaticAttentionPlan
+        from wllm_amd.kernels.attention_plan import KEY_CHUNK, StaticAttentionPlan, row_tiles
+        group = num_heads // num_kv_heads
         fixed = -(-max_context // KEY_CHUNK)
-        max_slots = (max_total_keys // KEY_CHUNK + 2 * segments) * num_kv_heads
-        return StaticAttentionPlan(segments, num_heads // num_kv_heads, num_kv_heads, window, fixed, max_slots,
-                                   head_dim, device)
+        max_slots = (max_total_keys // KEY_CHUNK + 2 * segments) * num_kv_heads * row_tiles(1, group)
+        return StaticAttentionPlan(segments, group, num_kv_heads, window, fixed, max_slots, head_dim, device)
 
     def _ensure_partials(self, slots: int, head_dim: int, device) -> None:
         need = max(1, slots) * 16 * head_dim
@@ -375,14 +375,29 @@ class HipBackend:
                 torch.mm(x, weight.t(), out=out)
                 return
         # float32, few rows, a long K axis: the segments of K are summed by workgroups of their own
-        partial = None
         if x.dtype == torch.float32 and m <= 16:
             segments = self.lib.wllm_gemm_generic_segments(k)
-            if segments > 1:
-                partial = self._gemm_partial(segments * m * weight.shape[0], x.device)
+            n = weight.shape[0]
+            if segments > 1 and segments * m * n > self.GEMM_PARTIAL_FLOATS:
+                # more partial sums than the buffer holds (logits of a large vocabulary): some rows at a
+                # time; a row's sums do not depend on the rows beside it
+                rows = self.GEMM_PARTIAL_FLOATS // (segments * n)
+                if rows < 1:
+                    raise KernelError(f"linear: {segments} segments of {n} columns need more than the "
+                                      f"{self.GEMM_PARTIAL_FLOATS} floats of the split-sum buffer for one row")
+                for r in range(0, m, rows):
+                    self._generic(x[r:r + rows], weight, out[r:r + rows], segments)
+                return
+            self._generic(x, weight, out, segments)
+            return
+        self._generic(x, weight, out, 1)
+
+    def _generic(self, x, weight, out, segments: int) -> None:
+        m, n = x.shape[0], weight.shape[0]
+        partial = self._gemm_partial(segments * m * n, x.device) if segments > 1 else None
         self._check(self.lib.wllm_gemm_generic(
             _ptr(x), _ptr(weight), int(x.dtype == torch.bfloat16), _ptr(out), int(out.dtype == torch.bfloat16),
-            _ptr(partial), x.shape[0], weight.shape[0], x.shape[1], self._stream()), "linear")
+            _ptr(partial), m, n, x.shape[1], self._stream()), "linear")
 
     def gated_linear(self, x, weight, out, activation, scratch, tiles=None):
         self._on_gpu(x, weight, out, scratch, tiles)
