@@ -23,6 +23,18 @@ class EmulatedKernels:
     def _count(self, name):
         self.calls[name] = self.calls.get(name, 0) + 1
 
+    def run_registered(self, op, args, kwargs):
+        """An operation that went through `ops.register_op`: the framework's own have their emulation
+        here under their name; one that a part registered brings its own."""
+        own = getattr(self, op.name, None)
+        if own is not None:
+            own(*args, **kwargs)
+            return
+        self._count(op.name)
+        if op.emulate is None:
+            raise NotImplementedError(f"operation {op.name!r} was registered without an emulation")
+        op.emulate(*args, **kwargs)
+
     def embed_lookup(self, ids, table, scale, out):
         self._count("embed_lookup")
         out.copy_((table[ids.long()].to(self.acc) * scale).to(out.dtype))

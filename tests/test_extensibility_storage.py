@@ -198,7 +198,7 @@ def check_toy3(folder, device, dtype="float32"):
         assert len(cache.groups) == 2, "compressed vectors and keys/values: two groups of pages"
         latent_group = cache.groups[cache.group_of_entry[0]]
         assert tuple(latent_group.storage.shape[2:]) == (4, R) and latent_group.storage.dtype == torch.float32
-        assert cache.state[0].dtype == torch.int32 and tuple(cache.state[0].shape) == (4, 1)
+        assert cache.state[0].dtype == torch.int32 and tuple(cache.state[0].shape) == (4 + 1, 1)      # max_requests rows and the padding row
         got = replay_and_collect(TraceReplayer(runner), trace)
         tol = dict(atol=5e-5, rtol=2e-4) if dtype == "float32" else dict(atol=8e-2, rtol=3e-2)      # logits up to 3 from weights of std 0.2
         compare_with_plain(got, plain, **tol)

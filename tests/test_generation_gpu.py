@@ -9,7 +9,8 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import TINY, VARIED, assert_varied, compare_with_plain, random_ids, replay_and_collect, trace_tail, trace_whole
+from helpers import (TINY, VARIED, assert_varied, bfloat16_row_errors, compare_replay, plain_exact_and_rounded, plain_for, random_ids,
+                     replay_and_collect, trace_tail, trace_whole)
 from plain import gemma_plain
 from wllm_amd.engine import LLM, ModelRunner, Request, Scheduler
 from wllm_amd.engine.replay import TraceReplayer
@@ -24,25 +25,52 @@ def plain_model(folder):
     return gemma_plain.read_config(folder), gemma_plain.read_weights(folder, torch.float32)
 
 
-@pytest.mark.parametrize("name,lengths,new", [("A", [7, 16, 23], 8), ("B", [5, 31, 64], 6), ("C", [9, 20], 6), ("M", [33, 70], 6),
-                                              ("AV", [7, 16, 23], 12), ("MV", [33, 70, 12], 12)])
+@pytest.mark.parametrize("name,lengths,new", [("C", [9, 20], 6), ("AV", [7, 16, 23], 12), ("MV", [33, 70, 12], 12)])
 def test_greedy_generation_through_the_entry_point_float32(model_folders, varied_folders, name, lengths, new):
-    # the first case is a tiny workload of its own: prompts of 7/16/23 ids, 8 greedy tokens each, pages of 4.
-    # A, B and M repeat their last prompt token (the tied head's self-logit wins); C, AV and MV do not.
+    """Greedy decoding of models whose continuation varies (so that a wrong key, page or position
+    changes the tokens): the plain implementation's full recomputation, token for token."""
     folder = model_folders[name] if name in model_folders else varied_folders[name]
     cfg, w = plain_model(folder)
     prompts = [random_ids(i + 1, n, cfg["vocab_size"]) for i, n in enumerate(lengths)]
     llm = LLM(folder, dtype="float32", num_blocks=64, block_size=(TINY.get(name) or VARIED[name])["page_size"])
     outs = llm.generate(prompts, max_new_tokens=new)
-    if name in ("C", "AV", "MV"):
-        for o in outs:
-            assert_varied(o.token_ids)
     for p, o in zip(prompts, outs):
+        assert_varied(o.token_ids)
         assert o.token_ids == gemma_plain.generate_greedy(cfg, w, p, new)
         assert o.finish_reason == "length" and len(o.logprobs) == new
         full = gemma_plain.forward_logits(cfg, w, p + o.token_ids[:-1])
         ref_lp = torch.log_softmax(full[len(p) - 1:].double(), -1).gather(-1, torch.tensor(o.token_ids)[:, None])[:, 0]
         assert torch.allclose(torch.tensor(o.logprobs, dtype=torch.float64), ref_lp, atol=1e-4)
+    llm.runner.cache.check()
+
+
+@pytest.mark.parametrize("name,lengths,new,temperature", [("A", [7, 16, 23], 8, 0.3), ("B", [5, 31, 64], 6, 0.5),
+                                                          ("M", [33, 70], 6, 0.8)])
+def test_seeded_sampling_through_the_entry_point_float32(model_folders, name, lengths, new, temperature):
+    """The first case is a tiny workload of its own: prompts of 7/16/23 ids, 8 tokens each, pages of 4.
+    Greedy decoding of these three models repeats the last prompt token whatever the context adds (the
+    tied head's logit of a token for itself wins), so they sample, at a temperature at which the
+    context decides among a handful of tokens: every token must be the one that the plain
+    implementation's distribution gives the request's uniform number."""
+    from plain import sampling_plain
+    folder = model_folders[name]
+    cfg, w = plain_model(folder)
+    prompts = [random_ids(i + 1, n, cfg["vocab_size"]) for i, n in enumerate(lengths)]
+    params = [SamplingParams(temperature=temperature, seed=900 + i) for i in range(len(prompts))]
+    llm = LLM(folder, dtype="float32", num_blocks=64, block_size=TINY[name]["page_size"])
+    outs = llm.generate(prompts, params, max_new_tokens=new)
+    assert len({t for o in outs for t in o.token_ids}) >= 6, "the sampled tokens vary"
+    for i, (p, o) in enumerate(zip(prompts, outs)):
+        tokens = list(p)
+        for k, t in enumerate(o.token_ids):
+            logits = gemma_plain.forward_logits(cfg, w, tokens)[-1]
+            u = sampling_plain.philox_uniform(900 + i, k)
+            _, _, _, (low, high) = sampling_plain.sample_row(logits, temperature, 0, 1.0, 0.0, 1.0, [], u)
+            assert low[t] - 1e-4 <= u <= high[t] + 1e-4, f"request {i} token {k}"
+            ref_lp = float(torch.log_softmax(logits.double() / temperature, -1)[t])
+            assert abs(o.logprobs[k] - ref_lp) < 1e-4
+            tokens.append(t)
+        assert o.finish_reason == "length"
     llm.runner.cache.check()
 
 
@@ -101,13 +129,12 @@ def test_chunked_prefill_beside_decodes_with_seeded_temperature(model_folders):
 def test_long_decoding(model_folders, dtype):
     """300 tokens decoded one by one after a short prompt, over many page boundaries."""
     folder = model_folders["M"]
-    cfg, w = plain_model(folder)
+    cfg, _ = plain_model(folder)
     toks = random_ids(9, 340, cfg["vocab_size"])
-    plain = {"r": gemma_plain.forward_logits(cfg, w, toks, scale_rounding=torch.bfloat16 if dtype == "bfloat16" else None)}
+    plain = plain_for(cfg, folder, {"r": toks}, dtype)
     runner = ModelRunner.create(load_model(folder, dtype, "cuda"), num_pages=22, page_size=16, max_requests=2)
     got = replay_and_collect(TraceReplayer(runner), trace_tail({"r": toks}, tail=300))
-    tol = dict(atol=2e-5, rtol=1e-4) if dtype == "float32" else dict(atol=1e-2, rtol=1e-2)
-    compare_with_plain(got, plain, **tol)
+    compare_replay(got, plain, dtype)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -115,15 +142,13 @@ def test_long_decoding(model_folders, dtype):
 def test_first_tokens_of_a_sequence(model_folders, name, dtype):
     """Prompts of one, two and three tokens, whole and token by token."""
     folder = model_folders[name]
-    cfg, w = plain_model(folder)
+    cfg, _ = plain_model(folder)
     requests = {f"r{n}": random_ids(n, n, cfg["vocab_size"]) for n in (1, 2, 3)}
-    plain = {rid: gemma_plain.forward_logits(cfg, w, t, scale_rounding=torch.bfloat16 if dtype == "bfloat16" else None)
-             for rid, t in requests.items()}
+    plain = plain_for(cfg, folder, requests, dtype)
     model = load_model(folder, dtype, "cuda")
-    tol = dict(atol=2e-5, rtol=1e-4) if dtype == "float32" else dict(atol=1e-2, rtol=1e-2)
     for trace in (trace_whole(requests), trace_tail(requests, tail=3)):
         runner = ModelRunner.create(model, num_pages=8, page_size=TINY[name]["page_size"], max_requests=2)
-        compare_with_plain(replay_and_collect(TraceReplayer(runner), trace), plain, **tol)
+        compare_replay(replay_and_collect(TraceReplayer(runner), trace), plain, dtype)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -144,15 +169,20 @@ def test_trace_run_program(model_folders, tmp_path, dtype):
                           input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stderr[-2000:]
     assert proc.stdout.split() == ["done", "0", "done", "1", "done", "2", "done", "7"]
-    rounding = torch.bfloat16 if dtype == "bfloat16" else None
-    pa = gemma_plain.forward_logits(cfg, w, a, scale_rounding=rounding)
-    pb = gemma_plain.forward_logits(cfg, w, b, scale_rounding=rounding)
-    expect = {0: [pa[0], pa[16]], 1: [pb[19]], 2: [pb[20], pa[29]], 7: [pb[1]]}
-    atol, rtol = (2e-5, 1e-4) if dtype == "float32" else (1e-2, 1e-2)
+    expect = {0: [("a", 0), ("a", 16)], 1: [("b", 19)], 2: [("b", 20), ("a", 29)], 7: [("b", 1)]}
+    if dtype == "float32":
+        plain = {"a": gemma_plain.forward_logits(cfg, w, a), "b": gemma_plain.forward_logits(cfg, w, b)}
+    else:
+        w64 = gemma_plain.read_weights(folder, torch.float64)
+        plain = {"a": plain_exact_and_rounded(cfg, w64, a), "b": plain_exact_and_rounded(cfg, w64, b)}
     for step, rows in expect.items():
         got = torch.from_numpy(np.fromfile(out / f"{step}.f32", dtype="<f4").reshape(len(rows), 512))
-        ref = torch.stack(rows)
-        assert ((got.double() - ref.double()).abs() <= atol + rtol * ref.double().abs()).all(), f"step {step}"
+        for row, (rid, pos) in zip(got, rows):
+            if dtype == "float32":
+                ref = plain[rid][pos].double()
+                assert ((row.double() - ref).abs() <= 2e-5 + 1e-4 * ref.abs()).all(), f"step {step}"
+            else:
+                assert max(bfloat16_row_errors(row, plain[rid][0][pos], [r[pos] for r in plain[rid][1]])) <= 1.0, f"step {step}"
 
 
 def test_trace_run_says_when_a_trace_holds_more_than_max_tokens(model_folders, tmp_path):
@@ -326,6 +356,66 @@ def test_looking_ahead_gives_the_same_tokens_on_the_gpu(varied_folders, dtype, g
     for a, b in zip(stepwise, ahead):
         assert a.output_token_ids == b.output_token_ids and a.finish_reason == b.finish_reason
         assert torch.allclose(torch.tensor(a.logprobs), torch.tensor(b.logprobs), atol=1e-5 if dtype == "float32" else 2e-2)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_requests_preempted_between_replayed_graphs_and_steps_run_ahead(varied_folders, dtype):
+    """Pages run out in the middle of decoding (`admission="prompt_only"` admits on the prompts alone)
+    while decode steps replay captured graphs and every step is started before the one before it was
+    read: the request admitted last gives its pages back, keeps what it generated, comes back through
+    a prompt of its own and goes on.  In float32 every request generates what it generates with pages
+    to spare, step by step and kernel by kernel; in bfloat16 (where a token recomputed inside a prompt
+    is rounded differently from the token that was decoded) every request still completes, the cache's
+    books are right after every step, and the requests that were never preempted generate the same."""
+    model = load_model(varied_folders["MV"], dtype, "cuda")
+    prompts = [random_ids(300 + i, n, 1000) for i, n in enumerate([20, 37, 12, 30, 25])]
+    news = [40, 30, 45, 28, 35]
+
+    def run(pages, admission, graphs, lookahead):
+        runner = ModelRunner.create(model, num_pages=pages, page_size=16, max_requests=4)
+        if graphs:
+            runner.enable_graphs(buckets=(1, 2, 4))
+        s = Scheduler(runner, max_prefill_tokens_per_step=32, admission=admission, lookahead=lookahead)
+        reqs = [Request(i, p, n) for i, (p, n) in enumerate(zip(prompts, news))]
+        for r in reqs:
+            s.add_request(r)
+        steps = 0
+        while s.has_unfinished_requests():
+            s.step()
+            runner.cache.check()
+            steps += 1
+            assert steps < 2000
+        assert not runner.cache.requests
+        return reqs, s, runner
+
+    roomy, s0, _ = run(40, "pledged", False, False)
+    assert s0.stats["preemptions"] == 0
+    tight, s1, runner = run(9 + 1, "prompt_only", True, True)       # nine pages for requests, one for the graphs' padding rows
+    assert s1.stats["preemptions"] >= 2 and runner.graph_steps > 20
+    assert sum(r.num_preemptions > 0 for r in tight) >= 2
+    for a, b in zip(roomy, tight):
+        assert b.finish_reason == "length" and len(b.output_token_ids) == len(a.output_token_ids)
+        assert_varied(b.output_token_ids)
+        if dtype == "float32" or b.num_preemptions == 0:
+            assert a.output_token_ids == b.output_token_ids, f"request {a.request_id} (preempted {b.num_preemptions} times)"
+
+
+def test_command_line_takes_stop_tokens(varied_folders):
+    """`--stop-token-ids`: the request ends with the first of them that it generates, which is kept
+    (the reference's finishing rule, src/wllm/engine/sequence.py:53-59)."""
+    folder = varied_folders["AV"]
+    cfg, w = plain_model(folder)
+    prompt = random_ids(5, 9, 512)
+    free = gemma_plain.generate_greedy(cfg, w, prompt, 8)
+    stop = free[3]
+    first = free.index(stop)
+    args = [sys.executable, "-m", "wllm_amd.cli", "generate", "--model", folder, "--dtype", "float32", "--num-blocks", "32",
+            "--block-size", "4", "--max-new-tokens", "8", "--prompt-ids", ",".join(str(t) for t in prompt),
+            "--stop-token-ids", f"{stop},511"]
+    proc = subprocess.run(args, capture_output=True, text=True, timeout=300, cwd=ROOT)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    line = [json.loads(l) for l in proc.stdout.splitlines() if l.startswith("{")][0]
+    assert line["token_ids"] == free[:first + 1] and line["finish_reason"] == "stop"
 
 
 def test_command_line_generates_what_the_entry_point_generates(varied_folders, tmp_path):

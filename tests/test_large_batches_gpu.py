@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import (TINY, assert_varied, compare_with_plain, max_live_tokens, random_ids, replay_and_collect,
+from helpers import (TINY, assert_varied, compare_replay, plain_for, max_live_tokens, random_ids, replay_and_collect,
                      trace_mixed)
 from plain import gemma_plain
 from wllm_amd.engine import LLM, ModelRunner
@@ -19,7 +19,13 @@ from wllm_amd.engine.replay import TraceReplayer, pages_for_max_tokens
 from wllm_amd.parts import load_model
 
 pytestmark = pytest.mark.gpu
-TOLERANCE = {"float32": dict(atol=2e-5, rtol=1e-4), "bfloat16": dict(atol=1e-2, rtol=1e-2)}
+_PLAIN = {}      # what the requests are compared with, made once per (model, requests, dtype)
+
+
+def plain_of(key, cfg, folder, requests, dtype):
+    if (key, dtype) not in _PLAIN:
+        _PLAIN[(key, dtype)] = plain_for(cfg, folder, requests, dtype)
+    return _PLAIN[(key, dtype)]
 DECODED = 8
 # live requests -> how many end half way, so that the count crosses the edge of a bucket of
 # (1, 2, 4, 8, 16, 32, 48, 64, 128, 256): 17 -> 15, 48 -> 30, 64 -> 47, 65 -> 63, 130 -> 127
@@ -66,8 +72,7 @@ def models(model_folders):
 
 @pytest.fixture(scope="module")
 def plain_models(model_folders):
-    return {name: (gemma_plain.read_config(model_folders[name]), gemma_plain.read_weights(model_folders[name], torch.float32))
-            for name in ("A", "M")}
+    return {name: (gemma_plain.read_config(model_folders[name]), model_folders[name]) for name in ("A", "M")}
 
 
 @pytest.mark.parametrize("graphs", [False, True])
@@ -77,9 +82,8 @@ def plain_models(model_folders):
 def test_decode_steps_of_many_requests(models, plain_models, name, count, dtype, graphs):
     longest = {"A": 100, "M": 200}[name]
     requests = many_requests(name, count, longest)
-    cfg, w = plain_models[name]
-    rounding = torch.bfloat16 if dtype == "bfloat16" else None
-    plain = {rid: gemma_plain.forward_logits(cfg, w, t, scale_rounding=rounding) for rid, t in requests.items()}
+    cfg, folder = plain_models[name]
+    plain = plain_of((name, count), cfg, folder, requests, dtype)
     trace = decode_trace(requests, DROPS[count])
     page_size = TINY[name]["page_size"]
     pages = pages_for_max_tokens(max_live_tokens(trace, round_to=page_size), page_size) + (1 if graphs else 0)
@@ -97,8 +101,8 @@ def test_decode_steps_of_many_requests(models, plain_models, name, count, dtype,
         assert runner.graph_steps == DECODED
         assert used == sorted({next(b for b in runner.graph_buckets if b >= n) for n in (count, after)}), used
         assert used[-1] > count or count in runner.graph_buckets, "padding rows, unless the batch fills its bucket"
-    worst = compare_with_plain(got, plain, **TOLERANCE[dtype])
-    print(f"{name} {dtype} {count} live, graphs {graphs}: worst error {worst:.3f} x tolerance")
+    worst = compare_replay(got, plain, dtype)
+    print(f"{name} {dtype} {count} live, graphs {graphs}: worst error {worst:.3f} x bound")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -107,9 +111,8 @@ def test_mixed_steps_of_24_live_requests(models, plain_models, dtype):
     vocab = TINY["M"]["config"].vocab_size
     rng = np.random.default_rng(5)
     requests = {f"r{i}": random_ids(300 + i, int(n), vocab) for i, n in enumerate(rng.integers(20, 150, size=40))}
-    cfg, w = plain_models["M"]
-    rounding = torch.bfloat16 if dtype == "bfloat16" else None
-    plain = {rid: gemma_plain.forward_logits(cfg, w, t, scale_rounding=rounding) for rid, t in requests.items()}
+    cfg, folder = plain_models["M"]
+    plain = plain_of("mixed24", cfg, folder, requests, dtype)
     trace = trace_mixed(requests, seed=3, live=24)
     assert max(len(s["entries"]) for s in trace) >= 20
     pages = pages_for_max_tokens(max_live_tokens(trace, round_to=16), 16)
@@ -117,7 +120,7 @@ def test_mixed_steps_of_24_live_requests(models, plain_models, dtype):
     got = replay_and_collect(TraceReplayer(runner), trace)
     runner.cache.check()
     assert len(got) == sum(len(t) for t in requests.values())
-    compare_with_plain(got, plain, **TOLERANCE[dtype])
+    compare_replay(got, plain, dtype)
 
 
 def test_forty_requests_generate_what_the_plain_implementation_generates(varied_folders):

@@ -5,16 +5,13 @@ vocabulary so that the plain implementation stays fast.  The prompts are long en
 attention's work to be cut along the keys (several pieces of 128 keys in decode steps, a late
 portion of a prompt split over workgroups).
 
-float32 is held to the tolerance of the tiny configurations.  The bfloat16 bound here is a second line
-behind the tiny configurations' element-wise one: it shows a wrong page, key or head, not a rounding
-made at another point than the plain implementation makes it.  In bfloat16 an activation of these
-widths is the sum of thousands of rounded terms, so single logits stray further than in the tiny
-models; the measure is each position's error against the length of its logits vector, which a
-missed key, a wrong page or a wrong head would raise to the order of one."""
+float32 is held to the tolerance of the tiny configurations, bfloat16 to the bound that the plain
+implementation's own rounded run sets for each row (helpers.compare_with_bfloat16_bound), as
+everywhere."""
 import pytest
 import torch
 
-from helpers import max_live_tokens, random_ids, replay_and_collect, trace_mixed, trace_portions, trace_tail, trace_whole
+from helpers import compare_replay, max_live_tokens, plain_for, random_ids, replay_and_collect, trace_mixed, trace_portions, trace_tail, trace_whole
 from plain import gemma_plain
 from wllm_amd.config import GemmaConfig
 from wllm_amd.engine import ModelRunner
@@ -33,10 +30,6 @@ SIZES = {
 }
 LENGTHS = [300, 70, 650, 161]
 PAGE_SIZE = 16
-FLOAT32 = dict(atol=2e-5, rtol=1e-4)
-# eight bits of mantissa: a rounding is 2^-9 of a value on average; a position's logits carry those of a
-# handful of activations a layer
-BFLOAT16_ROW_ERROR = 0.01
 
 
 @pytest.fixture(scope="module")
@@ -51,10 +44,7 @@ def plain_logits(folders):
     out = {}
     for name, folder in folders.items():
         cfg = gemma_plain.read_config(folder)
-        w = gemma_plain.read_weights(folder, torch.float32)
-        requests = _requests(name)
-        out[name] = {rounding: {rid: gemma_plain.forward_logits(cfg, w, toks, scale_rounding=rounding)
-                                for rid, toks in requests.items()} for rounding in (None, torch.bfloat16)}
+        out[name] = {dtype: plain_for(cfg, folder, _requests(name), dtype) for dtype in ("float32", "bfloat16")}
     return out
 
 
@@ -66,7 +56,7 @@ def _requests(name):
 @pytest.mark.parametrize("name", list(SIZES))
 def test_layer_sizes_of_the_measured_models(folders, plain_logits, name, dtype):
     requests = _requests(name)
-    plain = plain_logits[name][torch.bfloat16 if dtype == "bfloat16" else None]
+    plain = plain_logits[name][dtype]
     model = load_model(folders[name], dtype, "cuda")
     for family in (trace_whole, trace_tail, trace_portions, trace_mixed):
         trace = family(requests)
@@ -75,16 +65,5 @@ def test_layer_sizes_of_the_measured_models(folders, plain_logits, name, dtype):
         got = replay_and_collect(TraceReplayer(runner), trace)
         runner.cache.check()
         assert len(got) == sum(LENGTHS)
-        worst = 0.0
-        for (rid, pos), row in sorted(got.items()):
-            ref = plain[rid][pos].double()
-            row = row.double()
-            assert torch.isfinite(row).all(), f"{family.__name__}: request {rid!r} position {pos}: logits are not finite"
-            if dtype == "float32":
-                err = ((row - ref).abs() / (FLOAT32["atol"] + FLOAT32["rtol"] * ref.abs())).max().item()
-                assert err <= 1.0, f"{family.__name__}: request {rid!r} position {pos}: {err:.2f} x tolerance"
-            else:
-                err = ((row - ref).norm() / ref.norm()).item()
-                assert err <= BFLOAT16_ROW_ERROR, f"{family.__name__}: request {rid!r} position {pos}: row error {err:.4f}"
-            worst = max(worst, err)
-        print(f"{name} {dtype} {family.__name__}: worst {worst:.4f}")
+        worst = compare_replay(got, plain, dtype)
+        print(f"{name} {dtype} {family.__name__}: worst {worst:.3f} x bound")

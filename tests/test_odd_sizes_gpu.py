@@ -6,7 +6,7 @@ changing size, and mixed portions with pages handed out again, in float32 and in
 import pytest
 import torch
 
-from helpers import (compare_with_plain, max_live_tokens, random_ids, replay_and_collect, trace_mixed, trace_portions,
+from helpers import (compare_replay, plain_for, max_live_tokens, random_ids, replay_and_collect, trace_mixed, trace_portions,
                      trace_tail, trace_whole)
 from plain import gemma_plain
 from wllm_amd.config import GemmaConfig
@@ -33,7 +33,6 @@ ODD = {
     "width_not_4": (cfg(211, 70, 90, 2, 5, 1, 32), 8),
 }
 LENGTHS = [37, 70, 33, 52]
-TOLERANCE = {"float32": dict(atol=2e-5, rtol=1e-4), "bfloat16": dict(atol=1e-2, rtol=1e-2)}
 
 
 @pytest.fixture(scope="module")
@@ -49,10 +48,7 @@ def test_odd_sizes_follow_the_plain_implementation(folders, name, dtype):
     config, page_size = ODD[name]
     requests = {f"r{i}": random_ids(31 * i + len(name), n, config.vocab_size) for i, n in enumerate(LENGTHS)}
     plain_cfg = gemma_plain.read_config(folders[name])
-    weights = gemma_plain.read_weights(folders[name], torch.float32)
-    rounding = torch.bfloat16 if dtype == "bfloat16" else None
-    plain = {rid: gemma_plain.forward_logits(plain_cfg, weights, toks, scale_rounding=rounding)
-             for rid, toks in requests.items()}
+    plain = plain_for(plain_cfg, folders[name], requests, dtype)
     model = load_model(folders[name], dtype, "cuda")
     for family in (trace_whole, trace_tail, trace_portions, trace_mixed):
         trace = family(requests)
@@ -62,4 +58,4 @@ def test_odd_sizes_follow_the_plain_implementation(folders, name, dtype):
         got = replay_and_collect(TraceReplayer(runner), trace)
         runner.cache.check()
         assert len(got) == sum(LENGTHS)
-        compare_with_plain(got, plain, **TOLERANCE[dtype])
+        compare_replay(got, plain, dtype)

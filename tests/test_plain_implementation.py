@@ -323,6 +323,88 @@ def test_biases_are_added_before_the_rotation():
     assert not torch.allclose(got[:, 0], running_mean[:, 0], atol=1e-3), "biases after the rotation would give this"
 
 
+# ---- the bound of the bfloat16 comparisons ---------------------------------------------------------
+def test_the_rounded_run_rounds_and_stays_near_the_exact_one(model_folders):
+    """`round_to=torch.bfloat16` changes every row a little (a few roundings of 2^-9 each) and no row much."""
+    from helpers import plain_exact_and_rounded
+    cfg = P.read_config(model_folders["M"])
+    w = P.read_weights(model_folders["M"], torch.float64)
+    exact, realisations = plain_exact_and_rounded(cfg, w, torch.randint(0, cfg["vocab_size"], (40,)))
+    assert len(realisations) == 4
+    for rounded in realisations:
+        rel = (rounded - exact).pow(2).mean(-1).sqrt() / exact.pow(2).mean(-1).sqrt()
+        assert (rel > 2.0 ** -11).all() and (rel < 0.05).all(), rel
+        assert torch.equal(rounded, rounded.to(torch.bfloat16).double()), "the logits themselves are rounded"
+    # realisations are draws of the same noise: they differ from each other as much as from the exact run
+    assert (realisations[0] - realisations[1]).abs().max() > 0.3 * (realisations[0] - exact).abs().max()
+    # no rounding asked for: the same numbers as before
+    assert torch.equal(P.forward_logits(cfg, w, [1, 2, 3], round_to=None), P.forward_logits(cfg, w, [1, 2, 3]))
+
+
+def test_a_lost_or_foreign_key_that_carries_weight_is_far_beyond_the_bfloat16_bound(model_folders, tmp_path):
+    """The bound of the bfloat16 comparisons is a multiple of the rounded run's own distance from the
+    exact logits.  A fault is no rounding: in a model whose attention is sharp (queries and keys scaled
+    up, as tests/test_engine_gpu.py does), a query that loses the key it weighs most, or sees a key
+    of the future in its place, lands many times the bound away, rounded like everything else.  A key
+    that carries no weight (one of hundreds under flat attention) hides below bfloat16's rounding from
+    any bound; the float32 comparisons, fifty times as narrow as one such key's share, are there for it."""
+    import os
+    from helpers import bfloat16_row_errors, plain_exact_and_rounded
+    from wllm_amd.weights import Checkpoint, write_safetensors
+    src, folder = model_folders["M"], str(tmp_path / "sharp")
+    os.makedirs(folder)
+    ck = Checkpoint(src)
+    tensors = {n: ck.tensor(n) for n in ck.names()}
+    ck.close()
+    for n in tensors:
+        if n.endswith(("q_proj.weight", "k_proj.weight")):
+            tensors[n] = (tensors[n].float() * 6.0).to(torch.bfloat16)
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors)
+    with open(os.path.join(src, "config.json")) as f, open(os.path.join(folder, "config.json"), "w") as g:
+        g.write(f.read())
+    cfg = P.read_config(folder)
+    w = P.read_weights(folder, torch.float64)
+    T = 200
+    toks = torch.randint(0, cfg["vocab_size"], (T,), generator=torch.Generator().manual_seed(5))
+    exact, rounded = plain_exact_and_rounded(cfg, w, toks)
+    # the key each query of layer 0 weighs most, over its heads
+    nh, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    h = P.rms_norm_one_plus_w(P.embed(toks, w["model.embed_tokens.weight"], cfg["hidden_size"]),
+                              w["model.layers.0.input_layernorm.weight"], cfg["rms_norm_eps"])
+    cos, sin = P.rope_cos_sin(torch.arange(T), d, cfg["rope_theta"], torch.float64)
+    q = P.apply_rope((h @ w["model.layers.0.self_attn.q_proj.weight"].T).view(T, nh, d), cos, sin)
+    k = P.apply_rope((h @ w["model.layers.0.self_attn.k_proj.weight"].T).view(T, nkv, d), cos, sin)
+    scores = torch.einsum("qhd,khd->hqk", q, k.repeat_interleave(nh // nkv, 1)) / math.sqrt(d)
+    probs = torch.softmax(scores.masked_fill(~torch.ones(T, T, dtype=torch.bool).tril(), float("-inf")), -1).mean(0)
+    checked = 0
+    # the four late queries whose heads agree most on one key
+    late = sorted(range(50, T), key=lambda i: -float(probs[i].max()))[:4]
+    for p_ in late:
+        top = int(probs[p_].argmax())
+        assert probs[p_, top] > 0.2, "the attention is sharp"
+
+        def lose(layer, allowed, p_=p_, top=top):
+            if layer == 0:
+                allowed = allowed.clone()
+                allowed[p_, top] = False
+            return allowed
+
+        bad = P.forward_logits(cfg, w, toks, round_to=torch.bfloat16, tamper=lose)
+        assert max(bfloat16_row_errors(bad[p_], exact[p_], [r[p_] for r in rounded])) > 4.0, (p_, top)
+        # the rows before it are the rounded run's own and within the bound
+        assert max(bfloat16_row_errors(bad[p_ - 1], exact[p_ - 1], [r[p_ - 1] for r in rounded])) <= 1.0
+        checked += 1
+    # a key of the future (a stale slot of the page): a query early enough for one key to move it
+    def foreign(layer, allowed):
+        if layer == 0:
+            allowed = allowed.clone()
+            allowed[3, 4:40] = True
+        return allowed
+    bad = P.forward_logits(cfg, w, toks, round_to=torch.bfloat16, tamper=foreign)
+    assert max(bfloat16_row_errors(bad[3], exact[3], [r[3] for r in rounded])) > 4.0
+    assert checked == 4
+
+
 def test_head_dim_key_wins_over_the_derived_value(tmp_path):
     # the reference's own vector: 3072 / 16 gives 192, the key says 256
     # (tests/test_gemma_architecture.py:40-60)

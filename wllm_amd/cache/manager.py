@@ -140,7 +140,14 @@ class CacheManager:
         for entry, need in (state_shapes or {}).items():
             if not isinstance(need, StateNeed):
                 need = StateNeed(tuple(need))
-            self.state[entry] = torch.zeros((max_requests,) + tuple(need.shape), dtype=need.dtype, device=device)
+            # one row more than there are requests: `padding_slot`, for the rows of a captured graph
+            # that stand for no request (they read and write it, and nobody else does)
+            self.state[entry] = torch.zeros((max_requests + 1,) + tuple(need.shape), dtype=need.dtype, device=device)
+
+    @property
+    def padding_slot(self) -> int:
+        """The state row set aside for rows of a batch that belong to no request."""
+        return self.max_requests
 
     # ---- requests ----------------------------------------------------------
     def open(self, request) -> int:

@@ -66,7 +66,9 @@ def cmd_generate(args) -> int:
     sp = SamplingParams(temperature=args.temperature, top_k=args.top_k, top_p=args.top_p, min_p=args.min_p,
                         repetition_penalty=args.repetition_penalty, seed=args.seed)
     llm = _llm(args)
-    outs = llm.generate(prompts, sp, max_new_tokens=args.max_new_tokens, eos_token_id=args.eos_token_id)
+    stops = [int(t) for t in (args.stop_token_ids or "").split(",") if t.strip()]
+    outs = llm.generate(prompts, sp, max_new_tokens=args.max_new_tokens, eos_token_id=args.eos_token_id,
+                        stop_token_ids=stops)
     for o in outs:
         print(json.dumps({"prompt_token_ids": o.prompt_token_ids, "token_ids": o.token_ids,
                           "finish_reason": o.finish_reason}))
@@ -140,6 +142,8 @@ def main(argv=None) -> int:
     g.add_argument("--repetition-penalty", type=float, default=1.0)
     g.add_argument("--seed", type=int, default=None)
     g.add_argument("--eos-token-id", type=int, default=None)
+    # the reference's finishing rule takes a set of stop tokens beside the end token (src/wllm/engine/sequence.py:53-59)
+    g.add_argument("--stop-token-ids", default=None, help="comma-separated token ids that end a request (the token is kept)")
     g.set_defaults(func=cmd_generate)
 
     r = sub.add_parser("random-model", help="write a model folder with seeded random weights")

@@ -119,6 +119,27 @@ __device__ __forceinline__ float stack_sum(const float* __restrict__ p, int spli
 // rescaling, which a probability does not need.
 __device__ __forceinline__ float exp2_probability(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// The activations of a gated feed-forward, by the number the host passes (the table `ACTIVATIONS` of
+// the Python side holds the same numbers): every kernel that applies one goes through `activate`,
+// so a new activation is one line here, one there, and a case in `WLLM_BY_ACTIVATION`.
+constexpr int kActGeluTanh = 0;      // 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
+constexpr int kActSilu = 1;          // z / (1 + exp(-z))
+constexpr int kActivations = 2;
+
+template <int ACT>
+__device__ __forceinline__ float activate(float z) {
+    static_assert(ACT >= 0 && ACT < kActivations, "unknown activation");
+    if (ACT == kActGeluTanh) return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    return z / (1.f + expf(-z));
+}
+
+// Runs `statement` with the compile-time constant ACT set to the activation's number.
+#define WLLM_BY_ACTIVATION(activation, statement)                                     \
+    switch (activation) {                                                              \
+        case kActGeluTanh: { constexpr int ACT = kActGeluTanh; statement; } break;     \
+        default: { constexpr int ACT = kActSilu; statement; } break;                   \
+    }
+
 // One rotated pair (a, b) -> (a cos - b sin, b cos + a sin).  The products are fused in one fixed
 // way, so that every kernel that rotates gives the same bits for the same numbers.
 __device__ __forceinline__ void rotate_pair(float a, float b, float s, float c, float& ra, float& rb) {

@@ -424,12 +424,6 @@ WLLM_API int wllm_rope_cache_write(void* qkv, int is_bf16, const float* parts, i
 }
 
 // ---- gated activation: out = act(g) * u with g, u the two halves of a row -----------------------
-__device__ __forceinline__ float gelu_tanh(float z) {
-    // 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
-    const float k = 0.7978845608028654f;
-    return 0.5f * z * (1.f + tanhf(k * (z + 0.044715f * z * z * z)));
-}
-__device__ __forceinline__ float silu(float z) { return z / (1.f + expf(-z)); }
 
 template <typename T, int ACT>
 __global__ void gated_activation_kernel(const T* __restrict__ gate_up, T* __restrict__ out, long long total,
@@ -440,7 +434,7 @@ __global__ void gated_activation_kernel(const T* __restrict__ gate_up, T* __rest
         const int c = static_cast<int>(i % inter);
         const float g = to_float(gate_up[r * 2 * inter + c]);
         const float u = to_float(gate_up[r * 2 * inter + inter + c]);
-        out[i] = from_float<T>((ACT == 0 ? gelu_tanh(g) : silu(g)) * u);
+        out[i] = from_float<T>(activate<ACT>(g) * u);
     }
 }
 
@@ -463,7 +457,7 @@ gated_activation_bf16x8_kernel(const bf16* __restrict__ gate_up, bf16* __restric
             for (int k = 0; k < 4; ++k) {
                 const float g0 = __uint_as_float(gw[k] << 16), g1 = __uint_as_float(gw[k] & 0xffff0000u);
                 const float u0 = __uint_as_float(uw[k] << 16), u1 = __uint_as_float(uw[k] & 0xffff0000u);
-                ow[k] = pack2_bf16((ACT == 0 ? gelu_tanh(g0) : silu(g0)) * u0, (ACT == 0 ? gelu_tanh(g1) : silu(g1)) * u1);
+                ow[k] = pack2_bf16(activate<ACT>(g0) * u0, activate<ACT>(g1) * u1);
             }
             *reinterpret_cast<uint4*>(dst + v * 8) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
         }
@@ -472,27 +466,21 @@ gated_activation_bf16x8_kernel(const bf16* __restrict__ gate_up, bf16* __restric
 
 WLLM_API int wllm_gated_activation(const void* gate_up, void* out, int is_bf16, int activation, int n, int inter,
                                    hipStream_t stream) {
+    if (activation < 0 || activation >= kActivations) return -1;
     const long long total = static_cast<long long>(n) * inter;
     if (is_bf16 && inter % 8 == 0) {
         const int vecs = inter / 8;
         const dim3 grid(vecs < 2048 ? (vecs + 255) / 256 : 8, n < 16384 ? n : 16384);
-        if (activation == 0)
-            gated_activation_bf16x8_kernel<0><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(gate_up),
-                                                                        static_cast<bf16*>(out), n, inter);
-        else
-            gated_activation_bf16x8_kernel<1><<<grid, 256, 0, stream>>>(static_cast<const bf16*>(gate_up),
-                                                                        static_cast<bf16*>(out), n, inter);
+        WLLM_BY_ACTIVATION(activation, (gated_activation_bf16x8_kernel<ACT><<<grid, 256, 0, stream>>>(
+                                           static_cast<const bf16*>(gate_up), static_cast<bf16*>(out), n, inter)));
         return launch_status();
     }
     long long blocks = (total + 255) / 256;
     if (blocks > 65536) blocks = 65536;
-#define LAUNCH(T, A)                                                                                              \
-    gated_activation_kernel<T, A><<<static_cast<int>(blocks), 256, 0, stream>>>(static_cast<const T*>(gate_up), \
-                                                                                static_cast<T*>(out), total, inter)
-    if (is_bf16 && activation == 0) LAUNCH(bf16, 0);
-    else if (is_bf16) LAUNCH(bf16, 1);
-    else if (activation == 0) LAUNCH(float, 0);
-    else LAUNCH(float, 1);
+#define LAUNCH(T)                                                                                                   \
+    WLLM_BY_ACTIVATION(activation, (gated_activation_kernel<T, ACT><<<static_cast<int>(blocks), 256, 0, stream>>>( \
+                                       static_cast<const T*>(gate_up), static_cast<T*>(out), total, inter)))
+    if (is_bf16) { LAUNCH(bf16); } else { LAUNCH(float); }
 #undef LAUNCH
     return launch_status();
 }

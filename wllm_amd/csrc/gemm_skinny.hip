@@ -333,10 +333,6 @@ WLLM_API int wllm_gemm_skinny(const void* x, const void* w, int tiled, void* out
 // A wavefront streams 16 gate rows and the 16 up rows that belong to them; both results land
 // in the same lanes, so the activation and the product are made in registers and only [M, I]
 // is written.
-__device__ __forceinline__ float act_gelu_tanh(float z) {
-    return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
-}
-__device__ __forceinline__ float act_silu(float z) { return z / (1.f + expf(-z)); }
 
 // A workgroup is TPW tiles of 16 gate rows (with their up rows) times 2 halves of the K axis; the
 // halves are added through shared memory in a fixed order before the activation.  A workgroup is 2
@@ -536,7 +532,7 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, NormOnLoad norm, const bf16
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const float gate = accg[t][v] + red[t * 8 + v], upv = accu[t][v] + red[t * 8 + 4 + v];
-            r[v] = (ACT == 0 ? act_gelu_tanh(gate) : act_silu(gate)) * upv;
+            r[v] = activate<ACT>(gate) * upv;
         }
         bf16* o = out + static_cast<size_t>(m) * inter + n;
         if (n + 3 < inter && (inter % 4 == 0)) {
@@ -551,7 +547,7 @@ gemm_skinny_gated_kernel(const bf16* __restrict__ x, NormOnLoad norm, const bf16
 
 static int gated_launch(const void* x, NormOnLoad norm, bool with_norm, const void* w, int tiled, void* out, int M,
                         int inter, int K, int activation, int chunk, hipStream_t stream) {
-    if (M < 1 || M > 64 || K % 64 != 0 || chunk % 32 != 0 || activation < 0 || activation > 1) return -1;
+    if (M < 1 || M > 64 || K % 64 != 0 || chunk % 32 != 0 || activation < 0 || activation >= kActivations) return -1;
     const int mt = (M + 15) / 16;
     if (chunk > K / 2) chunk = K / 2;
     // the norm on load: at most 16 rows, whole chunks of 256 keys
@@ -598,9 +594,9 @@ static int gated_launch(const void* x, NormOnLoad norm, bool with_norm, const vo
         default: LAUNCH(4, A); break; \
     }
     if (with_norm) {
-        if (activation == 0) { LAUNCH_N(0) } else { LAUNCH_N(1) }
+        WLLM_BY_ACTIVATION(activation, LAUNCH_N(ACT))
     } else {
-        if (activation == 0) { BY_MT(0) } else { BY_MT(1) }
+        WLLM_BY_ACTIVATION(activation, BY_MT(ACT))
     }
 #undef BY_MT
 #undef LAUNCH_N

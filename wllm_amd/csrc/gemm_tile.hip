@@ -49,12 +49,8 @@ static __device__ __forceinline__ void load_to_shared(const void* base, uint32_t
                  : "=&s"(saved_m0) : "v"(offset), "s"(base), "s"(lds_address) : "memory");
 }
 
-static __device__ __forceinline__ float tile_gelu_tanh(float z) {
-    return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
-}
-static __device__ __forceinline__ float tile_silu(float z) { return z / (1.f + expf(-z)); }
 
-// GATED: 0 plain, 1 gelu_tanh, 2 silu.  N is the number of rows of w (plain) or of gate rows (gated).
+// GATED: 0 plain, 1 + the activation's number for the gated product.  N is the number of rows of w (plain) or of gate rows (gated).
 // (Tiles of 256 rows of x with eight wavefronts were no faster: the rate is set by the reads of
 // fragments from shared memory, which take as long as the products they feed.)
 // STAGES: how many stages' tiles shared memory holds.  Two, and two workgroups a compute unit, as
@@ -176,7 +172,7 @@ gemm_tile_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, bf16* _
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     const float gate = acc[a][b][v], up = acc[a + 2][b][v];
-                    r[v] = (GATED == 1 ? tile_gelu_tanh(gate) : tile_silu(gate)) * up;
+                    r[v] = activate<(GATED > 0 ? GATED - 1 : 0)>(gate) * up;
                 }
                 bf16* o = out + static_cast<size_t>(m) * N + n;
                 if (n + 3 < N && N % 4 == 0) {
@@ -223,13 +219,13 @@ gemm_tile_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w, bf16* _
     }
 }
 
-// out[M, N] = x . w^T (activation 0, w [N, K]), or the gated product (activation 1: gelu_tanh, 2:
-// silu; w [2N, K], gate rows first).  splits > 1 (plain only): `out` is null and `partial` float32
+// out[M, N] = x . w^T (gated 0, w [N, K]), or the gated product (gated = 1 + the activation's number;
+// w [2N, K], gate rows first).  splits > 1 (plain only): `out` is null and `partial` float32
 // [splits, M, N] takes the pieces' sums.  K must be a multiple of 64 * splits and the operands smaller
 // than 4 GiB.  Returns 0, a HIP error code, or -1 for sizes it does not take.
 WLLM_API int wllm_gemm_tile(const void* x, const void* w, void* out, float* partial, int M, int N, int K, int splits,
                             int activation, hipStream_t stream) {
-    if (M < 1 || N < 1 || K < kStageKeys || splits < 1 || K % (kStageKeys * splits) != 0 || activation < 0 || activation > 2)
+    if (M < 1 || N < 1 || K < kStageKeys || splits < 1 || K % (kStageKeys * splits) != 0 || activation < 0 || activation > kActivations)
         return -1;
     if ((splits > 1) != (partial != nullptr) || (splits == 1 && out == nullptr) || (splits > 1 && activation != 0)) return -1;
     const size_t w_rows = static_cast<size_t>(activation ? 2 : 1) * N;
@@ -270,8 +266,7 @@ WLLM_API int wllm_gemm_tile(const void* x, const void* w, void* out, float* part
     if (deep) LAUNCH(GATED, 4);         \
     else LAUNCH(GATED, 2)
     if (activation == 0) { BY_STAGES(0); }
-    else if (activation == 1) { BY_STAGES(1); }
-    else { BY_STAGES(2); }
+    else { WLLM_BY_ACTIVATION(activation - 1, BY_STAGES(ACT + 1)) }
 #undef BY_STAGES
 #undef LAUNCH
     return launch_status();

@@ -1,7 +1,6 @@
 // An entry point of the kernel library that allocates nothing.
 //
-// It has no counterpart in the reference (Sehastrajit-S/wLLM samples with torch operations, each of
-// which may allocate, src/wllm/engine/sampling.py:101-143).  It is for callers that cannot call
+// It has no counterpart in the reference.  It is for callers that cannot call
 // hipMalloc: code under HIP graph capture, tight serving loops that must not touch the allocator,
 // harnesses that forbid allocation.  The caller passes inputs and outputs; everything else the
 // kernels need lives in a device array that is part of the library's image.

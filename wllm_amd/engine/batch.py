@@ -98,28 +98,34 @@ class StepContext:
         self.requests = requests
         self.max_q_len = int(host_q_len.max()) if num_segments else 0
         self.max_ctx_len = int(host_ctx_len.max()) if num_segments else 0
-        self._attention_plans: dict = {}
-        # set by a captured graph: plans of fixed shape, refreshed in place before each replay
-        self.static_plans = False
-        self.static_max_context = 0
-        self.static_max_total_keys = 0
+        self._plans: dict = {}             # key -> (plan, refresh)
+        # set by a captured graph: its kernels hold the addresses of what a part makes for the step, so
+        # a plan has a fixed shape, sized by these limits, and is rewritten in place before each replay
+        self.captured = False
+        self.capture_max_context = 0       # the longest context of a request the graph takes
+        self.capture_max_tokens = 0        # the most tokens all its requests hold together (the pool's)
 
-    def attention_plan(self, *, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, window: int):
-        """The step's work items for attention of this shape; made once, shared by all layers."""
-        from wllm_amd.kernels import ops
-        key = (num_heads, num_kv_heads, head_dim, page_size, window)
-        if key not in self._attention_plans and self.static_plans:
-            plan = ops.backend().static_attention_plan(
-                self.num_segments, num_heads, num_kv_heads, head_dim, page_size, window, self.dtype, self.device,
-                self.static_max_context, self.static_max_total_keys)
-            if plan is not None:
-                plan.update(self.host_q_len, self.host_ctx_len)
-            self._attention_plans[key] = plan
-        if key not in self._attention_plans:
-            self._attention_plans[key] = ops.plan_paged_attention(
-                self.host_q_len, self.host_ctx_len, num_heads=num_heads, num_kv_heads=num_kv_heads,
-                head_dim=head_dim, page_size=page_size, window=window, dtype=self.dtype, device=self.device)
-        return self._attention_plans[key]
+    def plan(self, key, build, refresh=None):
+        """What a part prepares on the host for a step (work items, a routing table, the chunks of a
+        scan), made once per step and `key` and shared by every layer that asks under the same key.
+        `build(ctx)` makes it from the step's host arrays (`host_q_len`, `host_ctx_len`, ...) and may
+        return None.  In a captured graph (`ctx.captured`) `build` runs once, when the graph is first
+        run, and makes a plan of fixed shape in device memory sized by `capture_max_context` and
+        `capture_max_tokens`; `refresh(plan, ctx)` then rewrites its contents in place before every
+        replay, the first included.  A part whose plan needs a refresh and gives none cannot be
+        captured."""
+        if key not in self._plans:
+            made = build(self)
+            self._plans[key] = (made, refresh)
+            if self.captured and made is not None and refresh is not None:
+                refresh(made, self)
+        return self._plans[key][0]
+
+    def refresh_plans(self) -> None:
+        """Before a replay of the captured graph: every plan takes the step's contents."""
+        for made, refresh in self._plans.values():
+            if made is not None and refresh is not None:
+                refresh(made, self)
 
     def buffer(self, name: str, shape: tuple, dtype: torch.dtype) -> torch.Tensor:
         return self._workspace.get(name, shape, dtype)

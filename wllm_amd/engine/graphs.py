@@ -78,9 +78,9 @@ class DecodeGraph:
             host_ctx_len=np.ones(b, dtype=np.int32), host_state_slots=np.zeros(b, dtype=np.int32),
             requests=[None] * b)
         self.ctx.max_q_len, self.ctx.max_ctx_len = 1, max_context
-        self.ctx.static_plans = True
-        self.ctx.static_max_context = max_context
-        self.ctx.static_max_total_keys = max(g_.pool.num_pages for g_ in cache.groups) * cache.page_size
+        self.ctx.captured = True
+        self.ctx.capture_max_context = max_context
+        self.ctx.capture_max_tokens = max(g_.pool.num_pages for g_ in cache.groups) * cache.page_size
         self.graph = None
         self.logits = None
         self._copied = torch.cuda.Event()
@@ -107,7 +107,7 @@ class DecodeGraph:
         cl[:n] = old + 1
         cl[n:] = 1
         st[:n] = [cache.slot(e.request) for e in entries]
-        st[n:] = 0
+        st[n:] = cache.padding_slot         # a state row that belongs to no request
         rows[:] = np.arange(b)
         for gi in range(g):
             slots = self._field(8 + gi)
@@ -128,23 +128,24 @@ class DecodeGraph:
         self.ctx.host_ctx_len = cl.copy()
         self.ctx.host_state_slots = st.copy()
         self.ctx.requests = [e.request for e in entries] + [None] * (b - n)
-        for plan in self.ctx._attention_plans.values():
-            if plan is not None:
-                plan.update(self.ctx.host_q_len, self.ctx.host_ctx_len)
+        self.ctx.refresh_plans()
         self.dev.copy_(self.host, non_blocking=True)
         self._copied.record()
         self._in_flight = True
 
     def run(self, entries: list, reserved: list, feed_tokens=None) -> torch.Tensor:
-        self.fill(entries, reserved)
-        if feed_tokens is not None:
-            # outside the captured graph: the tensor of sampled tokens is not the graph's own
-            ops.feed_tokens(self.ctx.token_ids, self._feed_dst, self._feed_src, feed_tokens)
         if self.graph is None:
-            # once eagerly: scratch tensors and plans come into being, lazy library state settles
+            # Once eagerly, so that scratch tensors and plans come into being and lazy library state
+            # settles, with every row a padding row: the run before the capture must leave no trace in
+            # a request's pages or state (a mixer that updates a state would update it twice).
+            self.fill([], [])
             self.runner.model.forward(self.ctx)
             torch.cuda.synchronize()
             self.graph, self.logits = capture(lambda: self.runner.model.forward(self.ctx))
             self.workspace.freeze()
+        self.fill(entries, reserved)
+        if feed_tokens is not None:
+            # outside the captured graph: the tensor of sampled tokens is not the graph's own
+            ops.feed_tokens(self.ctx.token_ids, self._feed_dst, self._feed_src, feed_tokens)
         self.graph.replay()
         return self.logits[:len(entries)]

@@ -10,6 +10,8 @@ import numpy as np
 import torch
 
 from wllm_amd.kernels.attention_plan import AttentionPlan, build_work_items
+from wllm_amd.kernels import ops
+from wllm_amd.kernels.ops import ACTIVATIONS
 from wllm_amd.kernels.library import load
 from wllm_amd.kernels.staging import pack_int32
 
@@ -30,8 +32,6 @@ _SIGNATURES = {
     "wllm_gemm_residual": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "wllm_qkv_rope": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong,
                       c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
-    "wllm_feed_tokens": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
-    "wllm_embed_lookup": [c_void_p, c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
     "wllm_rms_norm": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                       c_float, c_float, c_void_p],
     "wllm_rope_cache_write": [c_void_p, c_int, c_void_p, c_int, c_longlong, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -40,7 +40,6 @@ _SIGNATURES = {
     "wllm_gemm_skinny_gated_norm": [c_void_p, c_void_p, c_int, c_void_p, c_float, c_float, c_void_p, c_int, c_void_p, c_int,
                                     c_int, c_int, c_int, c_void_p],
     "wllm_tile_weight": [c_void_p, c_void_p, c_int, c_int, c_void_p],
-    "wllm_gated_activation": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_paged_attention_generic": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                      c_float, c_int, c_void_p],
@@ -77,6 +76,7 @@ class HipBackend:
         self._sample_scratch = None
         self._partial_ml = None
         self._generic_partial_o = None
+        self._registered: dict = {}
         for name, argtypes in _SIGNATURES.items():
             fn = getattr(self.lib, name)
             fn.argtypes = argtypes
@@ -101,16 +101,18 @@ class HipBackend:
         if code != 0:
             raise KernelError(f"{what}: HIP error {code}")
 
-    def embed_lookup(self, ids, table, scale, out):
-        self._on_gpu(ids, table, out)
-        self._check(self.lib.wllm_embed_lookup(_ptr(ids), _ptr(table), int(table.dtype == torch.bfloat16), scale,
-                                               _ptr(out), ids.shape[0], table.shape[1], table.shape[0],
-                                               self._stream()), "embed_lookup")
-
-    def feed_tokens(self, ids, dst, src, source):
-        self._on_gpu(ids, dst, src, source)
-        self._check(self.lib.wllm_feed_tokens(_ptr(ids), _ptr(dst), _ptr(src), _ptr(source), dst.shape[0], ids.shape[0],
-                                              source.shape[0], self._stream()), "feed_tokens")
+    def run_registered(self, op, args, kwargs) -> None:
+        """An operation that a part registered (`ops.register_op`): its entry point is looked up once in
+        its library, given its signature, and launched on the current stream."""
+        fn = self._registered.get(op.name)
+        if fn is None or fn[0] is not op:
+            lib = op.library() if op.library is not None else self.lib
+            entry = getattr(lib, op.entry_point)
+            entry.argtypes = op.argtypes
+            entry.restype = c_int
+            fn = self._registered[op.name] = (op, entry)
+        self._on_gpu(*[a for a in list(args) + list(kwargs.values()) if isinstance(a, torch.Tensor)])
+        self._check(op.launch(fn[1], self._stream(), *args, **kwargs), op.name)
 
     def rms_norm(self, x, weight, eps, offset, out, delta, rows):
         self._on_gpu(x, weight, out, delta, rows)
@@ -405,7 +407,7 @@ class HipBackend:
         w, tiled = (tiles, 1) if tiles is not None else (weight, 0)
         if self.skinny_takes(x.dtype, m, k) and k % 64 == 0:
             self._check(self.lib.wllm_gemm_skinny_gated(
-                _ptr(x), _ptr(w), tiled, _ptr(out), m, out.shape[1], k, 0 if activation == "gelu_tanh" else 1,
+                _ptr(x), _ptr(w), tiled, _ptr(out), m, out.shape[1], k, ACTIVATIONS[activation],
                 self.GATED_CHUNK[-(-m // 16)], self._stream()), "gated_linear (few rows, matrix cores)")
             return
         n = out.shape[1]
@@ -413,11 +415,11 @@ class HipBackend:
                 and max(m, 2 * n) * k * 2 < 2 ** 32):
             # some hundred rows: the tiled product with the activation in its registers
             self._check(self.lib.wllm_gemm_tile(_ptr(x), _ptr(weight), _ptr(out), None, m, n, k, 1,
-                                                1 if activation == "gelu_tanh" else 2, self._stream()),
+                                                1 + ACTIVATIONS[activation], self._stream()),
                         "gated_linear (tiles)")
             return
         self.linear(x, weight, scratch)
-        self.gated_activation(scratch, out, activation)
+        ops.call("gated_activation", scratch, out, activation)
 
     @staticmethod
     def gated_linear_norm_takes(rows: int, dtype, in_features: int) -> bool:
@@ -430,14 +432,8 @@ class HipBackend:
         w, tiled = (tiles, 1) if tiles is not None else (weight, 0)
         self._check(self.lib.wllm_gemm_skinny_gated_norm(
             _ptr(x.residual), _ptr(x.sumsq), x.sumsq.shape[1], _ptr(x.weight), x.eps, x.offset, _ptr(w), tiled,
-            _ptr(out), x.shape[0], out.shape[1], x.shape[1], 0 if activation == "gelu_tanh" else 1, self._stream()),
+            _ptr(out), x.shape[0], out.shape[1], x.shape[1], ACTIVATIONS[activation], self._stream()),
             "gated_linear (norm on load)")
-
-    def gated_activation(self, gate_up, out, activation):
-        self._on_gpu(gate_up, out)
-        self._check(self.lib.wllm_gated_activation(
-            _ptr(gate_up), _ptr(out), int(gate_up.dtype == torch.bfloat16), 0 if activation == "gelu_tanh" else 1,
-            gate_up.shape[0], out.shape[1], self._stream()), "gated_activation")
 
     ARGMAX_ROWS = 4096       # rows per launch; the scratch (64 words a row) is allocated once
 

@@ -35,18 +35,22 @@ class KernelLibraryMissing(RuntimeError):
     """The kernel library is not built and cannot be built here."""
 
 
-def sources() -> list:
-    return sorted(f for f in os.listdir(SOURCE_DIR) if f.endswith(".hip"))
+def sources(source_dir: str = SOURCE_DIR) -> list:
+    return sorted(f for f in os.listdir(source_dir) if f.endswith(".hip"))
 
 
-def _fingerprint() -> str:
+def _fingerprint(source_dir: str = SOURCE_DIR) -> str:
+    """Of the flags and of every source and header of the folder (and, for a folder of kernels that
+    is not the framework's own, of the framework's headers it may include)."""
     h = hashlib.sha256()
     h.update(" ".join(FLAGS).encode())
-    for name in sorted(os.listdir(SOURCE_DIR)):
-        if name.endswith((".hip", ".h")):
-            h.update(name.encode())
-            with open(os.path.join(SOURCE_DIR, name), "rb") as f:
-                h.update(f.read())
+    folders = [source_dir] if os.path.samefile(source_dir, SOURCE_DIR) else [source_dir, SOURCE_DIR]
+    for folder in folders:
+        for name in sorted(os.listdir(folder)):
+            if name.endswith(".h") or (folder == source_dir and name.endswith(".hip")):
+                h.update(name.encode())
+                with open(os.path.join(folder, name), "rb") as f:
+                    h.update(f.read())
     return h.hexdigest()
 
 
@@ -70,11 +74,13 @@ def _writable(folder: str) -> bool:
         return False
 
 
-def _locations(fingerprint: str) -> list:
-    """(library path, object folder) candidates, in-tree first."""
+def _locations(fingerprint: str, source_dir: str = SOURCE_DIR, library_name: str = LIBRARY_NAME) -> list:
+    """(library path, object folder) candidates, beside the sources first (the framework's own
+    library lies in the package folder, one level above its sources)."""
     fallback = os.path.join(tempfile.gettempdir(), f"wllm_amd_build_{os.getuid()}_{fingerprint[:16]}")
-    return [(os.path.join(PACKAGE_DIR, LIBRARY_NAME), os.path.join(SOURCE_DIR, "_build")),
-            (os.path.join(fallback, LIBRARY_NAME), os.path.join(fallback, "obj"))]
+    beside = PACKAGE_DIR if os.path.samefile(source_dir, SOURCE_DIR) else source_dir
+    return [(os.path.join(beside, library_name), os.path.join(source_dir, "_build")),
+            (os.path.join(fallback, library_name), os.path.join(fallback, "obj"))]
 
 
 def _is_current(lib_path: str, fingerprint: str) -> bool:
@@ -85,20 +91,21 @@ def _is_current(lib_path: str, fingerprint: str) -> bool:
         return f.read().strip() == fingerprint
 
 
-def build(verbose: bool = True, force: bool = True) -> str:
-    """Compiles every source for gfx950 and links the library; returns its path."""
-    fingerprint = _fingerprint()
+def build(verbose: bool = True, force: bool = True, source_dir: str = SOURCE_DIR, library_name: str = LIBRARY_NAME) -> str:
+    """Compiles every source of the folder for gfx950 and links the library; returns its path.
+    The framework's headers are on the include path of any folder."""
+    fingerprint = _fingerprint(source_dir)
     hipcc = _hipcc()
     lib_path = obj_dir = None
-    for cand_lib, cand_obj in _locations(fingerprint):
+    for cand_lib, cand_obj in _locations(fingerprint, source_dir, library_name):
         if _writable(os.path.dirname(cand_lib)) and _writable(cand_obj):
             lib_path, obj_dir = cand_lib, cand_obj
             break
     if lib_path is None:
-        raise KernelLibraryMissing("no writable place for the kernel library (package folder and temporary folder)")
+        raise KernelLibraryMissing("no writable place for the kernel library (beside its sources and the temporary folder)")
     if not force and _is_current(lib_path, fingerprint):
         return lib_path
-    names = sources()
+    names = sources(source_dir)
     env = dict(os.environ)
     env.setdefault("TMPDIR", tempfile.gettempdir())
     t0 = time.time()
@@ -107,11 +114,11 @@ def build(verbose: bool = True, force: bool = True) -> str:
         if verbose:
             print(f"[wllm_amd build] {msg}", file=sys.stderr, flush=True)
 
-    say(f"compiling {len(names)} kernel files for {ARCH} with {hipcc}")
+    say(f"compiling {len(names)} kernel files of {source_dir} for {ARCH} with {hipcc}")
 
     def compile_one(name: str):
         obj = os.path.join(obj_dir, name[:-4] + ".o")
-        cmd = [hipcc] + FLAGS + ["-I", SOURCE_DIR, "-c", os.path.join(SOURCE_DIR, name), "-o", obj]
+        cmd = [hipcc] + FLAGS + ["-I", source_dir, "-I", SOURCE_DIR, "-c", os.path.join(source_dir, name), "-o", obj]
         r = subprocess.run(cmd, capture_output=True, text=True, env=env)
         return name, obj, r
 
@@ -134,25 +141,29 @@ def build(verbose: bool = True, force: bool = True) -> str:
     return lib_path
 
 
-_loaded = None
+_loaded: dict = {}
 
 
-def load(verbose: bool = True) -> ctypes.CDLL:
-    """The loaded library; built first when no build of the present sources exists."""
-    global _loaded
-    if _loaded is not None:
-        return _loaded
-    fingerprint = _fingerprint()
+def load(verbose: bool = True, source_dir: str = SOURCE_DIR, library_name: str = LIBRARY_NAME) -> ctypes.CDLL:
+    """The loaded library of a folder of kernels (the framework's own by default); built first when
+    no build of the present sources exists.  A part that brings kernels of its own keeps them in a
+    folder of `.hip` files and loads them with `load(source_dir=..., library_name=...)`: the same
+    compiler flags, the framework's headers on the include path, the library beside the sources."""
+    key = (os.path.realpath(source_dir), library_name)
+    if key in _loaded:
+        return _loaded[key]
+    fingerprint = _fingerprint(source_dir)
     path = None
-    for cand_lib, _ in _locations(fingerprint):
+    for cand_lib, _ in _locations(fingerprint, source_dir, library_name):
         if _is_current(cand_lib, fingerprint):
             path = cand_lib
             break
     if path is None:
-        path = build(verbose=verbose)
+        path = build(verbose=verbose, source_dir=source_dir, library_name=library_name)
     try:
-        _loaded = ctypes.CDLL(path)
+        lib = ctypes.CDLL(path)
     except OSError as e:
         raise KernelLibraryMissing(f"{path} cannot be loaded: {e}") from e
-    _loaded.wllm_path = path
-    return _loaded
+    lib.wllm_path = path
+    _loaded[key] = lib
+    return lib

@@ -66,6 +66,58 @@ def _dense(t: torch.Tensor, name: str, dtype, shape=None) -> None:
         raise KernelShapeError(f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
 
 
+# ---- operations that parts bring with them ------------------------------------------------------
+class RegisteredOp:
+    """An operation added by `register_op`: a kernel of a library of its own (or of the framework's)
+    with its host-side check, its launch and, for tests without a GPU, its plain emulation."""
+
+    def __init__(self, name, entry_point, argtypes, launch, check, emulate, library):
+        self.name, self.entry_point, self.argtypes = name, entry_point, list(argtypes)
+        self.launch, self.check, self.emulate, self.library = launch, check, emulate, library
+
+
+_REGISTERED: dict = {}
+
+
+def register_op(name: str, *, entry_point: str, argtypes, launch, check=None, emulate=None, library=None,
+                replace: bool = False) -> RegisteredOp:
+    """Adds an operation without a change to this package: a new part's kernel is a `.hip` file and a
+    Python file of the part's own.
+
+    entry_point, argtypes: the `extern "C"` function (returning 0, a HIP error code, or -1 for sizes it
+        does not take) and its ctypes signature, the stream last.
+    library: a function that returns the loaded library holding it (`library.load(source_dir=...)` of a
+        folder of kernels), or None for the framework's own library.
+    check(*args, **kwargs): raises `KernelShapeError` unless shapes, dtypes and layouts are what the kernel
+        and its grid assume; it runs on the host before every launch.
+    launch(fn, stream, *args, **kwargs) -> int: calls `fn` with raw pointers (`ops.pointer(tensor)`) and the stream.
+    emulate(*args, **kwargs): the same contract in plain torch, for the tests that run the engine's
+        bookkeeping without a GPU; never used by the engine.
+
+    `ops.call(name, ...)` then checks the operands and launches on the stream of the step."""
+    if name in _REGISTERED and not replace:
+        raise ValueError(f"operation {name!r} is already registered")
+    op = RegisteredOp(name, entry_point, argtypes, launch, check, emulate, library)
+    _REGISTERED[name] = op
+    return op
+
+
+def call(name: str, *args, **kwargs) -> None:
+    """Runs a registered operation on the current backend."""
+    op = _REGISTERED.get(name)
+    if op is None:
+        raise KeyError(f"operation {name!r} is not registered; known: {sorted(_REGISTERED)}")
+    if op.check is not None:
+        op.check(*args, **kwargs)
+    backend().run_registered(op, args, kwargs)
+
+
+def pointer(t: Optional[torch.Tensor]):
+    """A tensor's address as a ctypes argument (None: a null pointer)."""
+    import ctypes
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
 def embed_lookup(ids: torch.Tensor, table: torch.Tensor, scale: float, out: torch.Tensor) -> None:
     """out[i] = float32(table[ids[i]]) * scale.  ids int32 [n], table T [V, H], out float32 [n, H]."""
     _dense(ids, "ids", torch.int32)
@@ -74,7 +126,7 @@ def embed_lookup(ids: torch.Tensor, table: torch.Tensor, scale: float, out: torc
     _need(table.dim() == 2, "table: expected [vocab, hidden]")
     _dense(out, "out", torch.float32, (ids.shape[0], table.shape[1]))
     if ids.shape[0]:
-        backend().embed_lookup(ids, table, float(scale), out)
+        call("embed_lookup", ids, table, float(scale), out)
 
 
 def feed_tokens(ids: torch.Tensor, dst: torch.Tensor, src: torch.Tensor, source: torch.Tensor) -> None:
@@ -86,7 +138,7 @@ def feed_tokens(ids: torch.Tensor, dst: torch.Tensor, src: torch.Tensor, source:
         _need(t.dim() == 1, lambda: f"{name}: expected one axis")
     _need(dst.shape == src.shape, "dst and src: expected equal lengths")
     if dst.shape[0]:
-        backend().feed_tokens(ids, dst, src, source)
+        call("feed_tokens", ids, dst, src, source)
 
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, offset: float, out: torch.Tensor,
@@ -289,6 +341,19 @@ def plan_paged_attention(host_q_len, host_ctx_len, *, num_heads: int, num_kv_hea
                                           int(window), dtype, device)
 
 
+def static_attention_plan(segments: int, *, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int,
+                          window: int, dtype: torch.dtype, device, max_context: int, max_total_keys: int):
+    """The same for a captured graph of `segments` requests of one token each: a plan of fixed shape in
+    device memory, with room for contexts of up to `max_context` keys and `max_total_keys` keys of all
+    requests together, whose `update(host_q_len, host_ctx_len)` rewrites it in place before a replay.
+    None when the kernel that will run needs no plan."""
+    make = getattr(backend(), "static_attention_plan", None)
+    if make is None:
+        return None
+    return make(int(segments), num_heads, num_kv_heads, head_dim, page_size, int(window), dtype, device,
+                int(max_context), int(max_total_keys))
+
+
 def linear_splits(rows: int, out_features: int, in_features: int, dtype: torch.dtype) -> int:
     """Into how many partial sums over the input axis the product kernel for these sizes splits
     its work (1: it does not).  A caller that can take the sum later (the next norm, the rotation)
@@ -350,17 +415,19 @@ def linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, tiles: Opti
         backend().linear(x, weight, out, tiles)
 
 
-ACTIVATIONS = ("gelu_tanh", "silu")
+# the activations of a gated feed-forward and the numbers the kernels know them by (`common.h` holds
+# the same table): a new one is a line here, a line and a case there
+ACTIVATIONS = {"gelu_tanh": 0, "silu": 1}
 
 
 def gated_activation(gate_up: torch.Tensor, out: torch.Tensor, activation: str) -> None:
     """out = act(gate_up[:, :I]) * gate_up[:, I:], in float32, cast to T.  gate_up T [n, 2I]."""
-    _need(activation in ACTIVATIONS, lambda: f"activation {activation!r}: expected one of {ACTIVATIONS}")
+    _need(activation in ACTIVATIONS, lambda: f"activation {activation!r}: expected one of {sorted(ACTIVATIONS)}")
     _dense(gate_up, "gate_up", _ACT)
     _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "gate_up: expected [n, 2*intermediate]")
     _dense(out, "out", gate_up.dtype, (gate_up.shape[0], gate_up.shape[1] // 2))
     if gate_up.shape[0]:
-        backend().gated_activation(gate_up, out, activation)
+        call("gated_activation", gate_up, out, activation)
 
 
 class NormOnLoad:
@@ -397,7 +464,7 @@ def gated_linear(x, weight: torch.Tensor, out: torch.Tensor, activation: str,
     out T [m, I]; scratch T [m, 2I] may be used for the unfused product.  `tiles` is
     `tile_weight(weight, halves=2)`.  x may be a `NormOnLoad` where `gated_linear_norm_takes` says so:
     the norm is then applied as the kernel reads the residual stream (scratch is not used)."""
-    _need(activation in ACTIVATIONS, lambda: f"activation {activation!r}: expected one of {ACTIVATIONS}")
+    _need(activation in ACTIVATIONS, lambda: f"activation {activation!r}: expected one of {sorted(ACTIVATIONS)}")
     if isinstance(x, NormOnLoad):
         _need(gated_linear_norm_takes(x.shape[0], x.dtype, x.shape[1]), "gated_linear: no kernel with the norm on load for these sizes")
         _dense(weight, "weight", x.dtype)
@@ -459,3 +526,26 @@ def sample_rows(logits: torch.Tensor, params: torch.Tensor, seeds: torch.Tensor,
     if m:
         backend().sample_rows(logits, params, seeds, penalty_ids, penalty_offsets, out_tokens, out_logprobs,
                               truncations)
+
+
+# ---- the framework's own operations that go through the same door as a part's ------------------
+def _register_own() -> None:
+    from ctypes import c_float, c_int, c_void_p
+    p = pointer
+    register_op("embed_lookup", entry_point="wllm_embed_lookup",
+                argtypes=[c_void_p, c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
+                launch=lambda fn, stream, ids, table, scale, out: fn(
+                    p(ids), p(table), int(table.dtype == torch.bfloat16), scale, p(out), ids.shape[0], table.shape[1],
+                    table.shape[0], stream))
+    register_op("feed_tokens", entry_point="wllm_feed_tokens",
+                argtypes=[c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+                launch=lambda fn, stream, ids, dst, src, source: fn(
+                    p(ids), p(dst), p(src), p(source), dst.shape[0], ids.shape[0], source.shape[0], stream))
+    register_op("gated_activation", entry_point="wllm_gated_activation",
+                argtypes=[c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+                launch=lambda fn, stream, gate_up, out, activation: fn(
+                    p(gate_up), p(out), int(gate_up.dtype == torch.bfloat16), ACTIVATIONS[activation], gate_up.shape[0],
+                    out.shape[1], stream))
+
+
+_register_own()

@@ -82,6 +82,24 @@ class PagedAttention:
     def state_shape(self):
         return None
 
+    def _work_items(self, ctx, page_size: int):
+        """The step's work items for attention of this shape: made once a step, shared by all
+        layers of the shape; of fixed shape and rewritten in place in a captured graph."""
+        s = self.spec
+        shape = dict(num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim, page_size=page_size,
+                     window=s.window or 0)
+
+        def build(c):
+            if c.captured:
+                return ops.static_attention_plan(c.num_segments, max_context=c.capture_max_context,
+                                                 max_total_keys=c.capture_max_tokens, dtype=c.dtype, device=c.device, **shape)
+            return ops.plan_paged_attention(c.host_q_len, c.host_ctx_len, dtype=c.dtype, device=c.device, **shape)
+
+        def refresh(plan, c):
+            plan.update(c.host_q_len, c.host_ctx_len)
+
+        return ctx.plan(("attention",) + tuple(shape.values()), build, refresh)
+
     def forward(self, ctx, entry: int, h: torch.Tensor) -> torch.Tensor:
         s = self.spec
         n = h.shape[0]
@@ -121,7 +139,6 @@ class PagedAttention:
             ctx.seg_ctx_len, attn, num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim,
             page_size=pages.page_size, scale=s.scale, window=s.window or 0,
             max_q_len=ctx.max_q_len, max_ctx_len=ctx.max_ctx_len,
-            plan=ctx.attention_plan(num_heads=s.num_heads, num_kv_heads=s.num_kv_heads, head_dim=s.head_dim,
-                                    page_size=pages.page_size, window=s.window or 0))
+            plan=self._work_items(ctx, pages.page_size))
         # the stream adds the output projection: at once, or through the next norm, partial sums and all
         return Product("mixer_out", attn, self.w_o, self.t_o)
