@@ -40,29 +40,28 @@ def build_model(shape: dict, dtype: str, seed: int):
 
 
 def step_flops(model, tokens: int, context_before: int, logit_rows: int) -> float:
-    """Floating-point operations of one step over `tokens` new tokens of one request."""
+    """Floating-point operations of one step over `tokens` new tokens of one request, as the parts count them."""
+    keys = tokens * context_before + tokens * (tokens + 1) / 2.0       # what the queries see (causal)
     flops = 0.0
     for e in model.plan.schedule:
-        spec = model.plan.layers[e.layer]
-        m, f = spec.mixer, spec.feed_forward
-        qkv = (m.num_heads + 2 * m.num_kv_heads) * m.head_dim
-        flops += 2.0 * tokens * m.hidden_size * (qkv + m.num_heads * m.head_dim)
-        flops += 2.0 * tokens * f.hidden_size * f.intermediate_size * 3
-        # scores and weighted sums over the keys each query sees (causal)
-        keys = tokens * context_before + tokens * (tokens + 1) / 2.0
-        flops += 4.0 * m.num_heads * m.head_dim * keys
+        block = model.blocks[e.layer]
+        flops += block.mixer.flops(tokens, keys) + block.feed_forward.flops(tokens)
     flops += 2.0 * logit_rows * model.plan.head.hidden_size * model.plan.head.vocab_size
     return flops
 
 
 def kv_bytes_per_token(model) -> int:
+    """Bytes of cache a token holds over all layers: what a decode step reads of a live request, per token."""
+    import math
     total = 0
-    for i, need in model.cache_needs().items():
-        total += 2 * need.num_kv_heads * need.head_dim * (2 if model.dtype.itemsize == 2 else 4)
+    for need in model.cache_needs().values():
+        dtype = getattr(need, "dtype", None) or model.dtype
+        total += math.prod(need.page_shape(1)) * dtype.itemsize
     return total
 
 
 def measure_prefill(model, tokens: int, block_size: int, repeats: int = 6, warm: int = 3):
+    """Returns (mean seconds, best seconds) of `repeats` steps that run a prompt of `tokens` tokens whole."""
     import torch
 
     from wllm_amd.engine import ModelRunner, StepEntry
@@ -70,7 +69,7 @@ def measure_prefill(model, tokens: int, block_size: int, repeats: int = 6, warm:
     runner = ModelRunner.create(model, num_pages=pages, page_size=block_size, max_requests=2)
     g = torch.Generator().manual_seed(1)
     ids = torch.randint(0, model.plan.embedding.vocab_size, (tokens,), generator=g).tolist()
-    best = None
+    times = []
     for i in range(repeats + warm):     # the first runs find the clocks low and the library's products unchosen
         runner.open("p")
         torch.cuda.synchronize()
@@ -80,10 +79,48 @@ def measure_prefill(model, tokens: int, block_size: int, repeats: int = 6, warm:
         dt = time.perf_counter() - t0
         runner.close("p")
         if i >= warm:
-            best = dt if best is None else min(best, dt)
+            times.append(dt)
     del runner
     torch.cuda.empty_cache()
-    return best
+    return sum(times) / len(times), min(times)
+
+
+def measure_mixed_step(model, block_size: int, prompt_rows: int = 512, decoding: int = 64, context: int = 2048,
+                       repeats: int = 5):
+    """One step of `prompt_rows` rows of a prompt beside `decoding` decoded tokens of requests that hold
+    `context` tokens each: (mean seconds, share of the time that is the library's products)."""
+    import torch
+
+    from wllm_amd.engine import ModelRunner, StepEntry
+    from wllm_amd.kernels import ops
+    pages = decoding * (-(-(context + repeats + 4) // block_size)) + (-(-(prompt_rows * (repeats + 3)) // block_size)) + 2
+    runner = ModelRunner.create(model, num_pages=pages, page_size=block_size, max_requests=decoding + 1)
+    g = torch.Generator().manual_seed(3)
+    vocab = model.plan.embedding.vocab_size
+    for i in range(decoding):
+        runner.open(i)
+        for p in range(0, context, 2048):
+            runner.step([StepEntry(i, torch.randint(0, vocab, (min(2048, context - p),), generator=g).tolist(), [])])
+    runner.open("p")
+    backend = ops.backend()
+    times, library = [], []
+    for i in range(repeats + 2):
+        entries = [StepEntry(r, [int(torch.randint(0, vocab, (1,), generator=g))], [0]) for r in range(decoding)]
+        entries.append(StepEntry("p", torch.randint(0, vocab, (prompt_rows,), generator=g).tolist(), []))
+        backend.library_events = [] if i >= 2 else None
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        runner.step(entries)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        if i >= 2:
+            times.append(dt)
+            library.append(sum(a.elapsed_time(b) for a, b in backend.library_events) / 1000.0)
+        backend.library_events = None
+    del runner
+    torch.cuda.empty_cache()
+    mean = sum(times) / len(times)
+    return mean, (sum(library) / len(library)) / mean
 
 
 def measure_decode(model, batch: int, context: int, steps: int, warmup: int, block_size: int, hip_graphs: bool,
@@ -220,68 +257,84 @@ def main() -> int:
             print(json.dumps(run_stress(model, args)))
             return 0
         graphs = not args.no_graphs
-        weight_bytes = model.weight_bytes()
-        kv_per_token = kv_bytes_per_token(model)
+        points = {}
 
-        t_prefill = measure_prefill(model, args.prefill_tokens, args.block_size)
+        def decode_point(name, m, b, context, k, warm, dtype):
+            """A decode point: tokens a second, milliseconds a step, and the share of HBM's peak that the
+            bytes the step has to read (every weight once, the live requests' cache) make of its time."""
+            d, ctx_len = measure_decode(m, b, context, k, warm, args.block_size, graphs)
+            gbs = (m.weight_bytes() + b * ctx_len * kv_bytes_per_token(m)) / (d / k) / 1e9
+            if name is not None:
+                points[name] = round(k * b / d, 1)
+                points[name + "_ms"] = round(1000.0 * d / k, 4)
+                points[name + "_frac"] = round(gbs / PEAK_HBM_GBS, 4)
+            return d, gbs
+
+        def prefill_point(name, m, tokens, dtype, repeats=4):
+            mean, best = measure_prefill(m, tokens, args.block_size, repeats=repeats)
+            points[name] = round(tokens / mean, 1)
+            points[name + "_ms"] = round(1000.0 * mean, 3)
+            points[name + "_frac"] = round(step_flops(m, tokens, 0, 1) / mean / PEAK_FLOPS[dtype], 4)
+
+        t_prefill, t_prefill_best = measure_prefill(model, args.prefill_tokens, args.block_size)
         prefill_flops = step_flops(model, args.prefill_tokens, 0, 1)
 
-        dt, mean_ctx = measure_decode(model, args.batch, args.context, args.steps, args.warmup, args.block_size, graphs)
+        dt, achieved = decode_point(None, model, args.batch, args.context, args.steps, args.warmup, args.dtype)
         ms_per_step = 1000.0 * dt / args.steps
         value = args.steps * args.batch / dt
-        step_bytes = weight_bytes + args.batch * mean_ctx * kv_per_token
-        achieved = step_bytes / (dt / args.steps) / 1e9
 
-        points = {}
+        limit = model.plan.max_positions
         if not args.no_points:
             few = min(args.warmup, 4)
-
-            def point(b, context, k):
-                d, _ = measure_decode(model, b, context, k, few, args.block_size, graphs)
-                return round(k * b / d, 1)
-
             half = max(8, args.steps // 2)
-            points["decode_b1"] = point(1, args.context, args.steps)
-            points["decode_b64"] = point(64, args.context, half)
+            decode_point("decode_b1", model, 1, args.context, args.steps, few, args.dtype)
+            decode_point("decode_b64", model, 64, args.context, half, few, args.dtype)
             # the same batch near the longest context the configuration allows
-            limit = model.config.max_position_embeddings
             new_tokens = args.batch * (-(-limit // 2048)) + args.warmup + args.steps + 2      # as `measure_decode` counts them
             long_context = min(limit - 1024, (limit - new_tokens) // 256 * 256)
             if long_context > args.context:
-                points[f"decode_b{args.batch}_context_{long_context}"] = point(args.batch, long_context, args.steps)
+                decode_point(f"decode_b{args.batch}_context_{long_context}", model, args.batch, long_context, args.steps, few,
+                             args.dtype)
             if args.points == "all":
-                # further batch sizes and context lengths of the same configuration
-                points["decode_b128"] = point(128, args.context, half)
-                points["decode_b256"] = point(256, args.context, half)
+                # further batch sizes, context lengths and prompt lengths of the same configuration
+                decode_point("decode_b128", model, 128, args.context, half, few, args.dtype)
+                decode_point("decode_b256", model, 256, args.context, half, few, args.dtype)
                 for context in (4096, long_context):
                     if args.context < context <= limit - 1024:
-                        points[f"decode_b64_context_{context}"] = point(64, context, half)
+                        decode_point(f"decode_b64_context_{context}", model, 64, context, half, few, args.dtype)
+                for tokens in (512, 4096, 8192):
+                    if tokens <= limit and tokens != args.prefill_tokens:
+                        prefill_point(f"prefill_{tokens}", model, tokens, args.dtype)
+                # a step of a prompt's portion beside decoded tokens, and the library's share of it
+                mixed, share = measure_mixed_step(model, args.block_size)
+                points["mixed_512_rows_beside_64_decoded_ms"] = round(1000.0 * mixed, 3)
+                points["mixed_step_library_products_share"] = round(share, 3)
                 if args.dtype == "bf16" and args.shape == "gemma-2b" and args.layers is None:
                     # the continuous-batching stress workload on the same model: generated tokens a second
                     stress = run_stress(model, _StressDefaults)
-                    points["stress_64_requests_generated_tokens_per_s"] = stress["value"]
-                    points["stress_64_requests_seconds"] = stress["seconds"]
+                    points["stress_generated_tokens_per_s"] = stress["value"]
+                    points["stress_seconds"] = stress["seconds"]
+        plan = model.plan
+        layers_run = len(plan.schedule)
+        weight_bytes = model.weight_bytes()
         if not args.no_points and args.points == "all" and args.dtype == "bf16" and args.shape == "gemma-2b" and args.layers is None:
             # the other measured configurations, each with all its layers: the true 32-bit path of the same
-            # sizes, and decoding at the Gemma-7B layer sizes
-            c2 = model.config
+            # sizes, and the Gemma-7B layer sizes
             del model
             torch.cuda.empty_cache()
             other = build_model(shape, "fp32", args.seed)
-            d, _ = measure_decode(other, args.batch, args.context, half, 2, args.block_size, graphs)
-            points[f"fp32_{c2.num_hidden_layers}_layers_decode_b{args.batch}"] = round(half * args.batch / d, 1)
+            decode_point(f"fp32_decode_b{args.batch}", other, args.batch, args.context, half, 2, "fp32")
+            prefill_point(f"fp32_prefill_{args.prefill_tokens}", other, args.prefill_tokens, "fp32", repeats=2)
             del other
             torch.cuda.empty_cache()
-            big_shape = read_shape("gemma-7b")
-            other = build_model(big_shape, "bf16", args.seed)
+            other = build_model(read_shape("gemma-7b"), "bf16", args.seed)
             for b, k in ((1, half), (8, half), (64, max(8, half // 2))):
-                d, _ = measure_decode(other, b, args.context, k, 2, args.block_size, graphs)
-                points[f"gemma7b_{big_shape['num_hidden_layers']}_layers_decode_b{b}"] = round(k * b / d, 1)
+                decode_point(f"gemma7b_decode_b{b}", other, b, args.context, k, 2, "bf16")
+            prefill_point(f"gemma7b_prefill_{args.prefill_tokens}", other, args.prefill_tokens, "bf16", repeats=3)
             del other
             torch.cuda.empty_cache()
-            model = None
 
-    c = model.config if model is not None else c2
+    c = shape
     sizes = {"gemma-2b": "Gemma-2B", "gemma-7b": "Gemma-7B"}.get(args.shape, os.path.basename(args.shape))
     line = {
         "metric": f"decode tokens/s, {sizes} layer sizes, after {args.context:,}-token prompts",
@@ -297,20 +350,22 @@ def main() -> int:
         "dtype": args.dtype,
         "data": "synthetic: seeded random weights (normal, std 0.02) and seeded uniform token ids",
         "config": {
-            "model": f"{sizes} layer sizes (GemmaForCausalLM), random weights",
+            "model": f"{sizes} layer sizes ({c['architectures'][0]}), random weights",
             "global_batch": args.batch, "seq_len": args.context, "parallelism": "single GPU",
-            "layers": c.num_hidden_layers, "layers_of_full_model": full_layers, "hidden_size": c.hidden_size,
-            "intermediate_size": c.intermediate_size, "num_attention_heads": c.num_attention_heads,
-            "num_key_value_heads": c.num_key_value_heads, "head_dim": c.head_dim, "vocab_size": c.vocab_size,
-            "tied_embeddings": c.tie_word_embeddings, "rope_theta": c.rope_theta, "rms_norm_eps": c.rms_norm_eps,
-            "max_position_embeddings": c.max_position_embeddings, "kv_block_size": args.block_size,
+            "layers": layers_run, "layers_of_full_model": full_layers, "hidden_size": plan.embedding.hidden_size,
+            "intermediate_size": c.get("intermediate_size"), "num_attention_heads": c.get("num_attention_heads"),
+            "num_key_value_heads": c.get("num_key_value_heads", c.get("num_attention_heads")), "head_dim": c.get("head_dim"),
+            "vocab_size": plan.embedding.vocab_size, "tied_embeddings": plan.head.weight is None,
+            "rope_theta": c.get("rope_theta", 10000.0), "rms_norm_eps": c.get("rms_norm_eps", 1e-6),
+            "max_position_embeddings": limit, "kv_block_size": args.block_size,
             "sampling": "greedy", "hip_graphs": graphs, "lookahead": True,
         },
         "prefill": {"value": round(args.prefill_tokens / t_prefill, 1), "tokens": args.prefill_tokens,
-                    "ms": round(1000.0 * t_prefill, 3),
+                    "ms": round(1000.0 * t_prefill, 3), "ms_best": round(1000.0 * t_prefill_best, 3),
                     "frac": round(prefill_flops / t_prefill / PEAK_FLOPS[args.dtype], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+                     "frac": round(achieved / PEAK_HBM_GBS, 4),
+                     "bytes_per_step": int(achieved * 1e9 * dt / args.steps), "weight_bytes": weight_bytes},
         "points": points,
     }
     print(json.dumps(line))

@@ -4,7 +4,7 @@ from __future__ import annotations
 import numpy as np
 import torch
 
-from wllm_amd.config import GemmaConfig
+from wllm_amd.architectures import GemmaConfig
 from wllm_amd.parts import write_random_model_folder
 
 # Two tiny configurations that differ in every size and option, a third with

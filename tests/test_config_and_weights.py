@@ -5,7 +5,8 @@ import os
 import pytest
 import torch
 
-from wllm_amd.config import ConfigError, GemmaConfig, read_config_json, register_architecture, resolve_architecture
+from wllm_amd.architectures import GemmaConfig
+from wllm_amd.config import ConfigError, read_config_json, register_architecture, resolve_architecture
 from wllm_amd.parts import build_model, load_model, write_random_model_folder
 from wllm_amd.weights import Checkpoint, SafetensorsFile, WeightError, write_safetensors
 from helpers import TINY

@@ -14,7 +14,7 @@ import torch
 from helpers import (compare_replay, max_live_tokens, plain_for, random_ids, replay_and_collect, trace_mixed, trace_portions,
                      trace_tail, trace_whole)
 from plain import gemma_plain
-from wllm_amd.config import GemmaConfig
+from wllm_amd.architectures import GemmaConfig
 from wllm_amd.engine import ModelRunner
 from wllm_amd.engine.replay import TraceReplayer, pages_for_max_tokens
 from wllm_amd.parts import load_model, write_random_model_folder

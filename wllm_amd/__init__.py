@@ -10,5 +10,5 @@ hand-written gfx950 kernels behind all of it (`csrc`, `kernels`).
 
 __version__ = "0.1.0"
 
-from wllm_amd.config import GemmaConfig, register_architecture, resolve_architecture  # noqa: F401
+from wllm_amd.config import register_architecture, resolve_architecture  # noqa: F401
 from wllm_amd import architectures  # noqa: F401,E402  (registers the architectures)

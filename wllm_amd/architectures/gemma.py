@@ -12,7 +12,7 @@ from __future__ import annotations
 
 import math
 
-from wllm_amd.config.gemma import GemmaConfig
+from wllm_amd.architectures.gemma_config import GemmaConfig
 from wllm_amd.config.registry import register_architecture
 from wllm_amd.parts.specs import (
     AttentionSpec,

@@ -1,4 +1,5 @@
-from wllm_amd.config.gemma import GemmaConfig
+"""Reading config.json and the one registry from an architecture's name to its model.  The typed
+configuration of an architecture lives with the architecture (`wllm_amd/architectures`)."""
 from wllm_amd.config.registry import (
     ArchitectureEntry,
     ConfigError,
@@ -11,7 +12,6 @@ from wllm_amd.config.registry import (
 __all__ = [
     "ArchitectureEntry",
     "ConfigError",
-    "GemmaConfig",
     "read_config_json",
     "register_architecture",
     "registered_architectures",

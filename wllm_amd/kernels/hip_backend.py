@@ -77,6 +77,7 @@ class HipBackend:
         self._partial_ml = None
         self._generic_partial_o = None
         self._registered: dict = {}
+        self.library_events = None      # a list: every library product is bracketed by a pair of timing events
         for name, argtypes in _SIGNATURES.items():
             fn = getattr(self.lib, name)
             fn.argtypes = argtypes
@@ -374,6 +375,13 @@ class HipBackend:
                 return
             if out.dtype == torch.bfloat16 and m > 64:
                 # many rows: the library's matrix-core product (float32 accumulation)
+                if self.library_events is not None:     # a measurement asked for the library's share of a step
+                    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    begin.record()
+                    torch.mm(x, weight.t(), out=out)
+                    end.record()
+                    self.library_events.append((begin, end))
+                    return
                 torch.mm(x, weight.t(), out=out)
                 return
         # float32, few rows, a long K axis: the segments of K are summed by workgroups of their own

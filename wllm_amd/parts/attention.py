@@ -82,6 +82,12 @@ class PagedAttention:
     def state_shape(self):
         return None
 
+    def flops(self, tokens: int, keys: float) -> float:
+        """Floating-point operations of `tokens` tokens whose queries see `keys` keys in all (what a
+        measurement divides by its time)."""
+        s = self.spec
+        return 2.0 * tokens * s.hidden_size * (self.qkv_width + s.num_heads * s.head_dim) + 4.0 * s.num_heads * s.head_dim * keys
+
     def _work_items(self, ctx, page_size: int):
         """The step's work items for attention of this shape: made once a step, shared by all
         layers of the shape; of fixed shape and rewritten in place in a captured graph."""

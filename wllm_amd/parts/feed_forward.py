@@ -36,6 +36,10 @@ class GatedMLP:
             fetch, torch.cat([fetch.matrix(s.gate_weight), fetch.matrix(s.up_weight)], dim=0), halves=2)
         self.w_down, self.t_down = load_matrix(fetch, fetch.matrix(s.down_weight))
 
+    def flops(self, tokens: int) -> float:
+        """Floating-point operations of `tokens` tokens (what a measurement divides by its time)."""
+        return 6.0 * tokens * self.spec.hidden_size * self.spec.intermediate_size
+
     def takes_norm_on_load(self, rows: int, dtype: torch.dtype) -> bool:
         """Whether `forward` may be given `ops.NormOnLoad` instead of the normalised tensor."""
         return ops.gated_linear_norm_takes(rows, dtype, self.spec.hidden_size)
