@@ -35,7 +35,7 @@ def build_model(shape: dict, dtype: str, seed: int):
     model = build(shape)
     tdt = {"bf16": torch.bfloat16, "fp32": torch.float32}[dtype]
     model.load_from(RandomFetcher(model.expected_tensors(), seed, tdt, "cuda:0", std=0.02, norm_std=0.1,
-                                  tiled_copies=tdt == torch.bfloat16))
+                                  tiled_copies=True))
     return model
 
 

@@ -171,8 +171,14 @@ class EmulatedKernels:
         return self.splits
 
     def tile_weight(self, weight, tiles):
-        """[n, k] -> [band][step][g][i][8]: lane 16g + i of a wavefront holds w[16 band + i][32 step + 8g .. +8]."""
+        """bfloat16: [n, k] -> [band][step][g][i][8]: lane 16g + i of a wavefront holds w[16 band + i][32 step + 8g .. +8].
+        float32: [n, k] -> [band][chunk][g][i][4] with rows and keys padded with zeros to multiples of 16."""
         n, k = weight.shape
+        if weight.dtype == torch.float32:
+            padded = torch.zeros(-(-n // 16) * 16, -(-k // 16) * 16, dtype=weight.dtype, device=weight.device)
+            padded[:n, :k] = weight
+            tiles.copy_(padded.view(-1, 16, padded.shape[1] // 16, 4, 4).permute(0, 2, 3, 1, 4).reshape(-1))
+            return
         padded = torch.zeros(-(-n // 16) * 16, k, dtype=weight.dtype, device=weight.device)
         padded[:n] = weight
         tiles.copy_(padded.view(-1, 16, k // 32, 4, 8).permute(0, 2, 3, 1, 4).reshape(-1))
@@ -180,6 +186,12 @@ class EmulatedKernels:
     def _same_numbers(self, weight, tiles, halves):
         """A tile-major copy must hold the weight's numbers: the emulation computes from the weight."""
         if tiles is None:
+            return
+        if weight.dtype == torch.float32:
+            n, k = weight.shape
+            kp = -(-k // 16) * 16
+            back = tiles.view(-1, kp // 16, 4, 16, 4).permute(0, 3, 1, 2, 4).reshape(-1, kp)[:n, :k]
+            assert torch.equal(back, weight), "the tile-major copy differs from the weight"
             return
         n, k = weight.shape[0] // halves, weight.shape[1]
         size = -(-n // 16) * 16 * k

@@ -8,9 +8,10 @@ import pytest
 from wllm_amd.kernels import attention_plan as ap
 
 
-def covered(q_len, ctx_len, group, nkv, window, page_size):
+def covered(q_len, ctx_len, group, nkv, window, page_size, rows_per_item=64):
     items, reduces, slots, prefill, prefill_rows = ap.build_work_items(
-        np.array(q_len), np.array(ctx_len), group, nkv, window, page_size)
+        np.array(q_len), np.array(ctx_len), group, nkv, window, page_size, rows_per_item)
+    assert prefill_rows == rows_per_item
     cover = {}          # (seg, kvh, row) -> list of (first key, end key, slot)
     slot_users = {}
     def hold(slot, who):
@@ -78,7 +79,7 @@ def covered(q_len, ctx_len, group, nkv, window, page_size):
     return items, reduces, slots, prefill
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(24))
 def test_every_pair_is_covered_once(seed, monkeypatch):
     rng = np.random.default_rng(seed)
     # small targets so that small cases split the way large ones do
@@ -91,7 +92,7 @@ def test_every_pair_is_covered_once(seed, monkeypatch):
     n = int(rng.integers(1, 5))
     q_len = [int(rng.choice([1, 2, 5, 17, 70, 130, 400])) for _ in range(n)]
     ctx_len = [q + int(rng.choice([0, 1, 31, 128, 500, 1500])) for q in q_len]
-    covered(q_len, ctx_len, group, nkv, window, page_size)
+    covered(q_len, ctx_len, group, nkv, window, page_size, int(rng.choice([64, 128])))
 
 
 def test_a_late_portion_of_a_long_prompt_is_split_over_the_keys():

@@ -395,6 +395,29 @@ def test_float32_product_of_few_rows_has_the_bits_of_the_product_of_many(n, k):
         assert torch.equal(few, many[11:11 + rows]), f"{rows} rows"
 
 
+@pytest.mark.parametrize("m,n,k", [(8, 2048, 16384), (5, 2560, 2048), (16, 1000, 8192), (1, 777, 516), (3, 40000, 2048)])
+def test_float32_linear_leaves_partial_sums_to_the_caller(m, n, k):
+    """A float32 product of few rows and not many columns gives every segment of its K axis wavefronts
+    of their own; the stack of their sums, added in order, has the bits of the product made whole."""
+    torch.manual_seed(18)
+    x = torch.randn(m, k, device=DEV)
+    w = torch.randn(n, k, device=DEV) / math.sqrt(k)
+    s = ops.linear_splits(m, n, k, torch.float32)
+    whole = torch.zeros(m, n, device=DEV)
+    ops.linear(x, w, whole)
+    close(whole, x.double() @ w.double().T, torch.float32, "product")
+    if n >= 16384:
+        assert s == 1, "many columns are wavefronts enough"
+        return
+    assert s == -(-k // 512)
+    stack = torch.full((s, m, n), 7.0, device=DEV)
+    ops.linear(x, w, stack)
+    total = stack[0].clone()
+    for p in range(1, s):
+        total += stack[p]
+    assert torch.equal(total, whole)
+
+
 def test_tile_weight_is_the_documented_permutation():
     torch.manual_seed(12)
     for n, k, halves in ((40, 96, 1), (16, 32, 1), (2 * 23, 64, 2), (777, 2048, 1)):
@@ -404,7 +427,14 @@ def test_tile_weight_is_the_documented_permutation():
             ref = ops.tile_weight(w, halves)
         assert torch.equal(got, ref)
     assert ops.tile_weight(torch.randn(8, 40, device=DEV).to(torch.bfloat16)) is None      # 40 keys: no tiles
-    assert ops.tile_weight(torch.randn(8, 64, device=DEV)) is None                         # float32: no tiles
+    # float32: bands of 16 rows and chunks of 16 keys, both padded with zeros
+    for n, k in ((40, 96), (16, 16), (23, 20), (777, 2048), (5, 4)):
+        w = torch.randn(n, k, device=DEV)
+        got = ops.tile_weight(w)
+        with ops.use_backend(EmulatedKernels(precise=True)):
+            ref = ops.tile_weight(w)
+        assert got.shape == ref.shape == (ops.tiled_size(n, k, torch.float32),) and torch.equal(got, ref)
+    assert ops.tile_weight(torch.randn(8, 42, device=DEV)) is None                         # 42 keys: no tiles
 
 
 @pytest.mark.parametrize("m,n,k", [(8, 2048, 16384), (5, 2560, 2048), (64, 1000, 1024), (1, 777, 512), (16, 1000, 8192),

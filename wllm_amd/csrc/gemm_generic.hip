@@ -1,19 +1,15 @@
-// out[M, N] = x[M, K] * w[N, K]^T for float32 and bfloat16 operands, accumulated in float32 with
-// fused multiply-adds on the vector units.  No matrix-core instruction and no reduced-precision
-// mode is involved, so with float32 operands this is a true 32-bit product; it is the product
-// of the float32 path, and the product of last resort for bfloat16 (shapes the matrix-core
-// kernels do not take, float32 results from bfloat16 operands).
+// out[M, N] = x[M, K] * w[N, K]^T for float32 and bfloat16 operands, accumulated in float32.  It is
+// the product of the float32 path, and the product of last resort for bfloat16 (shapes the
+// bfloat16 matrix-core kernels do not take, float32 results from bfloat16 operands).  No
+// reduced-precision mode is involved anywhere: float32 operands are multiplied and added as float32,
+// on the matrix cores' float32 instruction where the K axis is a multiple of 4 (below), with fused
+// multiply-adds on the vector units otherwise (this kernel).
 //
 // A workgroup of 256 threads makes a 64x64 tile of the result; the K axis is walked in steps of
-// 16 through shared memory; a thread holds a 4x4 block.
-//
-// The order of an element's sum is fixed by K alone: the K axis is cut into segments of kSegment
+// 16 through shared memory; a thread holds a 4x4 block.  The K axis is cut into segments of kSegment
 // keys counted from 0, a segment is summed over k in ascending order of fused multiply-adds from
-// zero, and the segments' sums are added in ascending order.  Every kernel in this file sums in
-// that order, whatever the shape of the batch, so a row's result does not depend on the other rows
-// and a token's projection has the same bits in a decode step as inside a prompt.  (With one
-// segment, K <= kSegment, that is the plain ascending sum.)  The segments are what lets the
-// few-row kernel below spread a long K axis over many workgroups.
+// zero, and the segments' sums are added in ascending order: an order fixed by K alone, so a row's
+// result does not depend on the other rows of the batch.
 #include "common.h"
 
 constexpr int kTile = 64;
@@ -77,109 +73,203 @@ gemm_nt_kernel(const TI* __restrict__ x, const TI* __restrict__ w, TO* __restric
     }
 }
 
-// The same product for at most 16 rows of float32 (the decode steps of the float32 path).  The big
-// tile would leave all but N/64 workgroups idle and seven eighths of each tile empty; here a
-// workgroup makes ROWS rows x COLS columns, a thread one element, and the K axis is walked in chunks
-// through shared memory.  An element is still the sum over k in ascending order of fused
-// multiply-adds from zero within a segment of the K axis, so it has the same bits as the kernel above
-// gives it.  A workgroup takes one segment (blockIdx.y); with several segments their sums go to a
-// buffer of partial sums [segments, M, N] and a second kernel adds them in ascending order.
-//
-// What bounds it is how fast shared memory hands out operands (every product needs two), so the
-// tile is chosen for as many compute units as possible to share that work: 16 x 16 where there are
-// many columns; 8 columns, and 8 rows if the step has no more, for a projection back to the model's
-// width, whose N / 16 workgroups would be fewer than compute units.  There the chunks of the next
-// STAGES steps are on their way into registers while a chunk is summed: a trip to memory takes
-// microseconds, the sums of a chunk a fraction of one, and no other workgroup is there to hide it.
-constexpr int kFewRows = 16;
+// ---- float32 on the matrix cores ----------------------------------------------------------------
+// v_mfma_f32_16x16x4_f32 multiplies and accumulates IEEE float32 (no narrower format is involved), at
+// twice the rate that unpacked vector multiply-adds reach.  Both kernels below make an element of the
+// result by the same instructions on the same numbers in the same order, whatever the rows and columns
+// beside it, so a token's projection has the same bits in a decode step as inside a prompt:
+//   the K axis is cut into segments of kF32Segment keys counted from 0; within a segment the keys go
+//   in chunks of 16; a chunk is four instructions, the t-th of which takes the keys 16 q + 4 g + t
+//   (g = 0..3, the lane's group) and accumulates into the segment's sum, which starts at zero; the
+//   segments' sums are added in ascending order.
+// A lane (i, g) of a wavefront holds, of a chunk, w[n0 + i][16 q + 4 g .. + 3] and x[m0 + i][the same
+// keys]: one 16-byte load each, whose t-th element goes to the t-th instruction.  The first operand is
+// w, so a lane's four results are four consecutive columns of one row of out.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+constexpr int kF32Segment = 512;
+constexpr int kF32Chunk = 16;
 
-// One chunk of x and of w into a thread's registers, 16 bytes a piece; piece p is row p / (CHUNK / 4),
-// 16-byte column p % (CHUNK / 4).  Every lane loads, from a clamped address, and what lies outside the
-// operands is replaced by zeros afterwards (beyond K: the last piece again, then zeros): without a
-// branch around the loads the compiler counts exactly how many loads are in flight and waits only
-// for the stage it needs.
-template <int ROWS, int CHUNK, int THREADS>
-__device__ __forceinline__ void fetch_rows(float4 (&reg)[ROWS * (CHUNK / 4) / THREADS], const float* __restrict__ src, int tid,
-                                           int row0, int rows_end, int stride, int K, int k0) {
+__device__ __forceinline__ f32x4 mfma_chunk(const f32x4 a, const f32x4 b, f32x4 acc) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[0], b[0], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[1], b[1], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[2], b[2], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[3], b[3], acc, 0, 0, 0);
+    return acc;
+}
+
+// At most 16 rows (the decode steps of the float32 path): the weights stream from memory straight
+// into the lanes that multiply them, a wavefront a band of 16 columns, `U` chunks of it in flight at a
+// time; x comes through the caches (all wavefronts read the same few rows).  SPLIT: a wavefront takes
+// one segment of the K axis (blockIdx.y) and leaves its sum in partial[segment]; a second kernel adds
+// the segments in ascending order.  Otherwise it walks all segments and adds as it goes.
+// TILED: w is the weight's tile-major copy (`tile_weight_f32_kernel`): per band of 16 rows and chunk
+// of 16 keys one KiB in lane order, so that a wavefront's load is one contiguous KiB and its walk along
+// K one contiguous run (gate and up at Gemma-2B sizes: 76 us from the row-major weight, whose loads
+// touch 16 rows of 64 bytes each, 49 us from the copy).
+template <bool SPLIT, bool TILED>
+__global__ void __launch_bounds__(256)
+gemm_f32_few_rows_kernel(const float* __restrict__ x, const float* __restrict__ w, float* __restrict__ out, int M, int N,
+                         int K) {
+    constexpr int U = 8;
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int i = lane % 16, g = lane / 16;
+    const int n0 = (blockIdx.x * 4 + wave) * 16;
+    if (n0 >= N) return;
+    const int chunks_of_row = (K + kF32Chunk - 1) / kF32Chunk;
+    const float* wrow = TILED ? w + (static_cast<size_t>(n0 / 16) * chunks_of_row * 64 + lane) * 4
+                              : w + static_cast<size_t>(min(n0 + i, N - 1)) * K;
+    const float* xrow = x + static_cast<size_t>(min(i, M - 1)) * K;
+    const bool x_live = i < M;
+    const int segments = (K + kF32Segment - 1) / kF32Segment;
+    const int seg_first = SPLIT ? blockIdx.y : 0, seg_end = SPLIT ? blockIdx.y + 1 : segments;
+    f32x4 total = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int seg = seg_first; seg < seg_end; ++seg) {
+        const int k_begin = seg * kF32Segment, k_end = min(K, k_begin + kF32Segment);
+        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int k0 = k_begin; k0 < k_end; k0 += U * kF32Chunk) {
+            f32x4 a[U], b[U];
 #pragma unroll
-    for (int j = 0; j < ROWS * (CHUNK / 4) / THREADS; ++j) {
-        const int piece = j * THREADS + tid, row = row0 + piece / (CHUNK / 4), k = k0 + (piece % (CHUNK / 4)) * 4;
-        const float4 v = *reinterpret_cast<const float4*>(src + static_cast<size_t>(min(row, rows_end - 1)) * stride + min(k, K - 4));
-        const bool in = row < rows_end && k < K;       // element by element: a choice between two whole vectors goes through memory
-        reg[j] = make_float4(in ? v.x : 0.f, in ? v.y : 0.f, in ? v.z : 0.f, in ? v.w : 0.f);
+            for (int u = 0; u < U; ++u) {
+                // every lane loads, from a clamped address; what lies beyond the segment becomes zero
+                const int k = k0 + u * kF32Chunk + 4 * g;
+                // (a chunk beyond the row's last is clamped to the last: what it holds becomes zero below)
+                a[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(
+                    TILED ? wrow + static_cast<size_t>(min(k0 / kF32Chunk + u, chunks_of_row - 1)) * 256 : wrow + min(k, K - 4)));
+                b[u] = *reinterpret_cast<const f32x4*>(xrow + min(k, K - 4));
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int k = k0 + u * kF32Chunk + 4 * g;
+                const bool live = k < k_end;
+                const f32x4 zero = f32x4{0.f, 0.f, 0.f, 0.f};
+                const f32x4 av = live ? a[u] : zero, bv = live && x_live ? b[u] : zero;
+                if (k0 + u * kF32Chunk < k_end) acc = mfma_chunk(av, bv, acc);     // the same for all lanes
+            }
+        }
+        total = seg == seg_first ? acc : total + acc;
+    }
+    // lane (i, g) holds out[row i][n0 + 4 g .. + 3]
+    if (!x_live) return;
+    float* dst = out + (SPLIT ? static_cast<size_t>(blockIdx.y) * M * N : 0) + static_cast<size_t>(i) * N + n0 + 4 * g;
+    if (N % 4 == 0 && n0 + 4 * g + 3 < N) {
+        *reinterpret_cast<f32x4*>(dst) = total;
+    } else {
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+            if (n0 + 4 * g + v < N) dst[v] = total[v];
     }
 }
 
-template <int ROWS, int COLS, int CHUNK, int STAGES>
-__global__ void __launch_bounds__(ROWS * COLS)
-gemm_nt_few_rows_kernel(const float* __restrict__ x, const float* __restrict__ w, float* __restrict__ out, int M,
-                        int N, int K_all) {
-    constexpr int kThreads = ROWS * COLS;
-    // this workgroup's segment of the K axis: x and w begin at its first key, K is its length, and the row
-    // stride stays that of the whole operands
-    const int seg_begin = blockIdx.y * kSegment;
-    const int K = min(kSegment, K_all - seg_begin);
-    x += seg_begin;
-    w += seg_begin;
-    out += static_cast<size_t>(blockIdx.y) * M * N;
-    constexpr int kXPieces = ROWS * (CHUNK / 4) / kThreads, kWPieces = COLS * (CHUNK / 4) / kThreads;
-    static_assert(kXPieces * kThreads == ROWS * (CHUNK / 4) && kWPieces * kThreads == COLS * (CHUNK / 4), "whole pieces per thread");
-    __shared__ float4 xs[ROWS][CHUNK / 4 + 1];
-    __shared__ float4 ws[COLS][CHUNK / 4 + 1];
-    const int tid = threadIdx.x;
-    const int col0 = blockIdx.x * COLS;
-    const int r = tid / COLS, c = tid % COLS;
-    float4 xreg[STAGES][kXPieces], wreg[STAGES][kWPieces];
-    float acc = 0.f;
+// More rows: a workgroup of four wavefronts (2 x 2) makes 32 WM rows by 32 WN columns; the tiles of
+// x and w of a chunk go through shared memory, the next chunk's loads in flight while this one is
+// multiplied.  Rows of a tile are padded to 20 floats, so that the 16-byte fragment reads of 8 lanes
+// fall into different banks.
+template <int WM, int WN>
+__global__ void __launch_bounds__(256, 2)
+gemm_f32_tile_kernel(const float* __restrict__ x, const float* __restrict__ w, float* __restrict__ out, int M, int N, int K) {
+    constexpr int TM = 32 * WM, TN = 32 * WN, kStride = kF32Chunk + 4;
+    constexpr int XP = TM * 4 / 256, WP = TN * 4 / 256;       // 16-byte pieces of a chunk's tiles per thread
+    static_assert(XP * 256 == TM * 4 && WP * 256 == TN * 4, "whole pieces per thread");
+    __shared__ __align__(16) float xs[2][TM * kStride];
+    __shared__ __align__(16) float ws[2][TN * kStride];
+    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const int i = lane % 16, g = lane / 16;
+    const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
+    const int wm0 = (wave / 2) * (TM / 2), wn0 = (wave % 2) * (TN / 2);
+    // a thread's pieces: row tid / 4 (+ 64 per further piece), keys 4 (tid % 4) ..
+    const int p_row = tid / 4, p_k = (tid % 4) * 4;
+    const float* xsrc[XP];
+    const float* wsrc[WP];
 #pragma unroll
-    for (int s = 0; s < STAGES; ++s) {
-        fetch_rows<ROWS, CHUNK, kThreads>(xreg[s], x, tid, 0, M, K_all, K, s * CHUNK);
-        fetch_rows<COLS, CHUNK, kThreads>(wreg[s], w, tid, col0, N, K_all, K, s * CHUNK);
+    for (int p = 0; p < XP; ++p) xsrc[p] = x + static_cast<size_t>(min(m0 + p_row + 64 * p, M - 1)) * K;
+#pragma unroll
+    for (int p = 0; p < WP; ++p) wsrc[p] = w + static_cast<size_t>(min(n0 + p_row + 64 * p, N - 1)) * K;
+    // two sets of registers for chunks on their way: a chunk is asked for two chunks before it is
+    // multiplied, so a trip to memory has two chunks' products to hide behind
+    f32x4 xr[2][XP], wr[2][WP];
+    auto fetch = [&](f32x4 (&xq)[XP], f32x4 (&wq)[WP], int k0) {
+        const int k = k0 + p_k;
+        const bool live = k < K;
+        const f32x4 zero = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int p = 0; p < XP; ++p) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(xsrc[p] + min(k, K - 4));
+            xq[p] = live ? v : zero;
+        }
+#pragma unroll
+        for (int p = 0; p < WP; ++p) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(wsrc[p] + min(k, K - 4));
+            wq[p] = live ? v : zero;
+        }
+    };
+    auto stage = [&](int buf, const f32x4 (&xq)[XP], const f32x4 (&wq)[WP]) {
+#pragma unroll
+        for (int p = 0; p < XP; ++p) *reinterpret_cast<f32x4*>(&xs[buf][(p_row + 64 * p) * kStride + p_k]) = xq[p];
+#pragma unroll
+        for (int p = 0; p < WP; ++p) *reinterpret_cast<f32x4*>(&ws[buf][(p_row + 64 * p) * kStride + p_k]) = wq[p];
+    };
+    f32x4 acc[WM][WN], total[WM][WN];
+#pragma unroll
+    for (int jm = 0; jm < WM; ++jm)
+#pragma unroll
+        for (int jn = 0; jn < WN; ++jn) acc[jm][jn] = total[jm][jn] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const int chunks = (K + kF32Chunk - 1) / kF32Chunk;
+    constexpr int kChunksPerSegment = kF32Segment / kF32Chunk;
+    // chunk q: multiplied from tile q % 2 of shared memory; chunk q + 1 waits in the registers (q + 1) % 2
+    // and goes to the other tile when the products of chunk q are issued; chunk q + 2 is asked for
+    auto step = [&](int q, int buf, f32x4 (&x_next)[XP], f32x4 (&w_next)[WP], f32x4 (&x_ask)[XP], f32x4 (&w_ask)[WP]) {
+        if (q + 2 < chunks) fetch(x_ask, w_ask, (q + 2) * kF32Chunk);
+        f32x4 a[WN], b[WM];
+#pragma unroll
+        for (int jn = 0; jn < WN; ++jn) a[jn] = *reinterpret_cast<const f32x4*>(&ws[buf][(wn0 + 16 * jn + i) * kStride + 4 * g]);
+#pragma unroll
+        for (int jm = 0; jm < WM; ++jm) b[jm] = *reinterpret_cast<const f32x4*>(&xs[buf][(wm0 + 16 * jm + i) * kStride + 4 * g]);
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int jm = 0; jm < WM; ++jm)
+#pragma unroll
+                for (int jn = 0; jn < WN; ++jn)
+                    acc[jm][jn] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[jn][t], b[jm][t], acc[jm][jn], 0, 0, 0);
+        if ((q + 1) % kChunksPerSegment == 0 || q + 1 == chunks) {
+            // a segment ends: its sum joins the sums of the segments before it
+            const bool first = q < kChunksPerSegment;
+#pragma unroll
+            for (int jm = 0; jm < WM; ++jm)
+#pragma unroll
+                for (int jn = 0; jn < WN; ++jn) {
+                    total[jm][jn] = first ? acc[jm][jn] : total[jm][jn] + acc[jm][jn];
+                    acc[jm][jn] = f32x4{0.f, 0.f, 0.f, 0.f};
+                }
+        }
+        if (q + 1 < chunks) stage(buf ^ 1, x_next, w_next);
+        __syncthreads();
+    };
+    fetch(xr[0], wr[0], 0);
+    stage(0, xr[0], wr[0]);
+    if (chunks > 1) fetch(xr[1], wr[1], kF32Chunk);
+    __syncthreads();
+    for (int q = 0; q < chunks; q += 2) {
+        step(q, 0, xr[1], wr[1], xr[0], wr[0]);
+        if (q + 1 < chunks) step(q + 1, 1, xr[0], wr[0], xr[1], wr[1]);
     }
-    for (int k0 = 0; k0 < K; k0 += STAGES * CHUNK) {
 #pragma unroll
-        for (int s = 0; s < STAGES; ++s) {
-            const int kk = k0 + s * CHUNK;
-            if (kk >= K) continue;       // the same for all threads (no `break`: the stages must unroll, or the register sets become memory)
-            __syncthreads();
+    for (int jm = 0; jm < WM; ++jm) {
+        const int m = m0 + wm0 + 16 * jm + i;
+        if (m >= M) continue;
 #pragma unroll
-            for (int j = 0; j < kXPieces; ++j) xs[(j * kThreads + tid) / (CHUNK / 4)][(j * kThreads + tid) % (CHUNK / 4)] = xreg[s][j];
+        for (int jn = 0; jn < WN; ++jn) {
+            const int n = n0 + wn0 + 16 * jn + 4 * g;
+            float* dst = out + static_cast<size_t>(m) * N + n;
+            if (N % 4 == 0 && n + 3 < N) {
+                *reinterpret_cast<f32x4*>(dst) = total[jm][jn];
+            } else {
 #pragma unroll
-            for (int j = 0; j < kWPieces; ++j) ws[(j * kThreads + tid) / (CHUNK / 4)][(j * kThreads + tid) % (CHUNK / 4)] = wreg[s][j];
-            __syncthreads();
-            fetch_rows<ROWS, CHUNK, kThreads>(xreg[s], x, tid, 0, M, K_all, K, kk + STAGES * CHUNK);
-            fetch_rows<COLS, CHUNK, kThreads>(wreg[s], w, tid, col0, N, K_all, K, kk + STAGES * CHUNK);
-            // The whole chunk always (beyond K it holds zeros, which leave the sum as it is).  The reads of
-            // eight steps are asked for while the eight steps before them are summed: the chain of
-            // dependent additions is all a wavefront does here, and it should not wait for shared memory.
-            constexpr int kBatch = 8;
-            float4 a[2][kBatch], b[2][kBatch];
-#pragma unroll
-            for (int i = 0; i < kBatch; ++i) {
-                a[0][i] = xs[r][i];
-                b[0][i] = ws[c][i];
-            }
-#pragma unroll
-            for (int k4 = 0; k4 < CHUNK / 4; k4 += kBatch) {
-                const int cur = (k4 / kBatch) % 2, nxt = cur ^ 1;
-                if (k4 + kBatch < CHUNK / 4) {
-#pragma unroll
-                    for (int i = 0; i < kBatch; ++i) {
-                        a[nxt][i] = xs[r][k4 + kBatch + i];
-                        b[nxt][i] = ws[c][k4 + kBatch + i];
-                    }
-                }
-#pragma unroll
-                for (int i = 0; i < kBatch; ++i) {
-                    acc = fmaf(a[cur][i].x, b[cur][i].x, acc);
-                    acc = fmaf(a[cur][i].y, b[cur][i].y, acc);
-                    acc = fmaf(a[cur][i].z, b[cur][i].z, acc);
-                    acc = fmaf(a[cur][i].w, b[cur][i].w, acc);
-                }
+                for (int v = 0; v < 4; ++v)
+                    if (n + v < N) dst[v] = total[jm][jn][v];
             }
         }
     }
-    if (r < M && col0 + c < N) out[static_cast<size_t>(r) * N + col0 + c] = acc;
 }
 
 // out[i] = partial[0][i] + partial[1][i] + ... in ascending order of the segments.
@@ -192,28 +282,91 @@ gemm_segments_sum_kernel(const float* __restrict__ partial, float* __restrict__ 
     out[i] = total;
 }
 
-// Segments of the K axis, and with them the floats of `partial` that `wllm_gemm_generic` needs for a
-// float32 product of at most 16 rows: segments * M * N if there are several segments, none otherwise.
-WLLM_API int wllm_gemm_generic_segments(int K) { return (K + kSegment - 1) / kSegment; }
+namespace {
+// Whether the few-row kernel gives every segment of the K axis a wavefront of its own: where the bands
+// of 16 columns alone are too few wavefronts to keep the memory busy.
+bool few_rows_split(int N, int K) { return K > kF32Segment && (N + 15) / 16 < 1024; }
+bool f32_by_matrix_cores(int in_bf16, int out_bf16, int K) { return !in_bf16 && !out_bf16 && K % 4 == 0 && K >= 4; }
+}  // namespace
 
-WLLM_API int wllm_gemm_generic(const void* x, const void* w, int in_bf16, void* out, int out_bf16, void* partial, int M,
-                               int N, int K, hipStream_t stream) {
-    if (!in_bf16 && !out_bf16 && M >= 1 && M <= kFewRows && K % 4 == 0 && K >= 4 && N >= 1) {
-        const int segments = (K + kSegment - 1) / kSegment;
-        if (segments > 1 && !partial) return -1;
-        if (segments > 65535) return -1;
-        float* dst = segments > 1 ? static_cast<float*>(partial) : static_cast<float*>(out);
-#define FEW(ROWS, COLS, CHUNK, STAGES)                                                                       \
-    gemm_nt_few_rows_kernel<ROWS, COLS, CHUNK, STAGES><<<dim3((N + COLS - 1) / COLS, segments), ROWS * COLS, 0, stream>>>( \
-        static_cast<const float*>(x), static_cast<const float*>(w), dst, M, N, K)
-        // many workgroups: the large tile with one chunk on its way; few: small tiles, each with several
-        if (static_cast<long long>((N + kFewRows - 1) / kFewRows) * segments > 512) FEW(16, 16, 128, 1);
-        else if (M <= 8) FEW(8, 8, 128, 4);
-        else FEW(16, 8, 128, 4);
-#undef FEW
-        if (int err = launch_status()) return err;
-        if (segments > 1)
-            gemm_segments_sum_kernel<<<(M * N + 255) / 256, 256, 0, stream>>>(dst, static_cast<float*>(out), M * N, segments);
+// The tile-major copy of a float32 weight [N, K] (K a multiple of 4): for band b of 16 rows and chunk q
+// of 16 keys, lane 16 g + i finds w[16 b + i][16 q + 4 g .. + 3] at ((b * chunks + q) * 64 + lane) * 4;
+// rows beyond N and keys beyond K are zeros.
+__global__ void __launch_bounds__(256)
+tile_weight_f32_kernel(const float* __restrict__ w, float* __restrict__ tiles, int N, int K, int chunks, long long pieces) {
+    const long long piece = static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (piece >= pieces) return;
+    const int lane = piece % 64, i = lane % 16, g = lane / 16;
+    const long long tile = piece / 64;
+    const int q = tile % chunks;
+    const long long row = tile / chunks * 16 + i;
+    const int k = 16 * q + 4 * g;
+    f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (row < N && k < K) v = *reinterpret_cast<const f32x4*>(w + row * K + k);
+    *reinterpret_cast<f32x4*>(tiles + piece * 4) = v;
+}
+
+// Elements of the tile-major copy of a float32 weight [N, K].
+WLLM_API long long wllm_tiled_size_f32(int N, int K) {
+    return static_cast<long long>((N + 15) / 16) * 16 * ((K + kF32Chunk - 1) / kF32Chunk) * kF32Chunk;
+}
+
+WLLM_API int wllm_tile_weight_f32(const float* w, float* tiles, int N, int K, hipStream_t stream) {
+    if (N < 1 || K < 4 || K % 4 != 0) return -1;
+    const int chunks = (K + kF32Chunk - 1) / kF32Chunk;
+    const long long pieces = static_cast<long long>((N + 15) / 16) * chunks * 64;
+    const long long blocks = (pieces + 255) / 256;
+    if (blocks > 0x7fffffffLL) return -1;
+    tile_weight_f32_kernel<<<static_cast<unsigned>(blocks), 256, 0, stream>>>(w, tiles, N, K, chunks, pieces);
+    return launch_status();
+}
+
+// Into how many partial sums [segments, M, N] a float32 product of these sizes is split (1: it is not).
+// `wllm_gemm_generic` needs `partial` to hold them; with `out` null it leaves them there for a consumer
+// that adds them in ascending order.
+WLLM_API int wllm_gemm_f32_segments(int M, int N, int K) {
+    if (M < 1 || M > 16 || K % 4 != 0 || !few_rows_split(N, K)) return 1;
+    return (K + kF32Segment - 1) / kF32Segment;
+}
+
+// `tiles`: null, or the tile-major copy of a float32 w (`wllm_tile_weight_f32`), which the few-row kernel
+// streams faster; everything else reads w.
+WLLM_API int wllm_gemm_generic(const void* x, const void* w, const void* tiles, int in_bf16, void* out, int out_bf16,
+                               void* partial, int M, int N, int K, hipStream_t stream) {
+    if (M < 1 || N < 1 || K < 1) return -1;
+    if (f32_by_matrix_cores(in_bf16, out_bf16, K)) {
+        const float* xf = static_cast<const float*>(x);
+        const float* wf = static_cast<const float*>(w);
+        const float* tf = static_cast<const float*>(tiles);
+        float* of = static_cast<float*>(out);
+        if (M <= 16) {
+            const int bands = (N + 15) / 16, groups = (bands + 3) / 4;
+            if (few_rows_split(N, K)) {
+                const int segments = (K + kF32Segment - 1) / kF32Segment;
+                if (!partial || segments > 65535) return -1;
+                float* pf = static_cast<float*>(partial);
+                if (tf) gemm_f32_few_rows_kernel<true, true><<<dim3(groups, segments), 256, 0, stream>>>(xf, tf, pf, M, N, K);
+                else gemm_f32_few_rows_kernel<true, false><<<dim3(groups, segments), 256, 0, stream>>>(xf, wf, pf, M, N, K);
+                if (int err = launch_status()) return err;
+                if (of) gemm_segments_sum_kernel<<<(M * N + 255) / 256, 256, 0, stream>>>(pf, of, M * N, segments);
+            } else {
+                if (!of) return -1;
+                if (tf) gemm_f32_few_rows_kernel<false, true><<<groups, 256, 0, stream>>>(xf, tf, of, M, N, K);
+                else gemm_f32_few_rows_kernel<false, false><<<groups, 256, 0, stream>>>(xf, wf, of, M, N, K);
+            }
+            return launch_status();
+        }
+        if (!of) return -1;
+        // tiles of 128 x 128 where they fill the machine, smaller ones where a product has few columns or rows
+        const long long rows128 = (M + 127) / 128, cols128 = (N + 127) / 128, cols64 = (N + 63) / 64;
+        if (rows128 > 65535 || (M + 63) / 64 > 65535) return -1;
+        if (rows128 * cols128 >= 384) {
+            gemm_f32_tile_kernel<4, 4><<<dim3(cols128, rows128), 256, 0, stream>>>(xf, wf, of, M, N, K);
+        } else if (rows128 * cols64 >= 384) {
+            gemm_f32_tile_kernel<4, 2><<<dim3(cols64, rows128), 256, 0, stream>>>(xf, wf, of, M, N, K);
+        } else {
+            gemm_f32_tile_kernel<2, 2><<<dim3(cols64, (M + 63) / 64), 256, 0, stream>>>(xf, wf, of, M, N, K);
+        }
         return launch_status();
     }
     const dim3 grid((N + kTile - 1) / kTile, (M + kTile - 1) / kTile);

@@ -38,8 +38,8 @@ class LLM:
         """`model`: a folder with config.json and model.safetensors.  `num_blocks` pages of
         `block_size` tokens make the cache pool.  `max_prefill_tokens_per_step` enables
         chunked prefill.  `hip_graphs` replays captured graphs for decode-only steps.
-        `decode_weight_copy` keeps a second copy of the bfloat16 matrices in the order the decode
-        kernels read fastest (default: yes for bfloat16; costs the matrices' memory once more).
+        `decode_weight_copy` keeps a second copy of the matrices in the order the decode
+        kernels read fastest (default: yes; costs the matrices' memory once more).
         `lookahead` starts each step before the tokens of the step before it have been read, so the
         GPU does not wait for the host between steps; what is generated is the same.
         `step_row_multiple`: under chunked prefill a portion that the budget cuts is shortened so that

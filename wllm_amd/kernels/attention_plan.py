@@ -36,8 +36,7 @@ ITEM_INTS = 8
 PREFILL_TABLE_PAGES = 1024      # pages one prefill item may span (the kernel's shared block table)
 PREFILL_TARGET_ITEMS = 1024     # prefill items wanted in a step: about four for each compute unit
 PREFILL_MIN_CHUNK = 512         # keys; smaller pieces cost more in partial results than they gain
-PREFILL_ROWS = 64               # rows of a prefill item: with 64 two workgroups share a compute unit (128 rows
-                                # reuse the staged keys more, but fill the register file with one workgroup)
+PREFILL_ROWS = 64               # rows of a prefill item unless the kernel for the sizes at hand says otherwise
 
 
 @dataclass
@@ -112,7 +111,7 @@ MAX_HEADS = 1 << 16     # an item packs the key/value head and the tile's first 
 
 
 def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_heads: int, window: int,
-                     page_size: int = 16):
+                     page_size: int = 16, prefill_rows: int = PREFILL_ROWS):
     """Returns (items [n, 8], reduce_items [m, 8], partial slots, prefill items [p, 8], rows per
     prefill item) as int32 arrays."""
     q_len = np.asarray(q_len, dtype=np.int64)
@@ -177,9 +176,7 @@ def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_
     # ---- long segments: workgroups of 64 or 128 rows of one key/value head ----
     prefill = []
     long_idx = np.nonzero(~short)[0]
-    prefill_rows = PREFILL_ROWS
     if long_idx.size:
-        prefill_rows = PREFILL_ROWS
         blocks = []              # (segment, first rows, lowest key, end key) per long segment
         span_total = 0
         for s in long_idx:

@@ -52,8 +52,9 @@ _SIGNATURES = {
                                      c_void_p],
     "wllm_gemm_tile": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "wllm_split_sum": [c_void_p, c_void_p, c_int, c_longlong, c_int, c_void_p],
-    "wllm_gemm_generic": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
-    "wllm_gemm_generic_segments": [c_int],
+    "wllm_gemm_generic": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
+    "wllm_tile_weight_f32": [c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "wllm_gemm_f32_segments": [c_int, c_int, c_int],
     "wllm_argmax_rows": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "wllm_gemm_skinny": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
                          c_void_p],
@@ -324,10 +325,16 @@ class HipBackend:
             return self.skinny_split(out_features, in_features)
         if self.tile_takes(dtype, rows, out_features, in_features):
             return self.tile_splits(out_features, in_features, rows)
+        if dtype == torch.float32 and rows <= 16:
+            return self.lib.wllm_gemm_f32_segments(rows, out_features, in_features)
         return 1
 
     def tile_weight(self, weight, tiles) -> None:
         self._on_gpu(weight, tiles)
+        if weight.dtype == torch.float32:
+            self._check(self.lib.wllm_tile_weight_f32(_ptr(weight), _ptr(tiles), weight.shape[0], weight.shape[1],
+                                                      self._stream()), "tile_weight (float32)")
+            return
         self._check(self.lib.wllm_tile_weight(_ptr(weight), _ptr(tiles), weight.shape[0], weight.shape[1], self._stream()),
                     "tile_weight")
 
@@ -384,29 +391,34 @@ class HipBackend:
                     return
                 torch.mm(x, weight.t(), out=out)
                 return
-        # float32, few rows, a long K axis: the segments of K are summed by workgroups of their own
+        # float32, few rows, a long K axis: the segments of K are summed by wavefronts of their own
         if x.dtype == torch.float32 and m <= 16:
-            segments = self.lib.wllm_gemm_generic_segments(k)
             n = weight.shape[0]
+            segments = self.lib.wllm_gemm_f32_segments(m, n, k)
+            if out.dim() == 3:      # the caller adds the segments' sums later
+                self._check(self.lib.wllm_gemm_generic(_ptr(x), _ptr(weight), _ptr(tiles), 0, c_void_p(0), 0, _ptr(out), m, n, k,
+                                                       self._stream()), "linear (float32, partial sums)")
+                return
             if segments > 1 and segments * m * n > self.GEMM_PARTIAL_FLOATS:
-                # more partial sums than the buffer holds (logits of a large vocabulary): some rows at a
-                # time; a row's sums do not depend on the rows beside it
+                # more partial sums than the buffer holds: some rows at a time; a row's sums do not
+                # depend on the rows beside it
                 rows = self.GEMM_PARTIAL_FLOATS // (segments * n)
                 if rows < 1:
                     raise KernelError(f"linear: {segments} segments of {n} columns need more than the "
                                       f"{self.GEMM_PARTIAL_FLOATS} floats of the split-sum buffer for one row")
                 for r in range(0, m, rows):
-                    self._generic(x[r:r + rows], weight, out[r:r + rows], segments)
+                    self._generic(x[r:r + rows], weight, out[r:r + rows], segments, tiles)
                 return
-            self._generic(x, weight, out, segments)
+            self._generic(x, weight, out, segments, tiles)
             return
         self._generic(x, weight, out, 1)
 
-    def _generic(self, x, weight, out, segments: int) -> None:
+    def _generic(self, x, weight, out, segments: int, tiles=None) -> None:
         m, n = x.shape[0], weight.shape[0]
         partial = self._gemm_partial(segments * m * n, x.device) if segments > 1 else None
         self._check(self.lib.wllm_gemm_generic(
-            _ptr(x), _ptr(weight), int(x.dtype == torch.bfloat16), _ptr(out), int(out.dtype == torch.bfloat16),
+            _ptr(x), _ptr(weight), _ptr(tiles) if x.dtype == torch.float32 else c_void_p(0), int(x.dtype == torch.bfloat16),
+            _ptr(out), int(out.dtype == torch.bfloat16),
             _ptr(partial), m, n, x.shape[1], self._stream()), "linear")
 
     def gated_linear(self, x, weight, out, activation, scratch, tiles=None):
@@ -426,7 +438,9 @@ class HipBackend:
                                                 1 + ACTIVATIONS[activation], self._stream()),
                         "gated_linear (tiles)")
             return
-        self.linear(x, weight, scratch)
+        # (the tile-major copy of a stacked float32 matrix is that of the one matrix it is; a bfloat16 one's
+        # halves are tiled each by itself, which only the gated kernels above read)
+        self.linear(x, weight, scratch, tiles if x.dtype == torch.float32 else None)
         ops.call("gated_activation", scratch, out, activation)
 
     @staticmethod

@@ -361,22 +361,35 @@ def linear_splits(rows: int, out_features: int, in_features: int, dtype: torch.d
     return int(backend().linear_splits(rows, out_features, in_features, dtype))
 
 
-def tiled_size(rows: int, in_features: int) -> int:
+def tiled_size(rows: int, in_features: int, dtype: torch.dtype = torch.bfloat16) -> int:
     """Elements of the tile-major copy of a [rows, in_features] weight (`tile_weight`)."""
+    if dtype == torch.float32:
+        return -(-rows // 16) * 16 * -(-in_features // 16) * 16
     return -(-rows // 16) * 16 * in_features
 
 
 def tile_weight(weight: torch.Tensor, halves: int = 1) -> Optional[torch.Tensor]:
-    """The tile-major copy of a bfloat16 weight [n, k] that the few-row product kernels stream:
-    for each band of 16 rows (the last padded with zero rows) and each step of 32 keys, a tile of
-    1 KiB in which lane l = 16g + i of a wavefront finds w[16 * band + i][32 * step + 8g .. +8].
-    With halves = 2 (a stacked gate and up matrix) each half is tiled by itself, the gate's bands
-    first.  Returns a flat tensor, or None for weights the few-row kernels do not take (float32,
-    k not a multiple of 32)."""
+    """The tile-major copy of a weight [n, k] that the few-row product kernels stream: a wavefront's
+    load is one contiguous KiB of it, and its walk along k one contiguous run.
+    bfloat16 (k a multiple of 32): for each band of 16 rows (the last padded with zero rows) and each
+    step of 32 keys, a tile of 1 KiB in which lane l = 16g + i of a wavefront finds
+    w[16 * band + i][32 * step + 8g .. +8].  With halves = 2 (a stacked gate and up matrix) each half
+    is tiled by itself, the gate's bands first.
+    float32 (k a multiple of 4): for each band of 16 rows and each chunk of 16 keys (rows and keys
+    beyond the weight are zeros) a tile of 1 KiB in which lane l = 16g + i finds
+    w[16 * band + i][16 * chunk + 4g .. +4]; a stacked matrix is tiled as the one matrix it is.
+    Returns a flat tensor, or None for weights the few-row kernels do not take."""
     _dense(weight, "weight", _ACT)
     _need(weight.dim() == 2 and halves in (1, 2) and weight.shape[0] % halves == 0, "weight: expected [out, in]")
+    if weight.dtype == torch.float32:
+        n, k = weight.shape
+        if k % 4 != 0 or n == 0 or k < 4:
+            return None
+        tiles = torch.empty(tiled_size(n, k, torch.float32), dtype=weight.dtype, device=weight.device)
+        backend().tile_weight(weight, tiles)
+        return tiles
     n, k = weight.shape[0] // halves, weight.shape[1]
-    if weight.dtype != torch.bfloat16 or k % 32 != 0 or n == 0:
+    if k % 32 != 0 or n == 0:
         return None
     size = tiled_size(n, k)
     tiles = torch.empty(halves * size, dtype=weight.dtype, device=weight.device)
@@ -388,9 +401,13 @@ def tile_weight(weight: torch.Tensor, halves: int = 1) -> Optional[torch.Tensor]
 def _check_tiles(tiles, weight, halves: int) -> None:
     if tiles is None:
         return
+    if weight.dtype == torch.float32:
+        _need(weight.shape[1] % 4 == 0, "tiles: float32 weights have them only with in_features % 4 == 0")
+        _dense(tiles, "tiles", weight.dtype, (tiled_size(weight.shape[0], weight.shape[1], torch.float32),))
+        return
     n, k = weight.shape[0] // halves, weight.shape[1]
     _dense(tiles, "tiles", weight.dtype, (halves * tiled_size(n, k),))
-    _need(weight.dtype == torch.bfloat16 and k % 32 == 0, "tiles: only bfloat16 weights with in_features % 32 == 0 have them")
+    _need(k % 32 == 0, "tiles: bfloat16 weights have them only with in_features % 32 == 0")
 
 
 def linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, tiles: Optional[torch.Tensor] = None) -> None:

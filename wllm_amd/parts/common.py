@@ -43,8 +43,8 @@ def load_matrix(fetch, matrix: torch.Tensor, halves: int = 1):
     """A weight matrix on the device as the product kernels want it: (the matrix, row by row, for
     products of many rows; its tile-major copy for the few rows of a decode step, or None).  The
     copy doubles the weight's memory and is made only where the loader asks for it
-    (`fetch.tiled_copies`) and the few-row kernels take the weight (bfloat16, input size a
-    multiple of 32)."""
+    (`fetch.tiled_copies`) and the few-row kernels take the weight (bfloat16 with an input size that
+    is a multiple of 32, float32 with a multiple of 4)."""
     weight = fetch.to_device(matrix)
     tiles = ops.tile_weight(weight, halves) if getattr(fetch, "tiled_copies", False) else None
     return weight, tiles

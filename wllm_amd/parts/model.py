@@ -172,13 +172,13 @@ def build_model(raw_config: dict) -> CausalLM:
 
 def load_model(folder: str, dtype="bfloat16", device="cuda", tiled_copies: Optional[bool] = None) -> CausalLM:
     """A model folder (config.json, model.safetensors) to a loaded model.  `tiled_copies` (default:
-    yes for bfloat16) keeps a second copy of each matrix in the order the few-row product kernels
+    yes on a GPU) keeps a second copy of each matrix in the order the few-row product kernels
     of decode steps read fastest, at twice the matrices' memory."""
     dtype = resolve_dtype(dtype)
     model = build_model(read_config_json(folder))
     checkpoint = Checkpoint(folder)
     if tiled_copies is None:
-        tiled_copies = dtype == torch.bfloat16
+        tiled_copies = torch.device(device).type == "cuda"
     try:
         model.load(checkpoint, dtype, torch.device(device), tiled_copies=tiled_copies)
     finally:
