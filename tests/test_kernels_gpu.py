@@ -617,3 +617,44 @@ def test_gated_product_with_the_norm_on_load(tiled, act, m, inter, k, offset):
     with ops.use_backend(EmulatedKernels(precise=True)):
         ops.gated_linear(x, w, ref, act, None, tiles)
     close(out, ref, dtype, "against the emulation")
+
+
+def test_a_key_has_one_rounding_more_in_a_step_of_many_rows():
+    """Where queries and keys are rounded to bfloat16: once, after the rotation, in the fused projection of
+    a decode step; twice in a step of many rows (the library's product rounds the projection, the rotation
+    rounds again).  The same token's key and query, written by a step of 8 rows and by a step of 100, differ
+    by that one rounding and no more: every element within one step of the bfloat16 grid at the row's size
+    (2^-7 of the largest element), most of them equal."""
+    torch.manual_seed(21)
+    nh, nkv, d, ps, hidden = 4, 2, 64, 16, 256
+    width = (nh + 2 * nkv) * d
+    w = (torch.randn(width, hidden, device=DEV) / math.sqrt(hidden)).to(torch.bfloat16)
+    x = torch.randn(100, hidden, device=DEV).to(torch.bfloat16)
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).to(DEV)
+    kw = dict(num_heads=nh, num_kv_heads=nkv, head_dim=d, page_size=ps)
+
+    def run(rows):
+        positions = torch.arange(rows, device=DEV, dtype=torch.int32) + 37
+        slots = torch.arange(rows, device=DEV, dtype=torch.int32)
+        qkv = torch.zeros(rows, width, device=DEV, dtype=torch.bfloat16)
+        cache = torch.zeros(8, 2, nkv, ps * d, device=DEV, dtype=torch.bfloat16)
+        if ops.qkv_rope_takes(rows, torch.bfloat16, hidden, d, d):
+            ops.qkv_rope(x[:rows].contiguous(), w, qkv, None, positions, inv_freq, slots, cache, **kw)
+            path = "fused"
+        else:
+            ops.linear(x[:rows].contiguous(), w, qkv)
+            ops.rope_and_cache_write(qkv, None, positions, inv_freq, slots, cache, **kw)
+            path = "two kernels"
+        return qkv, cache, path
+
+    few, cache_few, path_few = run(8)
+    many, cache_many, path_many = run(100)
+    assert (path_few, path_many) == ("fused", "two kernels")
+    # what the cache holds is what the rows hold, in both
+    for qkv, cache, rows in ((few, cache_few, 8), (many, cache_many, 100)):
+        keys = cache[:, 0].view(8, nkv, ps, d).permute(0, 2, 1, 3).reshape(8 * ps, nkv * d)[:rows]
+        assert torch.equal(keys, qkv[:, nh * d:(nh + nkv) * d])
+    a, b = few.float(), many[:8].float()
+    grid = a.abs().amax(-1, keepdim=True) * 2.0 ** -7
+    assert ((a - b).abs() <= grid).all(), "more than one rounding apart"
+    assert (a == b).float().mean() > 0.5
