@@ -2,7 +2,9 @@
 through ctypes as a caller outside this package would call it, against the entry point it is a
 variant of (`wllm_sample_rows_split`, whose scratch area the caller allocates): two calls in a row,
 the second with a smaller input, give the same tokens and log-probabilities bit for bit; more rows
-than its maximum are refused with an error code that has a text."""
+than its maximum are refused with an error code that has a text.  Its tokens are also held against the
+plain sampler (tests/plain/sampling_plain.py), so that the check does not rest on another path of
+the library alone."""
 import ctypes
 from ctypes import c_char_p, c_int, c_void_p
 
@@ -78,6 +80,33 @@ def test_the_entry_point_without_allocation_gives_what_the_one_with_a_caller_buf
     _, tok, _ = _call(lib, True, *inputs)
     again = _call(lib, True, *inputs)[1]
     assert torch.equal(tok, again), "the last call's contents do not leak into the next"
+
+
+def test_the_entry_point_without_allocation_follows_the_plain_sampler():
+    """Every row's token is the one whose interval of the plain sampler's cumulative distribution holds
+    the row's uniform number (greedy rows: the argmax of the penalised logits), and its log-probability
+    is the plain sampler's."""
+    from plain import sampling_plain as S
+    lib = _library()
+    assert lib.wllm_sample_static_init() == 0
+    rows, vocab = 20, 1500
+    logits, params, seeds, ids, offsets = _inputs(rows, vocab, 6)
+    code, tokens, logprobs = _call(lib, True, logits, params, seeds, ids, offsets)
+    assert code == 0
+    for r in range(rows):
+        temperature, top_k, top_p, min_p, penalty = params[r].tolist()
+        generated = ids[int(offsets[r]):int(offsets[r + 1])].tolist()
+        u = S.philox_uniform(int(seeds[r, 0]), int(seeds[r, 1]))
+        token, logprob, keep, span = S.sample_row(logits[r].cpu(), temperature, int(top_k), top_p, min_p, penalty, generated, u)
+        got = int(tokens[r])
+        if temperature == 0.0:
+            assert got == token, f"row {r}"
+        else:
+            low, high = span
+            assert bool(keep[got]) and low[got] - 1e-4 <= u <= high[got] + 1e-4, f"row {r}: token {got} for u {u}"
+            logprob = float(torch.log_softmax(S.apply_repetition_penalty(logits[r].cpu().double(), generated, penalty)
+                                              / max(temperature, 1e-5), -1)[got])
+        assert abs(float(logprobs[r]) - logprob) < 1e-3, f"row {r}"
 
 
 def test_more_rows_than_the_maximum_are_refused_with_a_clear_error():
