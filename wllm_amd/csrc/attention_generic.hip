@@ -6,9 +6,11 @@
 // lo = max(0, p - window + 1).  The keys are cut into chunks of kChunkKeys keys counted from
 // key 0, so a chunk's boundaries depend on the key index alone.  One workgroup takes one
 // (token, key/value head, chunk); its eight wavefronts take 16 keys each, and a wavefront's
-// work is two trips to memory at most: the rows of its 16 keys (lane = key and quarter of the
-// head, 16-byte loads) and their values from the transposed page ([head_dim, page_size]; lane =
-// element of the head, four consecutive keys a load where pages are a multiple of four keys).
+// work is two trips to memory: the rows of its 16 keys (lane = key and quarter of the
+// head, 16-byte loads) and, asked for once the scores are made, their values from the transposed
+// page ([head_dim, page_size]; lane = element of the head, four consecutive keys a load where pages
+// are a multiple of four keys).  Keys and values are not held at once: at a head of 256 that is 126
+// registers instead of 168 and two workgroups a compute unit instead of one, which hide each other's trips.
 // The query heads of the group, up to 8 at a time, share each key and value read.  The
 // wavefronts' (maximum, sum, weighted sum) are merged through shared memory in wavefront
 // order.  A token whose keys lie in one chunk is finished there; otherwise the chunk's
@@ -22,6 +24,7 @@ constexpr int kChunkKeys = 128;       // keys per workgroup
 constexpr int kTileKeys = 16;         // keys per wavefront
 constexpr int kWaves = kChunkKeys / kTileKeys;
 constexpr int kMaxHeadDim = 256;
+constexpr int kMergeHeads = 4;        // heads whose weighted sums the wavefronts merge at a time
 
 template <typename T> struct Vec4;
 template <> struct Vec4<float> {
@@ -51,7 +54,7 @@ template <> struct Vec4<bf16> {
 // head per lane in the weighted sum (head_dim <= 64 * DPL); VEC4: pages hold a multiple of four
 // keys, so four consecutive keys' values of one element are one load.
 template <typename T, int NV, int DPL, bool VEC4>
-__global__ void __launch_bounds__(kWave * kWaves)
+__global__ void __launch_bounds__(kWave * kWaves, 4)
 paged_attention_generic_kernel(const T* __restrict__ qkv, const T* __restrict__ cache,
                                const int* __restrict__ block_tables, const int* __restrict__ token_segment,
                                const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
@@ -115,34 +118,6 @@ paged_attention_generic_kernel(const T* __restrict__ qkv, const T* __restrict__ 
         }
     }
     __syncthreads();                       // queries, offsets and slots are in shared memory
-    const int keys_before = key0 < lo ? lo - key0 : 0;                     // keys of the tile below the window
-    const int keys_end = min(kTileKeys, pos - key0 + 1);                   // keys of the tile up to the token's own
-    Vec4<T> vvec[DPL][kTileKeys / 4];
-#pragma unroll
-    for (int k = 0; k < DPL; ++k) {
-        const int d = lane + k * kWave;
-#pragma unroll
-        for (int jj = 0; jj < kTileKeys / 4; ++jj) {
-            const int j0 = jj * 4;
-            vvec[k][jj].zero();
-            if (d < head_dim && j0 < keys_end && j0 + 4 > keys_before) {
-                if (VEC4) {
-                    // four consecutive keys lie in one page; the first valid one says which
-                    const int jv = max(j0, keys_before);
-                    vvec[k][jj].load(cache + koff_s[jv] + v_off + static_cast<size_t>(d) * page_size + (slot_s[jv] - (jv - j0)));
-                } else {
-                    const T* p[4];
-#pragma unroll
-                    for (int u = 0; u < 4; ++u) {
-                        const int ju = min(max(j0 + u, keys_before), keys_end - 1);     // an invalid key reads a valid one's
-                        p[u] = cache + koff_s[ju] + v_off + static_cast<size_t>(d) * page_size + slot_s[ju];
-                    }
-                    vvec[k][jj].gather(p[0], p[1], p[2], p[3]);
-                }
-            }
-        }
-    }
-
     // ---- scores: a lane's part of the dot products, then the sum over the four lanes of a key ----
     float s[kGroupMax];
 #pragma unroll
@@ -179,6 +154,34 @@ paged_attention_generic_kernel(const T* __restrict__ qkv, const T* __restrict__ 
             if (c == 0) p_s[g * kTileKeys + j] = p;
         }
     }
+    const int keys_before = key0 < lo ? lo - key0 : 0;                     // keys of the tile below the window
+    const int keys_end = min(kTileKeys, pos - key0 + 1);                   // keys of the tile up to the token's own
+    Vec4<T> vvec[DPL][kTileKeys / 4];
+#pragma unroll
+    for (int k = 0; k < DPL; ++k) {
+        const int d = lane + k * kWave;
+#pragma unroll
+        for (int jj = 0; jj < kTileKeys / 4; ++jj) {
+            const int j0 = jj * 4;
+            vvec[k][jj].zero();
+            if (d < head_dim && j0 < keys_end && j0 + 4 > keys_before) {
+                if (VEC4) {
+                    // four consecutive keys lie in one page; the first valid one says which
+                    const int jv = max(j0, keys_before);
+                    vvec[k][jj].load(cache + koff_s[jv] + v_off + static_cast<size_t>(d) * page_size + (slot_s[jv] - (jv - j0)));
+                } else {
+                    const T* p[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int ju = min(max(j0 + u, keys_before), keys_end - 1);     // an invalid key reads a valid one's
+                        p[u] = cache + koff_s[ju] + v_off + static_cast<size_t>(d) * page_size + slot_s[ju];
+                    }
+                    vvec[k][jj].gather(p[0], p[1], p[2], p[3]);
+                }
+            }
+        }
+    }
+
     // lanes read below what other lanes of the wavefront wrote above: no reordering by the
     // scheduler, and the compiler is told that the memory changed
     __builtin_amdgcn_wave_barrier();
@@ -211,11 +214,12 @@ paged_attention_generic_kernel(const T* __restrict__ qkv, const T* __restrict__ 
         }
     }
 
-    // ---- merge the wavefronts, in their order: (m, l) of all heads at once, the weighted sums head
-    // by head through one buffer of [waves][head_dim] ----
+    // ---- merge the wavefronts, in their order: (m, l) of all heads at once, the weighted sums of
+    // kMergeHeads heads at a time through one buffer of [waves][kMergeHeads][head_dim] (two barriers a
+    // batch of heads: a head at a time they were 16 barriers for a group of 8, a third of the kernel) ----
     __syncthreads();
     float* ml_s = smem;                                              // [waves][g][2]
-    float* acc_s = smem + kWaves * kGroupMax * 2;                    // [waves][head_dim]
+    float* acc_s = smem + kWaves * kGroupMax * 2;                    // [waves][kMergeHeads][head_dim]
     if (lane == 0) {
 #pragma unroll
         for (int g = 0; g < kGroupMax; ++g) {
@@ -229,22 +233,27 @@ paged_attention_generic_kernel(const T* __restrict__ qkv, const T* __restrict__ 
     const size_t part_row = (static_cast<size_t>(blockIdx.x) * num_heads + head0) * max_chunks + chunk;
     const size_t part_stride = max_chunks;                          // between two heads of a token
 #pragma unroll
-    for (int g = 0; g < kGroupMax; ++g) {
-        if (g >= g_count) break;
+    for (int g0 = 0; g0 < kGroupMax; g0 += kMergeHeads) {
+        if (g0 >= g_count) break;
 #pragma unroll
-        for (int k = 0; k < DPL; ++k) {
-            const int d = lane + k * kWave;
-            if (d < head_dim) acc_s[wave * head_dim + d] = acc[g][k];
+        for (int gi = 0; gi < kMergeHeads; ++gi) {
+#pragma unroll
+            for (int k = 0; k < DPL; ++k) {
+                const int d = lane + k * kWave;
+                if (d < head_dim && g0 + gi < g_count) acc_s[(wave * kMergeHeads + gi) * head_dim + d] = acc[g0 + gi][k];
+            }
         }
         __syncthreads();
-        for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+        for (int e = threadIdx.x; e < kMergeHeads * head_dim; e += blockDim.x) {
+            const int gi = e / head_dim, d = e - gi * head_dim, g = g0 + gi;
+            if (g >= g_count) continue;
             float mm = -INFINITY;
             for (int w = 0; w < kWaves; ++w) mm = fmaxf(mm, ml_s[(w * kGroupMax + g) * 2]);
             float num = 0.f, den = 0.f;
             for (int w = 0; w < kWaves; ++w) {
                 const float mw = ml_s[(w * kGroupMax + g) * 2];
                 const float f = mw == -INFINITY ? 0.f : expf(mw - mm);
-                num = fmaf(acc_s[w * head_dim + d], f, num);
+                num = fmaf(acc_s[(w * kMergeHeads + gi) * head_dim + d], f, num);
                 den = fmaf(ml_s[(w * kGroupMax + g) * 2 + 1], f, den);
             }
             if (whole) {
@@ -294,7 +303,7 @@ paged_attention_generic_reduce_kernel(const float* __restrict__ partial_o, const
 static size_t generic_smem_bytes(int head_dim) {
     const size_t main_part = sizeof(float) * (kGroupMax * head_dim + kWaves * kGroupMax * kTileKeys) +
                              sizeof(long long) * kWaves * kTileKeys + sizeof(int) * kWaves * kTileKeys;
-    const size_t merge = sizeof(float) * (kWaves * kGroupMax * 2 + kWaves * head_dim);
+    const size_t merge = sizeof(float) * (kWaves * kGroupMax * 2 + kWaves * kMergeHeads * head_dim);
     return main_part > merge ? main_part : merge;
 }
 
