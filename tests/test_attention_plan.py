@@ -8,9 +8,9 @@ import pytest
 from wllm_amd.kernels import attention_plan as ap
 
 
-def covered(q_len, ctx_len, group, nkv, window, page_size, rows_per_item=64):
+def covered(q_len, ctx_len, group, nkv, window, page_size, rows_per_item=64, workgroup_slots=512):
     items, reduces, slots, prefill, prefill_rows = ap.build_work_items(
-        np.array(q_len), np.array(ctx_len), group, nkv, window, page_size, rows_per_item)
+        np.array(q_len), np.array(ctx_len), group, nkv, window, page_size, rows_per_item, workgroup_slots)
     assert prefill_rows == rows_per_item
     cover = {}          # (seg, kvh, row) -> list of (first key, end key, slot)
     slot_users = {}
@@ -83,8 +83,7 @@ def covered(q_len, ctx_len, group, nkv, window, page_size, rows_per_item=64):
 def test_every_pair_is_covered_once(seed, monkeypatch):
     rng = np.random.default_rng(seed)
     # small targets so that small cases split the way large ones do
-    monkeypatch.setattr(ap, "PREFILL_MIN_CHUNK", 128)
-    monkeypatch.setattr(ap, "PREFILL_TARGET_ITEMS", int(rng.choice([1, 8, 64, 1024])))
+    monkeypatch.setattr(ap, "PREFILL_MIN_PIECE", int(rng.choice([1, 4, 12])))
     monkeypatch.setattr(ap, "PREFILL_TABLE_PAGES", int(rng.choice([34, 1024])))
     group, nkv = int(rng.choice([1, 2, 3, 8, 17, 24, 32, 40])), int(rng.choice([1, 2, 3]))
     window = int(rng.choice([0, 0, 40, 300]))
@@ -92,7 +91,7 @@ def test_every_pair_is_covered_once(seed, monkeypatch):
     n = int(rng.integers(1, 5))
     q_len = [int(rng.choice([1, 2, 5, 17, 70, 130, 400])) for _ in range(n)]
     ctx_len = [q + int(rng.choice([0, 1, 31, 128, 500, 1500])) for q in q_len]
-    covered(q_len, ctx_len, group, nkv, window, page_size, int(rng.choice([64, 128])))
+    covered(q_len, ctx_len, group, nkv, window, page_size, int(rng.choice([64, 128])), int(rng.choice([2, 16, 128, 512])))
 
 
 def test_a_late_portion_of_a_long_prompt_is_split_over_the_keys():
@@ -101,6 +100,29 @@ def test_a_late_portion_of_a_long_prompt_is_split_over_the_keys():
     _, reduces, slots, prefill = covered([512], [2560], 8, 1, 0, 16)
     assert prefill.shape[0] >= 256
     assert slots > 0 and reduces.shape[0] == 512 * 8 // 16
+
+
+def test_prefill_items_fill_the_workgroup_slots_once_where_they_can():
+    """2,048 tokens of 8 heads on one key/value head: 256 blocks of rows over 1 to 64 groups of 32 keys.  The pieces
+    are as short as 512 workgroups allow, and the items come longest first, every second run of 256 turned round."""
+    _, _, _, prefill = covered([2048], [2048], 8, 1, 0, 16)
+    assert 400 < prefill.shape[0] <= 512
+    length = np.minimum(prefill[:, 4], (prefill[:, 2] + 63) // 8 + 1) - prefill[:, 3]     # up to the block's last row's key
+    assert length.max() <= 32 * ap.prefill_piece_length(np.arange(1, 65).repeat(4), 1, 512, 4096)
+    assert (np.diff(length[:256]) <= 0).all() and (np.diff(length[256:]) >= 0).all()
+    assert length[:256].min() >= length[256:].max()
+    # twice the prompt: 512 blocks of rows cannot be cut at all within one round, nor is any cut in two
+    _, reduces, slots, prefill = covered([4096], [4096], 8, 1, 0, 16)
+    assert prefill.shape[0] == 512 and slots == 0 and reduces.shape[0] == 0
+
+
+def test_piece_length():
+    span = np.array([64] * 8)
+    assert ap.prefill_piece_length(span, 1, 16, 128) == 32          # two pieces a block fill 16 slots
+    assert ap.prefill_piece_length(span, 2, 16, 128) == 64          # two heads: one piece a block
+    assert ap.prefill_piece_length(span, 4, 16, 128) == 64          # two rounds, uncut
+    assert ap.prefill_piece_length(span, 1, 512, 128) == ap.PREFILL_MIN_PIECE      # never shorter than this
+    assert ap.prefill_piece_length(span, 1, 4, 16) == 16            # the longest piece allowed: 4 a block, 8 rounds
 
 
 def test_a_whole_prompt_of_many_heads_is_not_split():

@@ -269,8 +269,8 @@ def test_paged_attention_matrix_cores(nh, nkv, d, ps, segs, window):
 def test_prompt_portions_whose_keys_are_split_over_workgroups(nh, nkv, d, ps, segs, window, small_pieces, monkeypatch):
     """Blocks of rows whose keys are cut into pieces, each piece a workgroup, combined by the reduce kernel."""
     from wllm_amd.kernels import attention_plan
-    if small_pieces:       # pieces of 128 keys, so that small cases are cut the way large ones are
-        monkeypatch.setattr(attention_plan, "PREFILL_MIN_CHUNK", 128)
+    if small_pieces:       # pieces down to 128 keys, so that small cases are cut the way large ones are
+        monkeypatch.setattr(attention_plan, "PREFILL_MIN_PIECE", 4)
     plan = _check_matrix_cores(nh, nkv, d, ps, segs, window)
     assert plan.num_prefill > 0 and plan.num_reduce > 0
     assert int((plan.prefill_items[:, 5] >= 0).sum()) > 0, "no block of rows was split"
@@ -281,7 +281,7 @@ def test_a_requests_attention_has_the_same_bits_alone_and_beside_a_long_prompt(m
     per element; both add a row's pieces in the same order, so a request's output does not change by
     a bit when a long prompt joins the step."""
     from wllm_amd.kernels import attention_plan
-    monkeypatch.setattr(attention_plan, "PREFILL_MIN_CHUNK", 128)
+    monkeypatch.setattr(attention_plan, "PREFILL_MIN_PIECE", 4)
     nh, nkv, d, ps = 8, 2, 64, 8
     dtype = torch.bfloat16
     args, kwargs = _attention_case(dtype, nh, nkv, d, ps, [(40, 700), (1, 600), (300, 900)], 0, seed=23)

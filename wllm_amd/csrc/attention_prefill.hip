@@ -326,9 +326,13 @@ paged_attention_prefill_kernel(const bf16* __restrict__ qkv, const bf16* __restr
 // straight to shared memory (lane l of a wavefront to base + 16 l), so staging costs no registers,
 // no writes to shared memory and no second barrier; two tiles of keys and values are held, and
 // the loads of block b+1 run while block b is multiplied.  Since a lane chooses its address, the
-// 16-byte chunks of a tile are placed so that fragment reads are free of bank conflicts: chunk c
-// of key row r lies at position c ^ (r % 8) of the row, chunk q (8 keys) of value row d at q ^
-// ((d / 2) % 4).  The keys of a block are staged in the order the second product wants them: row
+// 16-byte chunks of a tile are placed so that fragment reads are free of bank conflicts: the 16
+// lanes that read together (one chunk each of 16 rows) have to hit 16 different chunks of the 256
+// bytes that the banks span.  Chunk c of key row r lies at position c ^ (r % 16) of the row (heads
+// of 64, whose rows are 8 chunks and lie two to the 256 bytes: c ^ ((r / 2) % 8)), chunk q (8 keys)
+// of value row d at q ^ ((d / 2) % 4).  Measured with a loop of such reads alone, eight wavefronts a
+// compute unit: 4.0 clocks a read (256 bytes a clock), and 6.4 with c ^ (r % 8), where rows r and
+// r + 8 meet in the same banks.  The keys of a block are staged in the order the second product wants them: row
 // 16 t + 4 g + v of the tile holds key 8 g + 4 t + v, so that after the first product a lane's eight
 // scores are the keys 8 g .. 8 g + 7 of its row, the same eight keys that chunk g of a value row holds.
 // Nothing is cleared in flight: in the blocks at the edges of a request the stale keys' values are
@@ -453,13 +457,14 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
     const uint32_t page_bytes = static_cast<uint32_t>(page_elems * 2);
     // keys: wavefront load q = wave + 4 u of the tile carries the chunks 64 q .. 64 q + 63 of the tile in
     // shared-memory order
+    auto k_swizzle = [](int r) { return CPR >= 16 ? r % 16 : (r / 2) % 8; };      // what row r exchanges its chunks by
     int k_page[KU];
     const char* k_src[KU];
 #pragma unroll
     for (int u = 0; u < KU; ++u) {
         const int chunk_index = (wave + u * kPrefillWaves) * 64 + lane;       // position in the tile, in chunks
         const int r = chunk_index / CPR;                                      // row of the tile
-        const int chunk = (chunk_index % CPR) ^ (r % 8);                      // the chunk of the key's row that lies there
+        const int chunk = (chunk_index % CPR) ^ k_swizzle(r);                 // the chunk of the key's row that lies there
         const int rel = 8 * ((r % 16) / 4) + 4 * (r / 16) + r % 4;            // the key of the block that row r holds
         k_page[u] = rel >> shift;
         k_src[u] = reinterpret_cast<const char*>(cache + k_off + static_cast<size_t>(rel & mask) * HD + chunk * 8);
@@ -501,16 +506,18 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
     // One block: its tiles are k_s and v_s, the next block's loads go to k_next and v_next.  The loop below
     // names the two pairs of tiles in turn, so every address in shared memory is a constant plus a lane's
     // fixed offset.
-    // a lane's fragment reads: every address is the tile, the lane's offset and a constant.  Chunk (4 c + g)
-    // ^ (i % 8) of a key row is 4 (c ^ bit 2 of i) + (g ^ (i % 4)): an offset for even c and one for odd c.
-    const int k_lane_even = (i * CPR + 4 * ((i >> 2) & 1) + (g ^ (i & 3))) * 8;
-    const int k_lane_odd = (i * CPR + 4 * (1 - ((i >> 2) & 1)) + (g ^ (i & 3))) * 8;
+    // a lane's fragment reads: every address is the tile, the lane's offset and a constant.  With x what row i
+    // exchanges by, chunk (4 c + g) ^ x of a key row is 4 (c ^ (x >> 2)) + (g ^ (x & 3)), and x >> 2 touches the
+    // two low bits of c only: one offset for each c % 4.
+    const int k_x = k_swizzle(i);
+    int k_lane[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) k_lane[c] = (i * CPR + 4 * ((c ^ (k_x >> 2)) % DC) + (g ^ (k_x & 3))) * 8;
     const int v_lane = (i * 4 + (g ^ ((i / 2) % 4))) * 8;
     auto block = [&](int blk, const uint16_t* k_s, uint16_t* v_s, int next) {
         const int kbase = blk * kBlockKeys;
         __builtin_amdgcn_s_waitcnt(0);   // this lane's loads of the block have landed
         __syncthreads();                 // everyone's have, and everyone is done with the block before
-        if (blk + 1 < blk_end) issue(next, kbase + kBlockKeys);
         if (kbase + kBlockKeys > ctx || kbase < seg_lo) {
             // a block at the edge of the request: the values of keys that are not the request's are cleared
             if (tid < HD) {
@@ -521,21 +528,36 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
             }
             __syncthreads();
         }
-        if (!wave_active || kbase >= w_hi || kbase + kBlockKeys <= w_lo) return;
+        // The order below is kept as written (nothing moves across a sched_barrier): all fragments of the keys
+        // are asked for before the next block's loads are, the values' fragments before the softmax, so that
+        // a product waits for no read that was asked for just before it.  Left to itself the compiler keeps two
+        // reads in flight and every product waits a trip to shared memory.
+        const bool active = wave_active && kbase < w_hi && kbase + kBlockKeys > w_lo;
+        PPack kf[2 * DC], vf[DT];
+        if (active) {
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+                for (int c = 0; c < DC; ++c)
+                    kf[t2 * DC + c].u = *reinterpret_cast<const uint4*>(&k_s[k_lane[c % 4] + (16 * t2 * CPR + 4 * (c & ~3)) * 8]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (blk + 1 < blk_end) issue(next, kbase + kBlockKeys);
+        if (!active) return;
+        __builtin_amdgcn_sched_barrier(0);
         // ---- scores: tile t2, lane (i, g) gets the keys 8 g + 4 t2 + v of the block ----
         float sv[8];
 #pragma unroll
         for (int t2 = 0; t2 < 2; ++t2) {
             float4_t sc = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int c = 0; c < DC; ++c) {
-                PPack a;
-                a.u = *reinterpret_cast<const uint4*>(&k_s[((c & 1) ? k_lane_odd : k_lane_even) + (16 * t2 * CPR + 4 * (c & ~1)) * 8]);
-                sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qreg[c], sc, 0, 0, 0);
-            }
+            for (int c = 0; c < DC; ++c) sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t2 * DC + c].v, qreg[c], sc, 0, 0, 0);
 #pragma unroll
             for (int v = 0; v < 4; ++v) sv[4 * t2 + v] = sc[v];
         }
+#pragma unroll
+        for (int t = 0; t < DT; ++t) vf[t].u = *reinterpret_cast<const uint4*>(&v_s[v_lane + 16 * t * 4 * 8]);
+        __builtin_amdgcn_sched_barrier(0);
         // ---- softmax bookkeeping ----
         const bool inside = kbase + kBlockKeys - 1 <= t_pos_min && kbase >= t_lo_max;
         if (!inside) {
@@ -568,12 +590,9 @@ paged_attention_prefill_dma_kernel(const bf16* __restrict__ qkv, const bf16* __r
 #pragma unroll
             for (int t = 0; t < DT; ++t) acc[t] *= alpha;
         }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int t = 0; t < DT; ++t) {
-            PPack a;
-            a.u = *reinterpret_cast<const uint4*>(&v_s[v_lane + 16 * t * 4 * 8]);
-            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pv.v, acc[t], 0, 0, 0);
-        }
+        for (int t = 0; t < DT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[t].v, pv.v, acc[t], 0, 0, 0);
     };
     for (int blk = blk_first; blk < blk_end; blk += 2) {
         block(blk, k_s0, v_s0, 1);

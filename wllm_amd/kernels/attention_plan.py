@@ -34,8 +34,8 @@ KEY_CHUNK = 128
 ROWS_PER_TILE = 16
 ITEM_INTS = 8
 PREFILL_TABLE_PAGES = 1024      # pages one prefill item may span (the kernel's shared block table)
-PREFILL_TARGET_ITEMS = 1024     # prefill items wanted in a step: about four for each compute unit
-PREFILL_MIN_CHUNK = 512         # keys; smaller pieces cost more in partial results than they gain
+PREFILL_MIN_PIECE = 16          # groups of 32 keys; shorter pieces cost more in partial results than they gain
+WORKGROUP_SLOTS = 512           # prefill workgroups a device runs at once unless the caller knows better (two a compute unit)
 PREFILL_ROWS = 64               # rows of a prefill item unless the kernel for the sizes at hand says otherwise
 
 
@@ -110,8 +110,30 @@ def row_tiles(q_len: int, group: int) -> int:
 MAX_HEADS = 1 << 16     # an item packs the key/value head and the tile's first row into 16 bits each
 
 
+def prefill_piece_length(span: np.ndarray, num_kv_heads: int, workgroup_slots: int, longest: int) -> int:
+    """The most groups of 32 keys a prefill item gets, for blocks of rows that span `span` groups each
+    (per key/value head).  The shortest length with which the items fill the workgroup slots of the
+    device at most once, twice, ... (the fewest rounds that the longest allowed piece permits): every
+    further item costs a partial result that is written and read again, and items that start together
+    and are about equally long end together.  Never shorter than `PREFILL_MIN_PIECE` groups, below which
+    a piece's partial result costs more than its share of the keys."""
+    def count(length):
+        return int((-(-span // length)).sum()) * num_kv_heads
+    rounds = 1
+    while count(longest) > rounds * workgroup_slots:
+        rounds += 1
+    lo, hi = 1, longest                      # the least length whose count fits
+    while lo < hi:
+        mid = (lo + hi) // 2
+        if count(mid) <= rounds * workgroup_slots:
+            hi = mid
+        else:
+            lo = mid + 1
+    return min(longest, max(lo, PREFILL_MIN_PIECE))
+
+
 def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_heads: int, window: int,
-                     page_size: int = 16, prefill_rows: int = PREFILL_ROWS):
+                     page_size: int = 16, prefill_rows: int = PREFILL_ROWS, workgroup_slots: int = WORKGROUP_SLOTS):
     """Returns (items [n, 8], reduce_items [m, 8], partial slots, prefill items [p, 8], rows per
     prefill item) as int32 arrays."""
     q_len = np.asarray(q_len, dtype=np.int64)
@@ -174,66 +196,68 @@ def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_
             reduces.append(rs[keep_r].reshape(-1, ITEM_INTS))
         slots = int((n_split_seg * num_kv_heads * rt).sum())
     # ---- long segments: workgroups of 64 or 128 rows of one key/value head ----
-    prefill = []
+    prefill = np.zeros((0, ITEM_INTS), np.int32)
     long_idx = np.nonzero(~short)[0]
     if long_idx.size:
-        blocks = []              # (segment, first rows, lowest key, end key) per long segment
-        span_total = 0
-        for s in long_idx:
-            n_blocks = -(-int(rows[s]) // prefill_rows)
-            rb = np.arange(n_blocks, dtype=np.int64) * prefill_rows
-            first_pos = int(ctx_len[s] - q_len[s])
-            hi = first_pos + np.minimum(rows[s] - 1, rb + prefill_rows - 1) // group + 1
-            lo = np.maximum(0, first_pos + rb // group - window + 1) if window > 0 else np.zeros_like(rb)
-            blocks.append((int(s), rb, lo, hi))
-            span_total += int((hi - lo).sum()) * num_kv_heads
-        tiles = prefill_rows // ROWS_PER_TILE
+        # the blocks of rows of all long segments, one after the other
+        n_blocks = -(-rows[long_idx] // prefill_rows)
+        seg_of = np.repeat(long_idx, n_blocks)
+        rb = (np.arange(int(n_blocks.sum())) - np.repeat(np.cumsum(n_blocks) - n_blocks, n_blocks)) * prefill_rows
+        first_pos = (ctx_len - q_len)[seg_of]
+        hi = first_pos + np.minimum(rows[seg_of] - 1, rb + prefill_rows - 1) // group + 1
+        lo = np.maximum(0, first_pos + rb // group - window + 1) if window > 0 else np.zeros_like(rb)
+        # a block's keys are cut into equal pieces whose boundaries are multiples of 32 counted from the block's
+        # first group of 32
+        lo32 = lo // 32 * 32
+        span = -(-(hi - lo32) // 32)                                                  # in groups of 32 keys
         # a piece that starts inside a page touches up to two pages more than its keys fill
-        max_chunk = max(KEY_CHUNK, (PREFILL_TABLE_PAGES - 2) * page_size // KEY_CHUNK * KEY_CHUNK)
-        chunk = -(-span_total // (PREFILL_TARGET_ITEMS * KEY_CHUNK)) * KEY_CHUNK
-        chunk = min(max(chunk, PREFILL_MIN_CHUNK), max_chunk)
-        for s, rb, lo, hi in blocks:
-            # a block's keys are cut into pieces of about `chunk` keys, equal within the block,
-            # whose boundaries are multiples of 32 counted from the block's first group of 32
-            lo32 = lo // 32 * 32
-            span = hi - lo32
-            # no piece longer than `chunk`: the longest piece is what the last workgroups wait for
-            ns = np.maximum(np.maximum(1, -(-span // chunk)), -(-span // max_chunk))   # items per block
-            piece = -(-span // (ns * 32)) * 32
-            ns = -(-span // piece)
-            n_items = int(ns.sum())
-            block_of = np.repeat(np.arange(rb.size), ns)
-            j = np.arange(n_items) - np.repeat(np.cumsum(ns) - ns, ns)
-            split = ns > 1
-            # slots of a split block: [split][tile], blocks one after the other, per key/value head
-            block_slots = np.where(split, ns * tiles, 0)
-            block_base = np.cumsum(block_slots) - block_slots
-            per_head = int(block_slots.sum())
-            it = np.zeros((num_kv_heads, n_items, ITEM_INTS), dtype=np.int32)
-            it[..., 0] = s
-            it[..., 1] = kv[:, None]
-            it[..., 2] = rb[block_of][None, :]
-            it[..., 3] = (lo32[block_of] + j * piece[block_of])[None, :]
-            it[..., 4] = (lo32[block_of] + (j + 1) * piece[block_of])[None, :]
-            slot = slots + kv[:, None] * per_head + (block_base[block_of] + j * tiles)[None, :]
-            it[..., 5] = np.where(split[block_of][None, :], slot, -1)
-            # the last rows see the most keys: start them first
-            prefill.append(it[:, ::-1].reshape(-1, ITEM_INTS))
-            sb = np.nonzero(split)[0]
-            if sb.size:
-                t = np.arange(tiles, dtype=np.int64)
-                first_row = rb[sb][:, None] + t[None, :] * ROWS_PER_TILE           # [blocks, tiles]
-                live = first_row < rows[s]
-                rs = np.zeros((num_kv_heads, sb.size, tiles, ITEM_INTS), dtype=np.int32)
-                rs[..., 0] = s
-                rs[..., 1] = kv[:, None, None]
-                rs[..., 2] = slots + kv[:, None, None] * per_head + (block_base[sb][:, None] + t[None, :])[None]
-                rs[..., 3] = ns[sb][None, :, None]
-                rs[..., 4] = first_row[None]
-                rs[..., 5] = tiles
-                reduces.append(rs[:, live].reshape(-1, ITEM_INTS))
-            slots += per_head * num_kv_heads
-    prefill = np.concatenate(prefill) if prefill else np.zeros((0, ITEM_INTS), np.int32)
+        longest = max(KEY_CHUNK, (PREFILL_TABLE_PAGES - 2) * page_size // KEY_CHUNK * KEY_CHUNK) // 32
+        ns = -(-span // prefill_piece_length(span, num_kv_heads, workgroup_slots, longest))
+        piece = -(-span // ns)
+        ns = -(-span // piece)
+        tiles = prefill_rows // ROWS_PER_TILE
+        n_items = int(ns.sum())
+        block_of = np.repeat(np.arange(rb.size), ns)
+        j = np.arange(n_items) - np.repeat(np.cumsum(ns) - ns, ns)
+        split = ns > 1
+        # slots of a split block: [split][tile], blocks one after the other, per key/value head
+        block_slots = np.where(split, ns * tiles, 0)
+        block_base = np.cumsum(block_slots) - block_slots
+        per_head = int(block_slots.sum())
+        it = np.zeros((num_kv_heads, n_items, ITEM_INTS), dtype=np.int32)
+        it[..., 0] = seg_of[block_of][None, :]
+        it[..., 1] = kv[:, None]
+        it[..., 2] = rb[block_of][None, :]
+        it[..., 3] = (lo32[block_of] + j * piece[block_of] * 32)[None, :]
+        it[..., 4] = (lo32[block_of] + (j + 1) * piece[block_of] * 32)[None, :]
+        slot = slots + kv[:, None] * per_head + (block_base[block_of] + j * tiles)[None, :]
+        it[..., 5] = np.where(split[block_of][None, :], slot, -1)
+        it = it.reshape(-1, ITEM_INTS)
+        # The workgroups start in the order of the items, the first ones one on each compute unit, the next ones
+        # beside them: the longest pieces come first, and each further run of `workgroup_slots / 2` turns round,
+        # so that a long piece gets a short one for its neighbour and the last to start are the shortest.
+        length = np.minimum(it[:, 4], hi[block_of][None, :].repeat(num_kv_heads, 0).reshape(-1)) - it[:, 3]
+        order = np.argsort(-length, kind="stable")
+        run = max(1, workgroup_slots // 2)
+        turned = (np.arange(order.size) // run) % 2 == 1
+        place = np.arange(order.size)
+        run_first = place // run * run
+        run_last = np.minimum(run_first + run, order.size) - 1
+        prefill = it[order[np.where(turned, run_first + run_last - place, place)]]
+        sb = np.nonzero(split)[0]
+        if sb.size:
+            t = np.arange(tiles, dtype=np.int64)
+            first_row = rb[sb][:, None] + t[None, :] * ROWS_PER_TILE           # [blocks, tiles]
+            live = first_row < rows[seg_of[sb]][:, None]
+            rs = np.zeros((num_kv_heads, sb.size, tiles, ITEM_INTS), dtype=np.int32)
+            rs[..., 0] = seg_of[sb][None, :, None]
+            rs[..., 1] = kv[:, None, None]
+            rs[..., 2] = slots + kv[:, None, None] * per_head + (block_base[sb][:, None] + t[None, :])[None]
+            rs[..., 3] = ns[sb][None, :, None]
+            rs[..., 4] = first_row[None]
+            rs[..., 5] = tiles
+            reduces.append(rs[:, live].reshape(-1, ITEM_INTS))
+        slots += per_head * num_kv_heads
     items = np.concatenate(items) if items else np.zeros((0, ITEM_INTS), np.int32)
     reduces = np.concatenate(reduces) if reduces else np.zeros((0, ITEM_INTS), np.int32)
     return items, reduces, slots, prefill, prefill_rows

@@ -72,6 +72,7 @@ class HipBackend:
         self.lib = load()
         self._device_index = torch.cuda.current_device()
         self._partial_o = None
+        self._slots_of = {}                # device -> workgroups of the prompt kernel it runs at once
         self._gemm_partials = None
         self._argmax_scratch = None
         self._sample_scratch = None
@@ -177,7 +178,8 @@ class HipBackend:
         if not self.mfma_attention_takes(dtype, head_dim, page_size):
             return None
         items, reduces, slots, prefill, prefill_rows = build_work_items(
-            host_q_len, host_ctx_len, num_heads // num_kv_heads, num_kv_heads, window, page_size)
+            host_q_len, host_ctx_len, num_heads // num_kv_heads, num_kv_heads, window, page_size,
+            workgroup_slots=self._workgroup_slots(device))
         flat = np.concatenate([items.reshape(-1), reduces.reshape(-1), prefill.reshape(-1)])
         dev = pack_int32([flat], device)[0]
         n_i, n_r, n_p = items.shape[0], reduces.shape[0], prefill.shape[0]
@@ -186,6 +188,13 @@ class HipBackend:
         return AttentionPlan(dev[:a].view(n_i, 8), dev[a:b].view(n_r, 8) if n_r else None, n_i, n_r, slots,
                              self._partial_o, self._partial_ml, dev[b:].view(n_p, 8) if n_p else None, n_p,
                              prefill_rows)
+
+    def _workgroup_slots(self, device) -> int:
+        """Workgroups of the kernel for prompt portions that the device runs at once: two a compute unit."""
+        key = torch.device(device)
+        if key not in self._slots_of:
+            self._slots_of[key] = 2 * torch.cuda.get_device_properties(key).multi_processor_count
+        return self._slots_of[key]
 
     def static_attention_plan(self, segments, num_heads, num_kv_heads, head_dim, page_size, window, dtype, device,
                               max_context: int, max_total_keys: int):
