@@ -20,7 +20,9 @@ segments, 64 rows each, for the kernel that stages keys and values through share
 unused.  The keys of a block of rows are split over several prefill items when the step has too
 few blocks to fill the compute units (a portion of a prompt late in a long context) or when they
 span more pages than the kernel's shared copy of the block table holds; the pieces of a block are
-equal and begin at multiples of 32 keys.
+equal and begin at multiples of 32 keys (`prefill_piece_length` chooses how long).  The prefill
+items of a step are ordered by length, longest first, every second run of as many as the device has
+compute units turned round: workgroups start in this order.
 """
 from __future__ import annotations
 
