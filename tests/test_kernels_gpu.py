@@ -235,6 +235,22 @@ def test_paged_attention(dtype, nh, nkv, d, ps, segs, window):
     close(g[7], r[7], dtype, "attention output")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_context_bound_that_is_too_low_shows(dtype):
+    """The general kernel sizes its grid by the caller's bound on the context lengths, which themselves are in
+    device memory.  Tokens whose keys reach beyond the bound come out as NaN, never as attention over fewer keys;
+    the other tokens are what they are with the right bound."""
+    args, kwargs = _attention_case(dtype, 4, 2, 40, 8, [(3, 130), (2, 300), (1, 640)], 0)
+    ops.paged_attention(*args, **kwargs)
+    right = args[7].clone()
+    assert torch.isfinite(right.float()).all()
+    args[7].zero_()
+    ops.paged_attention(*args, **dict(kwargs, max_ctx_len=256))        # chunks of 128 keys: positions 256.. are cut
+    got = args[7].float()
+    assert torch.equal(args[7][:3], right[:3])                          # positions 127..129
+    assert torch.isnan(got[3:]).all()                                   # positions 298, 299 and 639
+
+
 MFMA_SHAPES = ATTENTION_SHAPES + [
     (8, 1, 256, 16, [(1, 2048), (1, 700), (1, 257), (1, 256), (1, 255)], 0),      # decoded tokens, keys split over workgroups
     (8, 1, 256, 16, [(2048, 2048)], 0),                                           # a whole prompt

@@ -69,6 +69,9 @@ paged_attention_generic_kernel(const T* __restrict__ qkv, const T* __restrict__ 
     const int lo = window > 0 ? max(0, pos - window + 1) : 0;
     const int c_lo = lo / kChunkKeys, c_hi = min(pos / kChunkKeys, max_chunks - 1);   // the bound keeps every access inside the buffers
     if (chunk < c_lo || chunk > c_hi) return;
+    // the caller's bound on the context lengths was below this token's: its keys beyond the bound are not
+    // read, and its result is made NaN (through the last chunk's sums), not a number that looks right
+    const bool cut_short = pos / kChunkKeys > max_chunks - 1;
 
     extern __shared__ float smem[];
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
@@ -256,6 +259,7 @@ paged_attention_generic_kernel(const T* __restrict__ qkv, const T* __restrict__ 
                 num = fmaf(acc_s[(w * kMergeHeads + gi) * head_dim + d], f, num);
                 den = fmaf(ml_s[(w * kGroupMax + g) * 2 + 1], f, den);
             }
+            if (cut_short) num = __builtin_nanf("");
             if (whole) {
                 orow[g * head_dim + d] = from_float<T>(num / den);
             } else {
@@ -311,7 +315,8 @@ static size_t generic_smem_bytes(int head_dim) {
 WLLM_API int wllm_paged_attention_generic_chunk_keys() { return kChunkKeys; }
 
 // Returns 0, a HIP error code, or -1 for a size the kernel does not take.  `max_ctx_len` bounds every
-// segment's context length (it sets the number of chunks in the grid).  partial_o holds
+// segment's context length (it sets the number of chunks in the grid; the lengths themselves are in
+// device memory, so a bound that is too low shows as NaN in the tokens it cuts short).  partial_o holds
 // partial_tokens * num_heads * max_chunks * head_dim floats and partial_ml partial_tokens * num_heads *
 // max_chunks * 2, with max_chunks = ceil(max_ctx_len / chunk keys); the tokens run in launches of
 // at most `partial_tokens`.
