@@ -121,9 +121,7 @@ def prefill_piece_length(span: np.ndarray, num_kv_heads: int, workgroup_slots: i
     a piece's partial result costs more than its share of the keys."""
     def count(length):
         return int((-(-span // length)).sum()) * num_kv_heads
-    rounds = 1
-    while count(longest) > rounds * workgroup_slots:
-        rounds += 1
+    rounds = max(1, -(-count(longest) // workgroup_slots))
     lo, hi = 1, longest                      # the least length whose count fits
     while lo < hi:
         mid = (lo + hi) // 2
