@@ -8,9 +8,10 @@ import pytest
 from wllm_amd.kernels import attention_plan as ap
 
 
-def covered(q_len, ctx_len, group, nkv, window, page_size, rows_per_item=64, workgroup_slots=512):
+def covered(q_len, ctx_len, group, nkv, window, page_size, rows_per_item=64, workgroup_slots=512, tiles_only=False):
     items, reduces, slots, prefill, prefill_rows = ap.build_work_items(
-        np.array(q_len), np.array(ctx_len), group, nkv, window, page_size, rows_per_item, workgroup_slots)
+        np.array(q_len), np.array(ctx_len), group, nkv, window, page_size, rows_per_item, workgroup_slots, tiles_only)
+    assert not (tiles_only and prefill.shape[0])
     assert prefill_rows == rows_per_item
     cover = {}          # (seg, kvh, row) -> list of (first key, end key, slot)
     slot_users = {}
@@ -20,10 +21,10 @@ def covered(q_len, ctx_len, group, nkv, window, page_size, rows_per_item=64, wor
         slot_users[slot] = who
     for n, it in enumerate(items):
         seg, head_and_row, new_tokens, first_token, kb, ke, slot, context = (int(v) for v in it)
-        kvh, row0 = head_and_row & 0xffff, head_and_row >> 16
+        kvh, row0 = head_and_row & 0xffff, (head_and_row >> 16) * 16      # the tile's number in the high 16 bits
         rows = q_len[seg] * group
         # short: at most 16 rows, or one token whose group of heads fills several tiles of 16
-        assert rows <= 16 or q_len[seg] == 1
+        assert rows <= 16 or q_len[seg] == 1 or tiles_only
         assert row0 % 16 == 0 and row0 < rows
         # the item carries the segment's lengths and the place of its first token in the step
         assert new_tokens == q_len[seg] and context == ctx_len[seg] and first_token == sum(q_len[:seg])
@@ -137,7 +138,31 @@ def test_a_decoded_token_of_a_large_group_stays_short():
     so a captured decode graph can hold it."""
     items, reduces, slots, prefill = covered([1, 1, 1], [50, 300, 129], 40, 2, 0, 16)
     assert prefill.shape[0] == 0
-    assert sorted(set(int(v) >> 16 for v in items[:, 1])) == [0, 16, 32]
+    assert sorted(set(int(v) >> 16 for v in items[:, 1])) == [0, 1, 2]
     # 1 + 3 + 2 chunks of keys, for 2 key/value heads and 3 tiles of rows
     assert items.shape[0] == (1 + 3 + 2) * 2 * 3
     assert reduces.shape[0] == 2 * 2 * 3 and slots == (3 + 2) * 2 * 3
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_tiles_only_covers_every_pair_once(seed):
+    """The float32 kernel's plan: every segment, prompts too, as tiles of 16 rows with chunks of 128 keys."""
+    rng = np.random.default_rng(100 + seed)
+    group, nkv = int(rng.choice([1, 2, 3, 8, 17, 24])), int(rng.choice([1, 2, 3]))
+    window = int(rng.choice([0, 0, 40, 300]))
+    n = int(rng.integers(1, 5))
+    q_len = [int(rng.choice([1, 2, 5, 17, 70, 130, 400])) for _ in range(n)]
+    ctx_len = [q + int(rng.choice([0, 1, 31, 128, 500, 1500])) for q in q_len]
+    items, reduces, slots, prefill = covered(q_len, ctx_len, group, nkv, window, 16, tiles_only=True)
+    assert prefill.shape[0] == 0 and items.shape[0] > 0
+
+
+def test_a_prompts_tiles_stop_at_their_last_rows_position():
+    # 300 tokens of one head: tile 0 (tokens 0..15) needs keys 0..15 only, the last tile (tokens 288..299) keys 0..299
+    items, reduces, slots, _ = covered([300], [300], 1, 1, 0, 16, tiles_only=True)
+    by_tile = {}
+    for it in items:
+        by_tile.setdefault(int(it[1]) >> 16, []).append((int(it[4]), int(it[5])))
+    assert by_tile[0] == [(0, 16)]
+    assert sorted(by_tile[18]) == [(0, 128), (128, 256), (256, 300)]
+    assert len(by_tile) == 19

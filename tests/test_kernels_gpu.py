@@ -269,10 +269,19 @@ MFMA_SHAPES = ATTENTION_SHAPES + [
 ]
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nh,nkv,d,ps,segs,window", MFMA_SHAPES)
-def test_paged_attention_matrix_cores(nh, nkv, d, ps, segs, window):
-    """The bfloat16 kernel the engine uses for these sizes (with its plan of work items)."""
-    _check_matrix_cores(nh, nkv, d, ps, segs, window)
+def test_paged_attention_matrix_cores(dtype, nh, nkv, d, ps, segs, window):
+    """The kernels the engine uses for these sizes, with their plan of work items: in bfloat16 tiles of 16 rows for
+    decoded tokens and blocks of 64 rows for prompts, in float32 tiles of 16 rows for everything."""
+    _check_matrix_cores(nh, nkv, d, ps, segs, window, dtype)
+
+
+def test_float32_matrix_cores_on_a_whole_prompt():
+    """2,048 tokens of 8 heads on one key head in float32: 1,024 tiles of rows, 8,704 work items, and the reduce
+    kernel for every tile beyond the first 128 keys."""
+    plan = _check_matrix_cores(8, 1, 256, 16, [(2048, 2048)], 0, torch.float32)
+    assert plan.num_prefill == 0 and plan.num_items == 8704 and plan.num_reduce == 1024 - 64
 
 
 @pytest.mark.parametrize("nh,nkv,d,ps,segs,window,small_pieces", [
@@ -314,8 +323,7 @@ def test_a_requests_attention_has_the_same_bits_alone_and_beside_a_long_prompt(m
     assert torch.equal(alone[7], beside)
 
 
-def _check_matrix_cores(nh, nkv, d, ps, segs, window):
-    dtype = torch.bfloat16
+def _check_matrix_cores(nh, nkv, d, ps, segs, window, dtype=torch.bfloat16):
     args, kwargs = _attention_case(dtype, nh, nkv, d, ps, segs, window, seed=11)
     ref_args = [a.clone() for a in args]
     kw = _with_plan(args, kwargs)
@@ -337,6 +345,8 @@ def _check_matrix_cores(nh, nkv, d, ps, segs, window):
         ops.paged_attention(*ref_args, **kwargs)
     assert torch.isfinite(args[7].float()).all()
     close(args[7], ref_args[7], dtype, "attention output")
+    if dtype == torch.float32 and expect_plan:
+        assert kw["plan"].num_prefill == 0
     return kw["plan"]
 
 

@@ -89,7 +89,7 @@ paged_attention_mfma_kernel(const bf16* __restrict__ qkv, const bf16* __restrict
     const int key_begin = item[4], key_end = item[5], partial_slot = item[6], ctx = item[7];
     const int live = live_items != nullptr ? live_items[0] : 0x7fffffff;
     if (static_cast<int>(blockIdx.x) >= live) return;
-    const int row_begin = item[1] >> 16;      // the tile's first row: 0 unless a token has more than 16 heads a group
+    const int row_begin = (item[1] >> 16) * kRowsPerTile;      // the tile's first row: 0 unless a token has more than 16 heads a group
     if (seg < 0) return;    // padding item
     const int lane = threadIdx.x % kWave;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);

@@ -8,8 +8,8 @@ partial results combined by a second kernel; chunk boundaries are multiples of t
 counted from key 0, so they depend on the key index only.  Longer segments are cut into
 workgroups of four tiles of 16 rows (prefill items).
 
-A work item is 8 int32: segment, key/value head in the low 16 bits with the tile's first row in the
-high 16, the segment's number of new tokens, the place of
+A work item is 8 int32: segment, key/value head in the low 16 bits with the tile's number (its first
+row / 16) in the high 16, the segment's number of new tokens, the place of
 its first token among the step's tokens, first key, end key, partial slot (-1: the workgroup writes
 the final result), the segment's context length: what the kernel needs of the segment comes with
 the item, in the one read it begins with, and not from the segments' arrays in a second trip to memory.  A partial slot holds
@@ -109,7 +109,58 @@ def row_tiles(q_len: int, group: int) -> int:
     return -(-(q_len * group) // ROWS_PER_TILE)
 
 
-MAX_HEADS = 1 << 16     # an item packs the key/value head and the tile's first row into 16 bits each
+MAX_HEADS = 1 << 16     # an item packs the key/value head and the tile's number into 16 bits each
+MAX_TILES = 1 << 15     # tiles of 16 rows a segment may have for one key/value head (the item's int32 stays positive)
+
+
+def build_tile_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_heads: int, window: int):
+    """Every segment, whatever its length, as tiles of 16 rows with their keys in chunks of `KEY_CHUNK`
+    counted from key 0 (the float32 kernel takes nothing else): a tile's chunks are those its rows can
+    need, from the lowest key of its first row's window to its last row's position.  Returns (items
+    [n, 8], reduce items [m, 8], partial slots) in the format of the short segments' items."""
+    q_len = np.asarray(q_len, dtype=np.int64)
+    ctx_len = np.asarray(ctx_len, dtype=np.int64)
+    rows = q_len * group
+    q_start = np.cumsum(q_len) - q_len
+    nt = -(-rows // ROWS_PER_TILE)
+    if nt.size and int(nt.max()) >= MAX_TILES:
+        raise ValueError(f"a segment of {int(rows.max())} rows a key/value head: a work item numbers at most {MAX_TILES} tiles")
+    seg_of = np.repeat(np.arange(q_len.size), nt)
+    tile = np.arange(int(nt.sum())) - np.repeat(np.cumsum(nt) - nt, nt)
+    row0 = tile * ROWS_PER_TILE
+    first_pos = (ctx_len - q_len)[seg_of]
+    last_row = np.minimum(rows[seg_of] - 1, row0 + ROWS_PER_TILE - 1)
+    lo = np.maximum(0, first_pos + row0 // group - window + 1) if window > 0 else np.zeros_like(row0)
+    hi = first_pos + last_row // group + 1
+    c0 = lo // KEY_CHUNK
+    ns = (hi - 1) // KEY_CHUNK - c0 + 1
+    n_items = int(ns.sum())
+    tile_of = np.repeat(np.arange(tile.size), ns)
+    j = np.arange(n_items) - np.repeat(np.cumsum(ns) - ns, ns)
+    chunk = c0[tile_of] + j
+    split = ns > 1
+    tile_slots = np.where(split, ns, 0)
+    tile_base = np.cumsum(tile_slots) - tile_slots
+    per_head = int(tile_slots.sum())
+    kv = np.arange(num_kv_heads, dtype=np.int64)
+    it = np.zeros((num_kv_heads, n_items, ITEM_INTS), dtype=np.int32)
+    it[..., 0] = seg_of[tile_of][None, :]
+    it[..., 1] = kv[:, None] | (tile[tile_of] << 16)[None, :]
+    it[..., 2] = q_len[seg_of[tile_of]][None, :]
+    it[..., 3] = q_start[seg_of[tile_of]][None, :]
+    it[..., 4] = np.maximum(lo[tile_of], chunk * KEY_CHUNK)[None, :]
+    it[..., 5] = np.minimum(hi[tile_of], (chunk + 1) * KEY_CHUNK)[None, :]
+    it[..., 6] = np.where(split[tile_of][None, :], kv[:, None] * per_head + (tile_base[tile_of] + j)[None, :], -1)
+    it[..., 7] = ctx_len[seg_of[tile_of]][None, :]
+    st = np.nonzero(split)[0]
+    rs = np.zeros((num_kv_heads, st.size, ITEM_INTS), dtype=np.int32)
+    rs[..., 0] = seg_of[st][None, :]
+    rs[..., 1] = kv[:, None]
+    rs[..., 2] = kv[:, None] * per_head + tile_base[st][None, :]
+    rs[..., 3] = ns[st][None, :]
+    rs[..., 4] = row0[st][None, :]
+    rs[..., 5] = 1
+    return it.reshape(-1, ITEM_INTS), rs.reshape(-1, ITEM_INTS), per_head * num_kv_heads
 
 
 def prefill_piece_length(span: np.ndarray, num_kv_heads: int, workgroup_slots: int, longest: int) -> int:
@@ -133,9 +184,16 @@ def prefill_piece_length(span: np.ndarray, num_kv_heads: int, workgroup_slots: i
 
 
 def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_heads: int, window: int,
-                     page_size: int = 16, prefill_rows: int = PREFILL_ROWS, workgroup_slots: int = WORKGROUP_SLOTS):
+                     page_size: int = 16, prefill_rows: int = PREFILL_ROWS, workgroup_slots: int = WORKGROUP_SLOTS,
+                     tiles_only: bool = False):
     """Returns (items [n, 8], reduce_items [m, 8], partial slots, prefill items [p, 8], rows per
-    prefill item) as int32 arrays."""
+    prefill item) as int32 arrays.  `tiles_only`: no prefill items; long segments too are cut into
+    tiles of 16 rows (`build_tile_items`)."""
+    if tiles_only:
+        if group * num_kv_heads >= MAX_HEADS:
+            raise ValueError(f"{group * num_kv_heads} query heads: a work item has 16 bits for a head")
+        items, reduces, slots = build_tile_items(q_len, ctx_len, group, num_kv_heads, window)
+        return items, reduces, slots, np.zeros((0, ITEM_INTS), np.int32), prefill_rows
     q_len = np.asarray(q_len, dtype=np.int64)
     ctx_len = np.asarray(ctx_len, dtype=np.int64)
     rows = q_len * group
@@ -172,7 +230,7 @@ def build_work_items(q_len: np.ndarray, ctx_len: np.ndarray, group: int, num_kv_
         S = idx.size
         it = np.zeros((S, num_kv_heads, T, width, ITEM_INTS), dtype=np.int32)
         it[..., 0] = np.where(live, idx[:, None], -1)[:, None, None, :]
-        it[..., 1] = (kv[None, :, None] | (tile[None, None, :] * ROWS_PER_TILE << 16))[..., None]
+        it[..., 1] = (kv[None, :, None] | (tile[None, None, :] << 16))[..., None]
         it[..., 2] = q_len[idx][:, None, None, None]
         it[..., 3] = q_start[idx][:, None, None, None]
         it[..., 4] = kb[:, None, None, :]

@@ -47,6 +47,8 @@ _SIGNATURES = {
     "wllm_paged_attention_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
                                   c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
                                   c_int, c_void_p],
+    "wllm_paged_attention_mfma_f32": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
+                                      c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
     "wllm_paged_attention_prefill": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                                      c_void_p],
@@ -170,8 +172,10 @@ class HipBackend:
 
     @staticmethod
     def mfma_attention_takes(dtype, head_dim: int, page_size: int) -> bool:
-        """The matrix-core kernel: bfloat16, head sizes 32..256 in steps of 32, pages of a multiple of 4."""
-        return dtype == torch.bfloat16 and head_dim % 32 == 0 and 32 <= head_dim <= 256 and page_size % 4 == 0
+        """The matrix-core kernels: bfloat16 or float32 (each with the instruction of its own type), head sizes
+        32..256 in steps of 32, pages of a multiple of 4."""
+        return (dtype in (torch.bfloat16, torch.float32) and head_dim % 32 == 0 and 32 <= head_dim <= 256
+                and page_size % 4 == 0)
 
     def plan_paged_attention(self, host_q_len, host_ctx_len, num_heads, num_kv_heads, head_dim, page_size, window,
                              dtype, device):
@@ -179,7 +183,7 @@ class HipBackend:
             return None
         items, reduces, slots, prefill, prefill_rows = build_work_items(
             host_q_len, host_ctx_len, num_heads // num_kv_heads, num_kv_heads, window, page_size,
-            workgroup_slots=self._workgroup_slots(device))
+            workgroup_slots=self._workgroup_slots(device), tiles_only=dtype == torch.float32)
         flat = np.concatenate([items.reshape(-1), reduces.reshape(-1), prefill.reshape(-1)])
         dev = pack_int32([flat], device)[0]
         n_i, n_r, n_p = items.shape[0], reduces.shape[0], prefill.shape[0]
@@ -224,6 +228,15 @@ class HipBackend:
         if plan is not None:
             if not self.mfma_attention_takes(qkv.dtype, head_dim, page_size):
                 raise KernelError("paged_attention: a plan was given for sizes the matrix-core kernel does not take")
+            if qkv.dtype == torch.float32:
+                if plan.num_prefill:
+                    raise KernelError("paged_attention: the float32 matrix-core kernel takes tiles of 16 rows only")
+                self._check(self.lib.wllm_paged_attention_mfma_f32(
+                    _ptr(qkv), _ptr(cache), _ptr(block_tables), _ptr(plan.items), _ptr(plan.live_items), plan.num_items,
+                    _ptr(plan.reduce_items), plan.num_reduce, _ptr(seg_q_start), _ptr(seg_q_len), _ptr(out),
+                    _ptr(plan.partial_o), _ptr(plan.partial_ml), num_heads, num_kv_heads, head_dim, page_size,
+                    block_tables.shape[1], scale, window, self._stream()), "paged_attention (matrix cores, float32)")
+                return
             if plan.num_prefill:
                 self._check(self.lib.wllm_paged_attention_prefill(
                     _ptr(qkv), _ptr(cache), _ptr(block_tables), _ptr(plan.prefill_items), plan.num_prefill,
