@@ -390,17 +390,17 @@ def test_linear(dtype, m, n, k):
 
 
 def test_float32_logits_of_a_large_vocabulary_at_few_rows():
-    """7 to 16 rows, two segments of the K axis and 120,000 columns: more partial sums than the buffer
+    """7 to 64 rows, two segments of the K axis and 120,000 columns: more partial sums than the buffer
     of split sums holds at once, so the rows run in groups; every group's rows have the bits they have
-    in a product of many rows."""
+    in a product of many rows (more than 64: the tiled kernel)."""
     torch.manual_seed(15)
     n, k = 120000, 3072
-    x = torch.randn(40, k, device=DEV)
+    x = torch.randn(100, k, device=DEV)
     w = torch.randn(n, k, device=DEV) / math.sqrt(k)
-    many = torch.zeros(40, n, device=DEV)
+    many = torch.zeros(100, n, device=DEV)
     ops.linear(x, w, many)
     close(many, x.double() @ w.double().T, torch.float32, "product of many rows")
-    for rows in (6, 7, 12, 16):
+    for rows in (6, 7, 12, 16, 40):
         few = torch.full((rows, n), 9.0, device=DEV)
         ops.linear(x[3:3 + rows].contiguous(), w, few)
         assert torch.equal(few, many[3:3 + rows]), f"{rows} rows"
@@ -411,17 +411,20 @@ def test_float32_product_of_few_rows_has_the_bits_of_the_product_of_many(n, k):
     """In float32 an element is the sum over k in ascending order whatever the number of rows, so a
     token's projection in a decode step equals, bit for bit, its projection inside a long prompt."""
     torch.manual_seed(14)
-    x = torch.randn(40, k, device=DEV)
+    x = torch.randn(100, k, device=DEV)
     w = torch.randn(n, k, device=DEV) / math.sqrt(k)
-    many = torch.zeros(40, n, device=DEV)
+    many = torch.zeros(100, n, device=DEV)          # more than 64 rows: the tiled kernel
     ops.linear(x, w, many)
-    for rows in (1, 7, 16):
-        few = torch.full((rows, n), 9.0, device=DEV)
-        ops.linear(x[11:11 + rows].contiguous(), w, few)
-        assert torch.equal(few, many[11:11 + rows]), f"{rows} rows"
+    close(many, x.double() @ w.double().T, torch.float32, "product of many rows")
+    for rows in (1, 7, 16, 17, 32, 47, 64):         # the kernel that streams the weights, one to four tiles of rows
+        for tiles in (None, ops.tile_weight(w)):
+            few = torch.full((rows, n), 9.0, device=DEV)
+            ops.linear(x[11:11 + rows].contiguous(), w, few, tiles=tiles)
+            assert torch.equal(few, many[11:11 + rows]), f"{rows} rows, tile-major copy {tiles is not None}"
 
 
-@pytest.mark.parametrize("m,n,k", [(8, 2048, 16384), (5, 2560, 2048), (16, 1000, 8192), (1, 777, 516), (3, 40000, 2048)])
+@pytest.mark.parametrize("m,n,k", [(8, 2048, 16384), (5, 2560, 2048), (16, 1000, 8192), (1, 777, 516), (3, 40000, 2048),
+                                   (40, 2048, 4096), (64, 1000, 2048)])
 def test_float32_linear_leaves_partial_sums_to_the_caller(m, n, k):
     """A float32 product of few rows and not many columns gives every segment of its K axis wavefronts
     of their own; the stack of their sums, added in order, has the bits of the product made whole."""

@@ -97,20 +97,22 @@ __device__ __forceinline__ f32x4 mfma_chunk(const f32x4 a, const f32x4 b, f32x4 
     return acc;
 }
 
-// At most 16 rows (the decode steps of the float32 path): the weights stream from memory straight
+// At most 64 rows (the decode steps of the float32 path): the weights stream from memory straight
 // into the lanes that multiply them, a wavefront a band of 16 columns, `U` chunks of it in flight at a
-// time; x comes through the caches (all wavefronts read the same few rows).  SPLIT: a wavefront takes
+// time; x comes through the caches (all wavefronts read the same few rows).  MT tiles of 16 rows: a
+// fragment of the weights feeds MT products, each row's sums in the one order (the tiled kernel below
+// took 300 us for the gate and up projections of 64 rows at the 2B sizes, this one streams them).  SPLIT: a wavefront takes
 // one segment of the K axis (blockIdx.y) and leaves its sum in partial[segment]; a second kernel adds
 // the segments in ascending order.  Otherwise it walks all segments and adds as it goes.
 // TILED: w is the weight's tile-major copy (`tile_weight_f32_kernel`): per band of 16 rows and chunk
 // of 16 keys one KiB in lane order, so that a wavefront's load is one contiguous KiB and its walk along
 // K one contiguous run (gate and up at Gemma-2B sizes: 76 us from the row-major weight, whose loads
 // touch 16 rows of 64 bytes each, 49 us from the copy).
-template <bool SPLIT, bool TILED>
+template <bool SPLIT, bool TILED, int MT>
 __global__ void __launch_bounds__(256)
 gemm_f32_few_rows_kernel(const float* __restrict__ x, const float* __restrict__ w, float* __restrict__ out, int M, int N,
                          int K) {
-    constexpr int U = 8;
+    constexpr int U = MT <= 2 ? 8 : 4;
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const int i = lane % 16, g = lane / 16;
     const int n0 = (blockIdx.x * 4 + wave) * 16;
@@ -118,16 +120,25 @@ gemm_f32_few_rows_kernel(const float* __restrict__ x, const float* __restrict__ 
     const int chunks_of_row = (K + kF32Chunk - 1) / kF32Chunk;
     const float* wrow = TILED ? w + (static_cast<size_t>(n0 / 16) * chunks_of_row * 64 + lane) * 4
                               : w + static_cast<size_t>(min(n0 + i, N - 1)) * K;
-    const float* xrow = x + static_cast<size_t>(min(i, M - 1)) * K;
-    const bool x_live = i < M;
+    const float* xrow[MT];
+    bool x_live[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        xrow[t] = x + static_cast<size_t>(min(16 * t + i, M - 1)) * K;
+        x_live[t] = 16 * t + i < M;
+    }
     const int segments = (K + kF32Segment - 1) / kF32Segment;
     const int seg_first = SPLIT ? blockIdx.y : 0, seg_end = SPLIT ? blockIdx.y + 1 : segments;
-    f32x4 total = f32x4{0.f, 0.f, 0.f, 0.f};
+    f32x4 total[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) total[t] = f32x4{0.f, 0.f, 0.f, 0.f};
     for (int seg = seg_first; seg < seg_end; ++seg) {
         const int k_begin = seg * kF32Segment, k_end = min(K, k_begin + kF32Segment);
-        f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+        f32x4 acc[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
         for (int k0 = k_begin; k0 < k_end; k0 += U * kF32Chunk) {
-            f32x4 a[U], b[U];
+            f32x4 a[U], b[MT][U];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 // every lane loads, from a clamped address; what lies beyond the segment becomes zero
@@ -135,28 +146,36 @@ gemm_f32_few_rows_kernel(const float* __restrict__ x, const float* __restrict__ 
                 // (a chunk beyond the row's last is clamped to the last: what it holds becomes zero below)
                 a[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(
                     TILED ? wrow + static_cast<size_t>(min(k0 / kF32Chunk + u, chunks_of_row - 1)) * 256 : wrow + min(k, K - 4)));
-                b[u] = *reinterpret_cast<const f32x4*>(xrow + min(k, K - 4));
+#pragma unroll
+                for (int t = 0; t < MT; ++t) b[t][u] = *reinterpret_cast<const f32x4*>(xrow[t] + min(k, K - 4));
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const int k = k0 + u * kF32Chunk + 4 * g;
                 const bool live = k < k_end;
                 const f32x4 zero = f32x4{0.f, 0.f, 0.f, 0.f};
-                const f32x4 av = live ? a[u] : zero, bv = live && x_live ? b[u] : zero;
-                if (k0 + u * kF32Chunk < k_end) acc = mfma_chunk(av, bv, acc);     // the same for all lanes
+                const f32x4 av = live ? a[u] : zero;
+                if (k0 + u * kF32Chunk < k_end) {     // the same for all lanes
+#pragma unroll
+                    for (int t = 0; t < MT; ++t) acc[t] = mfma_chunk(av, live && x_live[t] ? b[t][u] : zero, acc[t]);
+                }
             }
         }
-        total = seg == seg_first ? acc : total + acc;
-    }
-    // lane (i, g) holds out[row i][n0 + 4 g .. + 3]
-    if (!x_live) return;
-    float* dst = out + (SPLIT ? static_cast<size_t>(blockIdx.y) * M * N : 0) + static_cast<size_t>(i) * N + n0 + 4 * g;
-    if (N % 4 == 0 && n0 + 4 * g + 3 < N) {
-        *reinterpret_cast<f32x4*>(dst) = total;
-    } else {
 #pragma unroll
-        for (int v = 0; v < 4; ++v)
-            if (n0 + 4 * g + v < N) dst[v] = total[v];
+        for (int t = 0; t < MT; ++t) total[t] = seg == seg_first ? acc[t] : total[t] + acc[t];
+    }
+    // lane (i, g) holds out[row 16 t + i][n0 + 4 g .. + 3]
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        if (!x_live[t]) continue;
+        float* dst = out + (SPLIT ? static_cast<size_t>(blockIdx.y) * M * N : 0) + static_cast<size_t>(16 * t + i) * N + n0 + 4 * g;
+        if (N % 4 == 0 && n0 + 4 * g + 3 < N) {
+            *reinterpret_cast<f32x4*>(dst) = total[t];
+        } else {
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (n0 + 4 * g + v < N) dst[v] = total[t][v];
+        }
     }
 }
 
@@ -325,7 +344,7 @@ WLLM_API int wllm_tile_weight_f32(const float* w, float* tiles, int N, int K, hi
 // `wllm_gemm_generic` needs `partial` to hold them; with `out` null it leaves them there for a consumer
 // that adds them in ascending order.
 WLLM_API int wllm_gemm_f32_segments(int M, int N, int K) {
-    if (M < 1 || M > 16 || K % 4 != 0 || !few_rows_split(N, K)) return 1;
+    if (M < 1 || M > 64 || K % 4 != 0 || !few_rows_split(N, K)) return 1;
     return (K + kF32Segment - 1) / kF32Segment;
 }
 
@@ -339,21 +358,35 @@ WLLM_API int wllm_gemm_generic(const void* x, const void* w, const void* tiles, 
         const float* wf = static_cast<const float*>(w);
         const float* tf = static_cast<const float*>(tiles);
         float* of = static_cast<float*>(out);
-        if (M <= 16) {
+        if (M <= 64) {
             const int bands = (N + 15) / 16, groups = (bands + 3) / 4;
+            const int mt = (M + 15) / 16;
+#define FEW_ROWS(SPLIT, GRID, DST)                                                                                      \
+    do {                                                                                                                \
+        if (tf) {                                                                                                       \
+            if (mt == 1) gemm_f32_few_rows_kernel<SPLIT, true, 1><<<GRID, 256, 0, stream>>>(xf, tf, DST, M, N, K);       \
+            else if (mt == 2) gemm_f32_few_rows_kernel<SPLIT, true, 2><<<GRID, 256, 0, stream>>>(xf, tf, DST, M, N, K);  \
+            else if (mt == 3) gemm_f32_few_rows_kernel<SPLIT, true, 3><<<GRID, 256, 0, stream>>>(xf, tf, DST, M, N, K);  \
+            else gemm_f32_few_rows_kernel<SPLIT, true, 4><<<GRID, 256, 0, stream>>>(xf, tf, DST, M, N, K);               \
+        } else {                                                                                                        \
+            if (mt == 1) gemm_f32_few_rows_kernel<SPLIT, false, 1><<<GRID, 256, 0, stream>>>(xf, wf, DST, M, N, K);      \
+            else if (mt == 2) gemm_f32_few_rows_kernel<SPLIT, false, 2><<<GRID, 256, 0, stream>>>(xf, wf, DST, M, N, K); \
+            else if (mt == 3) gemm_f32_few_rows_kernel<SPLIT, false, 3><<<GRID, 256, 0, stream>>>(xf, wf, DST, M, N, K); \
+            else gemm_f32_few_rows_kernel<SPLIT, false, 4><<<GRID, 256, 0, stream>>>(xf, wf, DST, M, N, K);              \
+        }                                                                                                               \
+    } while (0)
             if (few_rows_split(N, K)) {
                 const int segments = (K + kF32Segment - 1) / kF32Segment;
                 if (!partial || segments > 65535) return -1;
                 float* pf = static_cast<float*>(partial);
-                if (tf) gemm_f32_few_rows_kernel<true, true><<<dim3(groups, segments), 256, 0, stream>>>(xf, tf, pf, M, N, K);
-                else gemm_f32_few_rows_kernel<true, false><<<dim3(groups, segments), 256, 0, stream>>>(xf, wf, pf, M, N, K);
+                FEW_ROWS(true, dim3(groups, segments), pf);
                 if (int err = launch_status()) return err;
                 if (of) gemm_segments_sum_kernel<<<(M * N + 255) / 256, 256, 0, stream>>>(pf, of, M * N, segments);
             } else {
                 if (!of) return -1;
-                if (tf) gemm_f32_few_rows_kernel<false, true><<<groups, 256, 0, stream>>>(xf, tf, of, M, N, K);
-                else gemm_f32_few_rows_kernel<false, false><<<groups, 256, 0, stream>>>(xf, wf, of, M, N, K);
+                FEW_ROWS(false, dim3(groups), of);
             }
+#undef FEW_ROWS
             return launch_status();
         }
         if (!of) return -1;

@@ -316,6 +316,7 @@ class HipBackend:
     # twice as fast alone (K axis of 2,048 in four pieces at 128 to 512 rows), but the rotation and the
     # norm that then add the pieces lose more than that: left to the library.
     TILE_MAX_ROWS = 1024
+    F32_FEW_ROWS = 64         # rows up to which the float32 product streams its weights a band a wavefront
     TILE_LONG_K = 8192
     TILE_GATED_MAX_ROWS = 256
 
@@ -347,7 +348,7 @@ class HipBackend:
             return self.skinny_split(out_features, in_features)
         if self.tile_takes(dtype, rows, out_features, in_features):
             return self.tile_splits(out_features, in_features, rows)
-        if dtype == torch.float32 and rows <= 16:
+        if dtype == torch.float32 and rows <= self.F32_FEW_ROWS:
             return self.lib.wllm_gemm_f32_segments(rows, out_features, in_features)
         return 1
 
@@ -414,7 +415,7 @@ class HipBackend:
                 torch.mm(x, weight.t(), out=out)
                 return
         # float32, few rows, a long K axis: the segments of K are summed by wavefronts of their own
-        if x.dtype == torch.float32 and m <= 16:
+        if x.dtype == torch.float32 and m <= self.F32_FEW_ROWS:
             n = weight.shape[0]
             segments = self.lib.wllm_gemm_f32_segments(m, n, k)
             if out.dim() == 3:      # the caller adds the segments' sums later
