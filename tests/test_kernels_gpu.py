@@ -4,6 +4,7 @@ counts and groups (up to 40 query heads a key/value head), partial rotation, win
 1 to 40 tokens."""
 import math
 
+import numpy as np
 import pytest
 import torch
 
@@ -687,3 +688,13 @@ def test_a_key_has_one_rounding_more_in_a_step_of_many_rows():
     grid = a.abs().amax(-1, keepdim=True) * 2.0 ** -7
     assert ((a - b).abs() <= grid).all(), "more than one rounding apart"
     assert (a == b).float().mean() > 0.5
+
+
+def test_float32_prompts_too_long_for_tiles_take_the_general_kernel():
+    """A float32 step whose tiles of 16 rows would leave more than a GiB of partial results gets no plan (the engine
+    then runs the kernel on the vector units); one that fits gets one without blocks of 64 rows."""
+    be = ops.backend()
+    n = 8192
+    assert be.plan_paged_attention(np.array([n]), np.array([n]), 8, 1, 256, 16, 0, torch.float32, DEV) is None
+    plan = be.plan_paged_attention(np.array([4096]), np.array([4096]), 8, 1, 256, 16, 0, torch.float32, DEV)
+    assert plan is not None and plan.num_prefill == 0 and plan.num_partial_slots * 16 * 256 <= be.TILE_PARTIAL_FLOATS

@@ -9,7 +9,7 @@ from ctypes import c_float, c_int, c_longlong, c_void_p
 import numpy as np
 import torch
 
-from wllm_amd.kernels.attention_plan import AttentionPlan, build_work_items
+from wllm_amd.kernels.attention_plan import MAX_TILES, AttentionPlan, build_work_items, row_tiles
 from wllm_amd.kernels import ops
 from wllm_amd.kernels.ops import ACTIVATIONS
 from wllm_amd.kernels.library import load
@@ -181,9 +181,14 @@ class HipBackend:
                              dtype, device):
         if not self.mfma_attention_takes(dtype, head_dim, page_size):
             return None
+        tiles_only = dtype == torch.float32
+        if tiles_only and len(host_q_len) and row_tiles(int(np.max(host_q_len)), num_heads // num_kv_heads) >= MAX_TILES:
+            return None         # more tiles of 16 rows than a work item can number: the general kernel takes the step
         items, reduces, slots, prefill, prefill_rows = build_work_items(
             host_q_len, host_ctx_len, num_heads // num_kv_heads, num_kv_heads, window, page_size,
-            workgroup_slots=self._workgroup_slots(device), tiles_only=dtype == torch.float32)
+            workgroup_slots=self._workgroup_slots(device), tiles_only=tiles_only)
+        if tiles_only and slots * 16 * head_dim > self.TILE_PARTIAL_FLOATS:
+            return None         # (a float32 prompt of many thousand tokens in one step: the general kernel)
         flat = np.concatenate([items.reshape(-1), reduces.reshape(-1), prefill.reshape(-1)])
         dev = pack_int32([flat], device)[0]
         n_i, n_r, n_p = items.shape[0], reduces.shape[0], prefill.shape[0]
@@ -220,6 +225,7 @@ class HipBackend:
             self._partial_ml = torch.empty(need, dtype=torch.float32, device=device)
 
     GENERIC_PARTIAL_FLOATS = 1 << 25       # 128 MiB of partial results for the general attention kernel
+    TILE_PARTIAL_FLOATS = 1 << 28          # 1 GiB: the most partial results a float32 step cut into tiles of 16 rows may leave
 
     def paged_attention(self, qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len, out,
                         num_heads, num_kv_heads, head_dim, page_size, scale, window, max_q_len, max_ctx_len,
