@@ -299,6 +299,183 @@ attention_reduce_f32_kernel(const int* __restrict__ reduce_items, const float* _
         float4_t{num[0] / den, num[1] / den, num[2] / den, num[3] / den};
 }
 
+// Prompt portions: a workgroup takes 64 rows (a wavefront a tile of 16) and walks their keys in blocks of 32,
+// which it stages once for all four wavefronts: the keys as rows of HD + 4 floats, the values transposed as rows of
+// 32 + 4 (16 lanes' 16-byte fragment reads fall into different banks).  The products are those of the kernel above
+// (lane group g takes the quarter g of the head in the scores, the keys 4g..4g+3 of a tile of 16 in the second
+// product); the maximum and the sums are carried from block to block.  (The next block's pieces asked for into
+// registers while this one is multiplied: 256 registers and spills, 216 to 231 us for 2,048 tokens where this form
+// takes 205 to 217.)  Work items are the bfloat16 prompt kernel's
+// (`attention_prefill.hip`): segment, key/value head, first row, first key, end key, partial slot (-1: final).
+constexpr int kBlockKeys = 32;
+
+template <int HD>
+__global__ void __launch_bounds__(256, 2)
+paged_attention_prefill_f32_kernel(const float* __restrict__ qkv, const float* __restrict__ cache,
+                                   const int* __restrict__ block_tables, const int* __restrict__ items,
+                                   const int* __restrict__ seg_q_start, const int* __restrict__ seg_q_len,
+                                   const int* __restrict__ seg_ctx_len, float* __restrict__ out,
+                                   float* __restrict__ partial_o, float* __restrict__ partial_ml, int num_heads,
+                                   int num_kv_heads, int page_size, int max_pages, float scale_log2e, int window) {
+    constexpr int DQ = HD / 4, DT = HD / 16;
+    constexpr int SK = HD + 4, SV = kBlockKeys + 4;
+    __shared__ __align__(16) float k_s[kBlockKeys * SK];
+    __shared__ __align__(16) float v_s[HD * SV];
+
+    const int* item = items + static_cast<size_t>(blockIdx.x) * kItemInts;
+    const int seg = item[0], kvh = item[1], row_begin = item[2];
+    const int key_begin = item[3], key_end = item[4], partial_slot = item[5];
+    if (seg < 0) return;
+    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const int i = lane % 16, g = lane / 16;
+    const int group = num_heads / num_kv_heads;
+    const int q_start = seg_q_start[seg], q_len = seg_q_len[seg], ctx = seg_ctx_len[seg];
+    const int total_rows = q_len * group;
+    const int first_pos = ctx - q_len;
+    const int seg_lo = window > 0 ? max(0, first_pos - window + 1) : 0;
+    const int width = (num_heads + 2 * num_kv_heads) * HD;
+    const size_t page_elems = static_cast<size_t>(2) * num_kv_heads * page_size * HD;
+    const size_t k_off = static_cast<size_t>(kvh) * page_size * HD;
+    const size_t v_off = (static_cast<size_t>(num_kv_heads) + kvh) * page_size * HD;
+    const int* table = block_tables + static_cast<size_t>(seg) * max_pages;
+
+    const int wr0 = row_begin + wave * 16;
+    const int row = wr0 + i;
+    const bool row_valid = row < total_rows;
+    const int tok = row_valid ? row / group : 0;
+    const int head = kvh * group + (row_valid ? row % group : 0);
+    const int pos = first_pos + tok;
+    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    // a block that lies wholly inside every row's range needs no mask (a wavefront-wide decision)
+    const int w_last_row = min(total_rows - 1, wr0 + 15);
+    const bool wave_active = wr0 < total_rows;
+    const int t_pos_min = (wave_active && w_last_row == wr0 + 15) ? first_pos + wr0 / group : -1;
+    const int t_lo_max = window > 0 ? max(0, first_pos + max(w_last_row, 0) / group - window + 1) : 0;
+    const int w_hi = wave_active ? first_pos + w_last_row / group + 1 : 0;                       // exclusive
+    const int w_lo = window > 0 ? max(0, first_pos + wr0 / group - window + 1) : 0;
+    const int b_last_row = min(total_rows - 1, row_begin + 63);
+    const int b_hi = first_pos + b_last_row / group + 1;
+    const int b_lo = window > 0 ? max(0, first_pos + row_begin / group - window + 1) : 0;
+    const int blk_first = max(b_lo, key_begin) / kBlockKeys;
+    const int blk_end = (min(b_hi, key_end) + kBlockKeys - 1) / kBlockKeys;
+
+    // the lane's quarter of its row of queries
+    float4_t qv[DQ / 4];
+    {
+        const float* qrow = qkv + static_cast<size_t>(q_start + tok) * width + static_cast<size_t>(head) * HD + g * DQ;
+#pragma unroll
+        for (int j = 0; j < DQ / 4; ++j)
+            qv[j] = row_valid ? *reinterpret_cast<const float4_t*>(qrow + 4 * j) : float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    float4_t acc[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t) acc[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+
+    for (int blk = blk_first; blk < blk_end; ++blk) {
+        const int kbase = blk * kBlockKeys;
+        __syncthreads();        // everyone is done with the block before
+        // ---- the block's keys, rows of the cache as they lie; a key beyond the table's width (it is masked) reads
+        //      the last page the table names ----
+#pragma unroll
+        for (int u = 0; u < kBlockKeys * (HD / 4) / 256; ++u) {
+            const int p = tid + 256 * u;
+            const int key = p / (HD / 4), c4 = p % (HD / 4);
+            const int kk = kbase + key;
+            const int page_index = kk / page_size, slot = kk - page_index * page_size;
+            const float* src = cache + static_cast<size_t>(table[min(page_index, max_pages - 1)]) * page_elems + k_off +
+                               static_cast<size_t>(slot) * HD + 4 * c4;
+            *reinterpret_cast<float4_t*>(k_s + key * SK + 4 * c4) = *reinterpret_cast<const float4_t*>(src);
+        }
+        // ---- its values, four keys of a transposed row a piece (one page: pages are multiples of 4 keys); what is
+        //      not the request's (stale slots, pages given back) may hold anything and is cleared ----
+        const bool edge = kbase < seg_lo || kbase + kBlockKeys > ctx;
+#pragma unroll
+        for (int u = 0; u < HD * (kBlockKeys / 4) / 256; ++u) {
+            const int p = tid + 256 * u;
+            const int d = p / (kBlockKeys / 4), q4 = p % (kBlockKeys / 4);
+            const int kk = kbase + 4 * q4;
+            const int page_index = kk / page_size, slot = kk - page_index * page_size;
+            const float* src = cache + static_cast<size_t>(table[min(page_index, max_pages - 1)]) * page_elems + v_off +
+                               static_cast<size_t>(d) * page_size + slot;
+            float4_t v = *reinterpret_cast<const float4_t*>(src);
+            if (edge) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (kk + e >= ctx || kk + e < seg_lo) v[e] = 0.f;
+            }
+            *reinterpret_cast<float4_t*>(v_s + d * SV + 4 * q4) = v;
+        }
+        __syncthreads();
+        if (!wave_active || kbase >= w_hi || kbase + kBlockKeys <= w_lo) continue;
+        // ---- scores: two tiles of 16 keys; the lane's keys are 16 t2 + 4 g + v ----
+        float sv[8];
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2) {
+            float4_t sc = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < DQ / 4; ++j) {
+                const float4_t kf = *reinterpret_cast<const float4_t*>(k_s + (16 * t2 + i) * SK + g * DQ + 4 * j);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sc = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[e], qv[j][e], sc, 0, 0, 0);
+            }
+#pragma unroll
+            for (int v = 0; v < 4; ++v) sv[4 * t2 + v] = sc[v];
+        }
+        const bool inside = kbase + kBlockKeys - 1 <= t_pos_min && kbase >= t_lo_max;
+        if (!inside) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int key = kbase + 16 * (e / 4) + 4 * g + e % 4;
+                if (!(row_valid && key <= pos && key >= lo)) sv[e] = -INFINITY;
+            }
+        }
+        float tile_max = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+        tile_max = max_across(max_across(tile_max, 16), 32);
+        const float m_new = fmaxf(m_run, tile_max);
+        const float mc = (m_new == -INFINITY ? 0.f : m_new) * scale_log2e;
+        const float alpha = exp2f(fmaf(m_run, scale_log2e, -mc));        // exp2(-inf) = 0: nothing was summed yet
+        float pe[8], psum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            pe[e] = exp2f(fmaf(sv[e], scale_log2e, -mc));                   // 0 for masked keys
+            psum += pe[e];
+        }
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        if (__builtin_amdgcn_readfirstlane(__any(alpha != 1.f))) {
+#pragma unroll
+            for (int t = 0; t < DT; ++t) acc[t] *= alpha;
+        }
+        // ---- out^T += V^T . P^T ----
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2) {
+                const float4_t vf = *reinterpret_cast<const float4_t*>(v_s + (16 * t + i) * SV + 16 * t2 + 4 * g);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(vf[v], pe[4 * t2 + v], acc[t], 0, 0, 0);
+            }
+        }
+    }
+    float l = sum_across(sum_across(l_run, 16), 32);
+    if (!row_valid) return;
+    if (partial_slot >= 0) {
+        // one slot per tile of 16 rows: [16][HD] accumulators and [16][2] (maximum, sum)
+        const size_t slot = static_cast<size_t>(partial_slot) + wave;
+        float* po = partial_o + (slot * 16 + i) * HD;
+#pragma unroll
+        for (int t = 0; t < DT; ++t) *reinterpret_cast<float4_t*>(po + t * 16 + 4 * g) = acc[t];
+        if (g == 0) *reinterpret_cast<float2*>(partial_ml + (slot * 16 + i) * 2) = make_float2(m_run, l);
+        return;
+    }
+    const float inv = 1.f / l;
+    float* orow = out + (static_cast<size_t>(q_start + tok) * num_heads + head) * HD;
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+        *reinterpret_cast<float4_t*>(orow + t * 16 + 4 * g) = float4_t{acc[t][0] * inv, acc[t][1] * inv, acc[t][2] * inv, acc[t][3] * inv};
+}
+
 template <int HD>
 int launch_f32(const float* qkv, const float* cache, const int* block_tables, const int* items, const int* live_items,
                int num_items, const int* reduce_items, int num_reduce_items, const int* seg_q_start, const int* seg_q_len,
@@ -345,3 +522,38 @@ WLLM_API int wllm_paged_attention_mfma_f32(const float* qkv, const float* cache,
     }
 #undef LAUNCH
 }
+
+// The prompt portions of a float32 step: `items` are prefill items of 64 rows (`rows_per_item` says what the plan was
+// made for).  Blocks whose keys were cut into pieces leave partial results for the reduce kernel, which
+// `wllm_paged_attention_mfma_f32` runs with the step's reduce items.  Returns 0, a HIP error code, or -1.
+WLLM_API int wllm_paged_attention_prefill_f32(const float* qkv, const float* cache, const int* block_tables, const int* items,
+                                              int num_items, int rows_per_item, const int* seg_q_start, const int* seg_q_len,
+                                              const int* seg_ctx_len, float* out, float* partial_o, float* partial_ml,
+                                              int num_heads, int num_kv_heads, int head_dim, int page_size, int max_pages,
+                                              float scale, int window, hipStream_t stream) {
+    if (head_dim % 32 != 0 || head_dim < 32 || head_dim > 256 || page_size % 4 != 0 || num_heads % num_kv_heads != 0 ||
+        rows_per_item != 64)
+        return -1;
+    if (num_items <= 0) return 0;
+    const float scale_log2e = scale * 1.4426950408889634f;
+#define LAUNCH(HD)                                                                                                    \
+    paged_attention_prefill_f32_kernel<HD><<<num_items, 256, 0, stream>>>(qkv, cache, block_tables, items, seg_q_start, \
+                                                                          seg_q_len, seg_ctx_len, out, partial_o,        \
+                                                                          partial_ml, num_heads, num_kv_heads, page_size, \
+                                                                          max_pages, scale_log2e, window);               \
+    break
+    switch (head_dim) {
+        case 32: LAUNCH(32);
+        case 64: LAUNCH(64);
+        case 96: LAUNCH(96);
+        case 128: LAUNCH(128);
+        case 160: LAUNCH(160);
+        case 192: LAUNCH(192);
+        case 224: LAUNCH(224);
+        case 256: LAUNCH(256);
+        default: return -1;
+    }
+#undef LAUNCH
+    return launch_status();
+}
+

@@ -9,7 +9,7 @@ from ctypes import c_float, c_int, c_longlong, c_void_p
 import numpy as np
 import torch
 
-from wllm_amd.kernels.attention_plan import MAX_TILES, AttentionPlan, build_work_items, row_tiles
+from wllm_amd.kernels.attention_plan import AttentionPlan, build_work_items
 from wllm_amd.kernels import ops
 from wllm_amd.kernels.ops import ACTIVATIONS
 from wllm_amd.kernels.library import load
@@ -49,6 +49,9 @@ _SIGNATURES = {
                                   c_int, c_void_p],
     "wllm_paged_attention_mfma_f32": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p,
                                       c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+    "wllm_paged_attention_prefill_f32": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                                         c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
+                                         c_void_p],
     "wllm_paged_attention_prefill": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                                      c_void_p],
@@ -181,14 +184,16 @@ class HipBackend:
                              dtype, device):
         if not self.mfma_attention_takes(dtype, head_dim, page_size):
             return None
-        tiles_only = dtype == torch.float32
-        if tiles_only and len(host_q_len) and row_tiles(int(np.max(host_q_len)), num_heads // num_kv_heads) >= MAX_TILES:
-            return None         # more tiles of 16 rows than a work item can number: the general kernel takes the step
+        group, slots_of_device = num_heads // num_kv_heads, self._workgroup_slots(device)
         items, reduces, slots, prefill, prefill_rows = build_work_items(
-            host_q_len, host_ctx_len, num_heads // num_kv_heads, num_kv_heads, window, page_size,
-            workgroup_slots=self._workgroup_slots(device), tiles_only=tiles_only)
-        if tiles_only and slots * 16 * head_dim > self.TILE_PARTIAL_FLOATS:
-            return None         # (a float32 prompt of many thousand tokens in one step: the general kernel)
+            host_q_len, host_ctx_len, group, num_kv_heads, window, page_size, workgroup_slots=slots_of_device)
+        if dtype == torch.float32 and 0 < prefill.shape[0] < slots_of_device // 2:
+            # float32 and few blocks of 64 rows (a prompt of some hundred tokens): tiles of 16 rows fill the device
+            # better than the blocks would (512 tokens of 8 heads: 43 against 96 us).  With so few blocks the tiles
+            # are few too (at most four a block) and so are their chunks (the blocks' keys were not worth cutting).
+            items, reduces, slots, prefill, prefill_rows = build_work_items(
+                host_q_len, host_ctx_len, group, num_kv_heads, window, page_size, workgroup_slots=slots_of_device,
+                tiles_only=True)
         flat = np.concatenate([items.reshape(-1), reduces.reshape(-1), prefill.reshape(-1)])
         dev = pack_int32([flat], device)[0]
         n_i, n_r, n_p = items.shape[0], reduces.shape[0], prefill.shape[0]
@@ -225,7 +230,6 @@ class HipBackend:
             self._partial_ml = torch.empty(need, dtype=torch.float32, device=device)
 
     GENERIC_PARTIAL_FLOATS = 1 << 25       # 128 MiB of partial results for the general attention kernel
-    TILE_PARTIAL_FLOATS = 1 << 28          # 1 GiB: the most partial results a float32 step cut into tiles of 16 rows may leave
 
     def paged_attention(self, qkv, cache, block_tables, token_segment, seg_q_start, seg_q_len, seg_ctx_len, out,
                         num_heads, num_kv_heads, head_dim, page_size, scale, window, max_q_len, max_ctx_len,
@@ -236,7 +240,14 @@ class HipBackend:
                 raise KernelError("paged_attention: a plan was given for sizes the matrix-core kernel does not take")
             if qkv.dtype == torch.float32:
                 if plan.num_prefill:
-                    raise KernelError("paged_attention: the float32 matrix-core kernel takes tiles of 16 rows only")
+                    self._check(self.lib.wllm_paged_attention_prefill_f32(
+                        _ptr(qkv), _ptr(cache), _ptr(block_tables), _ptr(plan.prefill_items), plan.num_prefill,
+                        plan.prefill_rows, _ptr(seg_q_start), _ptr(seg_q_len), _ptr(seg_ctx_len), _ptr(out),
+                        _ptr(plan.partial_o), _ptr(plan.partial_ml), num_heads, num_kv_heads, head_dim, page_size,
+                        block_tables.shape[1], scale, window, self._stream()),
+                        "paged_attention (prompt portions, matrix cores, float32)")
+                if plan.num_items == 0 and plan.num_reduce == 0:
+                    return
                 self._check(self.lib.wllm_paged_attention_mfma_f32(
                     _ptr(qkv), _ptr(cache), _ptr(block_tables), _ptr(plan.items), _ptr(plan.live_items), plan.num_items,
                     _ptr(plan.reduce_items), plan.num_reduce, _ptr(seg_q_start), _ptr(seg_q_len), _ptr(out),
